@@ -1,0 +1,121 @@
+"""ctypes binding of libeidola_attn_hip.so (the C ABI declared in include/eidola_attn.h).
+
+The reference (eidola-ai/eidola) has no operator or FFI interface for this path — its only
+engine seam is OpenAI-compatible HTTP (crates/eidola-server/src/backend.rs:87-108) — so the
+structures below mirror this repository's own header field for field.
+"""
+import ctypes as C
+import os
+
+KV_BF16 = 0
+KV_FP8_E4M3 = 1
+
+EID_OK = 0
+EID_ERR_INVALID_ARG = -1
+EID_ERR_UNSUPPORTED = -2
+EID_ERR_WORKSPACE = -3
+EID_ERR_HIP = -4
+
+_STATUS_NAMES = {
+    EID_ERR_INVALID_ARG: "EID_ERR_INVALID_ARG",
+    EID_ERR_UNSUPPORTED: "EID_ERR_UNSUPPORTED",
+    EID_ERR_WORKSPACE: "EID_ERR_WORKSPACE",
+    EID_ERR_HIP: "EID_ERR_HIP",
+}
+
+
+class EidError(RuntimeError):
+    """A non-zero eid_status, carrying the code and the library's thread-local message."""
+
+    def __init__(self, status, message):
+        self.status = status
+        self.name = _STATUS_NAMES.get(status, str(status))
+        super().__init__(f"{self.name}: {message}")
+
+
+class AttnDesc(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("num_seqs", C.c_int32),
+        ("num_q_tokens", C.c_int32),
+        ("max_q_len", C.c_int32),
+        ("max_kv_len", C.c_int32),
+        ("num_q_heads", C.c_int32),
+        ("num_kv_heads", C.c_int32),
+        ("head_dim", C.c_int32),
+        ("block_size", C.c_int32),
+        ("max_blocks_per_seq", C.c_int32),
+        ("num_blocks", C.c_int64),
+        ("softmax_scale", C.c_float),
+        ("window", C.c_int32),
+        ("kv_dtype", C.c_int32),
+        ("partition_size", C.c_int32),
+    ]
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p),
+        ("out", C.c_void_p),
+        ("lse", C.c_void_p),
+        ("k_cache", C.c_void_p),
+        ("v_cache", C.c_void_p),
+        ("block_table", C.c_void_p),
+        ("cu_seqlens_q", C.c_void_p),
+        ("seq_lens", C.c_void_p),
+        ("sinks", C.c_void_p),
+        ("k_scale", C.c_void_p),
+        ("v_scale", C.c_void_p),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
+    ]
+
+
+EXPORTS = ("eid_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
+           "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
+
+_lib = None
+
+
+def lib_path():
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
+                        "libeidola_attn_hip.so")
+
+
+def load_library():
+    """Load the HIP library; raises (never falls back) when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise EidError(EID_ERR_HIP, f"{path} is missing: run `python -c 'import "
+                       "__graft_entry__ as g; g.build()'` or `make -C eidola_amd/csrc`")
+    lib = C.CDLL(path)
+    P = C.c_void_p
+    lib.eid_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, P, P, C.c_int32, P, P, P]
+    lib.eid_kv_write.restype = C.c_int32
+    for name in ("eid_attn_decode", "eid_attn_varlen", "eid_lse_merge"):
+        fn = getattr(lib, name)
+        fn.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs), P]
+        fn.restype = C.c_int32
+    lib.eid_workspace_bytes.argtypes = [C.POINTER(AttnDesc)]
+    lib.eid_workspace_bytes.restype = C.c_size_t
+    lib.eid_partition_size.argtypes = [C.POINTER(AttnDesc)]
+    lib.eid_partition_size.restype = C.c_int32
+    lib.eid_last_error.argtypes = []
+    lib.eid_last_error.restype = C.c_char_p
+    lib.eid_version.argtypes = []
+    lib.eid_version.restype = C.c_uint32
+    _lib = lib
+    return lib
+
+
+def check(status):
+    if status != EID_OK:
+        raise EidError(status, load_library().eid_last_error().decode())
+
+
+def version():
+    v = load_library().eid_version()
+    return v >> 16, v & 0xFFFF

@@ -1,0 +1,515 @@
+// Paged sink-attention kernels for gfx950 (MI355X): one wavefront-level engine shared by
+//   * the bandwidth-bound split-KV kernel (decode and short-q verify rows), and
+//   * the tile kernel for long query chunks (chunked prefill),
+// plus the cross-partition log-sum-exp merge.
+//
+// Engine, per wavefront, per chunk of 64 context tokens (four 16-token pages):
+//   S^T[token][row] = K[token][:] . Q[row][:]   v_mfma_f32_16x16x32_bf16, tokens on M so a
+//        lane's 16-byte global load of a K row IS its A operand (no LDS hop for K);
+//   online softmax in base 2 on the accumulator layout (a lane owns 4 tokens of one row,
+//        the row maximum crosses the four 16-lane rows with v_permlane{16,32}_swap);
+//   P^T leaves the softmax already in B-operand layout (tokens on the contraction axis);
+//   O^T[dim][row] += V^T[dim][token] . P^T[token][row], with V staged row-major in LDS and
+//        read back transposed by ds_read_b64_tr_b16.
+// "row" = (query token, query head of the KV group): 8 heads share every K/V byte.
+#include "eid_device.h"
+#include "eid_params.h"
+
+namespace eid {
+
+constexpr int kVRowBytes = 144;                 // 128 B of bf16 + 16 B pad (bank spread)
+constexpr int kVPageBytes = kBlock * kVRowBytes;  // one 16-token page of V for one KV head
+constexpr int kWaveLdsBytes = 4 * kVPageBytes;  // 64 tokens
+
+__device__ __forceinline__ u32x4 ldg128(const uint8_t *p) { return *(const u32x4 *)p; }
+
+// Row bookkeeping of one 16-row MFMA column tile.
+struct RowInfo {
+  int pos;  // absolute position of the row's query token
+  int lo;   // first key the row may see
+};
+
+// One wavefront attends rows [16*NT) over keys [t_begin, t_end) of sequence `s`.
+// t_begin is a multiple of 16.  Tokens >= seq_len are never used (K masked, V zeroed).
+template <int NT, bool FP8>
+__device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
+                                       const int t_begin, const int t_end, const int seq_len,
+                                       const int pos_first, const int lo_last,
+                                       const Frag8 (&qf)[NT][2], const RowInfo (&ri)[NT],
+                                       uint8_t *wave_lds, float (&m)[NT], float (&lsum)[NT],
+                                       f32x4 (&acc)[NT][4]) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, g = lane >> 4;
+  const int Hkv = p.num_kv_heads;
+  constexpr int kElt = FP8 ? 1 : 2;
+  const uint32_t row_bytes = (uint32_t)Hkv * kHeadDim * kElt;
+  const size_t page_bytes = (size_t)kBlock * row_bytes;
+  const uint32_t lane_off = (uint32_t)i16 * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
+                            (uint32_t)g * (16 * kElt);
+  const int32_t *bt = p.block_table + (size_t)s * p.max_blocks_per_seq;
+  const int nblk_total = (t_end + kBlock - 1) / kBlock;
+  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
+
+  uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
+  const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
+
+  int ids = 0;
+  int ci = 0;
+  for (int tc = t_begin; tc < t_end; tc += kChunk, ++ci) {
+    if ((ci & 15) == 0) {  // page ids of the next 1024 tokens, one per lane
+      const int bi = tc / kBlock + lane;
+      ids = bi < nblk_total ? bt[bi] : 0;
+    }
+    const int nb = min(4, (t_end - tc + kBlock - 1) / kBlock);
+
+    // ---- global loads: each lane takes 32 B (bf16) / 16 B (fp8) of one token row ----
+    u32x4 kraw[4][kElt], vraw[4][kElt];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+#pragma unroll
+      for (int e = 0; e < kElt; ++e) {
+        kraw[b][e] = u32x4{0, 0, 0, 0};
+        vraw[b][e] = u32x4{0, 0, 0, 0};
+      }
+      if (b < nb) {
+        const int blk = __builtin_amdgcn_readlane(ids, (ci & 15) * 4 + b);
+        const uint8_t *kp = p.k_cache + (size_t)blk * page_bytes + lane_off;
+        const uint8_t *vp = p.v_cache + (size_t)blk * page_bytes + lane_off;
+#pragma unroll
+        for (int e = 0; e < kElt; ++e) {
+          kraw[b][e] = ldg128(kp + 16 * e);
+          vraw[b][e] = ldg128(vp + 16 * e);
+        }
+      }
+    }
+
+    // ---- V: zero rows past the sequence end, widen fp8, stage in LDS ----
+    const bool tail = tc + kChunk > seq_len;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      u32x4 v0, v1;
+      if constexpr (FP8) {
+        uint32_t lo4[4], hi4[4];
+        fp8x8_to_bf16x8(vraw[b][0][0], vraw[b][0][1], lo4);
+        fp8x8_to_bf16x8(vraw[b][0][2], vraw[b][0][3], hi4);
+        v0 = u32x4{lo4[0], lo4[1], lo4[2], lo4[3]};
+        v1 = u32x4{hi4[0], hi4[1], hi4[2], hi4[3]};
+      } else {
+        v0 = vraw[b][0];
+        v1 = vraw[b][kElt - 1];
+      }
+      if (tail && tc + b * kBlock + i16 >= seq_len) {
+        v0 = u32x4{0, 0, 0, 0};
+        v1 = u32x4{0, 0, 0, 0};
+      }
+      *(u32x4 *)(lds_wr + b * kVPageBytes) = v0;
+      *(u32x4 *)(lds_wr + b * kVPageBytes + 16) = v1;
+    }
+
+    // ---- K operands ----
+    Frag8 kf[4][2];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      if constexpr (FP8) {
+        fp8x8_to_bf16x8(kraw[b][0][0], kraw[b][0][1], kf[b][0].w);
+        fp8x8_to_bf16x8(kraw[b][0][2], kraw[b][0][3], kf[b][1].w);
+      } else {
+        kf[b][0].u = kraw[b][0];
+        kf[b][1].u = kraw[b][kElt - 1];
+      }
+    }
+
+    const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
+
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      // S^T = K Q^T, then scale into the base-2 domain
+      f32x4 S[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        z = mfma16x32(kf[b][0], qf[nt][0], z);
+        S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) S[b][r] *= c2;
+      }
+      if (need_mask) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = tc + b * kBlock + 4 * g + r;
+            if (j < ri[nt].lo || j > ri[nt].pos) S[b][r] = -INFINITY;
+          }
+      }
+      float mloc = S[0][0];
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, S[b][r]);
+      mloc = rowgroup_max(mloc);
+      const float m_new = fmaxf(m[nt], mloc);
+      const float alpha = fast_exp2(m[nt] - m_new);
+      m[nt] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          S[b][r] = fast_exp2(S[b][r] - m_new);
+          psum += S[b][r];
+        }
+      lsum[nt] = lsum[nt] * alpha + psum;
+      if (__any(alpha != 1.0f)) {
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+      }
+      // P^T as B operands: pair 0 = pages 0,1; pair 1 = pages 2,3
+      Frag8 pf[2];
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        pf[pr].w[0] = pack_bf16(S[2 * pr][0], S[2 * pr][1]);
+        pf[pr].w[1] = pack_bf16(S[2 * pr][2], S[2 * pr][3]);
+        pf[pr].w[2] = pack_bf16(S[2 * pr + 1][0], S[2 * pr + 1][1]);
+        pf[pr].w[3] = pack_bf16(S[2 * pr + 1][2], S[2 * pr + 1][3]);
+      }
+      // O^T += V^T P^T
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int pr = 0; pr < 2; ++pr) {
+          const u32x2 a = lds_read_tr16(lds_rd + (2 * pr) * kVPageBytes + 32 * mt);
+          const u32x2 b2 = lds_read_tr16(lds_rd + (2 * pr + 1) * kVPageBytes + 32 * mt);
+          Frag8 vf;
+          vf.w[0] = a[0];
+          vf.w[1] = a[1];
+          vf.w[2] = b2[0];
+          vf.w[3] = b2[1];
+          acc[nt][mt] = mfma16x32(vf, pf[pr], acc[nt][mt]);
+        }
+    }
+  }
+}
+
+// Finish a row tile: either normalise with the sink and store bf16 output (+lse), or store
+// the partition's partial (m, l, acc) for the merge kernel.
+template <int NT, bool FP8>
+__device__ __forceinline__ void finish(const AttnParams &p, const int s, const int kvh,
+                                       const int row0, const int qlen, const int tq0,
+                                       const bool direct, const int part, float (&m)[NT],
+                                       float (&lsum)[NT], f32x4 (&acc)[NT][4]) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, g = lane >> 4;
+  const int Hq = p.num_q_heads;
+  const float vs = FP8 ? p.v_scale[kvh] : 1.0f;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const float l = rowgroup_sum(lsum[nt]);
+    const int r = nt * 16 + i16;
+    const int t = tq0 + (r >> 3);
+    const int head = kvh * kGroup + (r & 7);
+    if (t >= qlen) continue;
+    if (direct) {
+      const float sink2 = p.sinks ? p.sinks[head] * kLog2e : -INFINITY;
+      const float M = fmaxf(m[nt], sink2);
+      const float w = fast_exp2(m[nt] - M);
+      const float den = l * w + fast_exp2(sink2 - M);
+      const float inv = w * vs / den;
+      uint16_t *o = p.out + ((size_t)(row0 + t) * Hq + head) * kHeadDim + 4 * g;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        u32x2 pk;
+        pk[0] = pack_bf16(acc[nt][mt][0] * inv, acc[nt][mt][1] * inv);
+        pk[1] = pack_bf16(acc[nt][mt][2] * inv, acc[nt][mt][3] * inv);
+        *(u32x2 *)(o + 16 * mt) = pk;
+      }
+      if (p.lse && g == 0) p.lse[(size_t)(row0 + t) * Hq + head] = (M + __log2f(den)) * kLn2;
+    } else {
+      const size_t idx = ((size_t)(s * p.ws_rows + t) * Hq + head) * p.nparts_max + part;
+      if (g == 0) {
+        float2 ml;
+        ml.x = l > 0.f ? m[nt] * kLn2 : -INFINITY;
+        ml.y = l;
+        *(float2 *)(p.ws_ml + idx * 2) = ml;
+      }
+      float *a = p.ws_acc + idx * kHeadDim + 4 * g;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        f32x4 v = acc[nt][mt];
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) v[r4] *= vs;
+        *(f32x4 *)(a + 16 * mt) = v;
+      }
+    }
+  }
+}
+
+template <int NT>
+__device__ __forceinline__ void load_q(const AttnParams &p, const int row0, const int qlen,
+                                       const int tq0, const int kvh, const int pos0,
+                                       Frag8 (&qf)[NT][2], RowInfo (&ri)[NT]) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int r = nt * 16 + i16;
+    const int t = tq0 + (r >> 3);
+    const bool valid = t < qlen;
+    const int tt = valid ? t : tq0;
+    const uint16_t *qp =
+        p.q + ((size_t)(row0 + tt) * p.num_q_heads + kvh * kGroup + (r & 7)) * kHeadDim + g * 16;
+    qf[nt][0].u = valid ? *(const u32x4 *)qp : u32x4{0, 0, 0, 0};
+    qf[nt][1].u = valid ? *(const u32x4 *)(qp + 8) : u32x4{0, 0, 0, 0};
+    ri[nt].pos = pos0 + tt;
+    ri[nt].lo = p.window > 0 ? max(0, ri[nt].pos - p.window + 1) : 0;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Split-KV kernel.  grid = (nparts_max, Hkv / WAVES, num_seqs); wave w of a workgroup owns
+// KV head blockIdx.y*WAVES + w of partition blockIdx.x of sequence blockIdx.z, so the
+// workgroup as a whole streams whole 16-token pages (all KV heads) of its partition.
+// ---------------------------------------------------------------------------------------
+template <int NT, bool FP8, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void splitkv_kernel(const AttnParams p) {
+  __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int part = blockIdx.x, s = blockIdx.z;
+  const int kvh = blockIdx.y * WAVES + wave;
+  int row0 = s, qlen = 1;
+  if (p.cu_seqlens_q) {
+    row0 = p.cu_seqlens_q[s];
+    qlen = p.cu_seqlens_q[s + 1] - row0;
+  }
+  if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows) return;
+  const int L = p.seq_lens[s];
+  if (L < qlen) return;
+  const int kb = kv_begin(L, qlen, p.window);
+  const int nparts = (L - kb + p.partition - 1) / p.partition;
+  if (part >= nparts) return;
+  const int t0 = kb + part * p.partition;
+  const int t1 = min(t0 + p.partition, L);
+  const int pos0 = L - qlen;
+  const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
+
+  Frag8 qf[NT][2];
+  RowInfo ri[NT];
+  load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
+  float m[NT], lsum[NT];
+  f32x4 acc[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    m[nt] = kNegBig;
+    lsum[nt] = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
+                  lsum, acc);
+  finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lsum, acc);
+}
+
+// ---------------------------------------------------------------------------------------
+// Tile kernel for long query chunks.  grid = (ceil(max_q_len / (WAVES*2*NT)), Hkv, num_seqs);
+// each wave owns 2*NT consecutive query tokens x 8 heads and walks its whole causal range.
+// ---------------------------------------------------------------------------------------
+template <int NT, bool FP8, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void tile_kernel(const AttnParams p) {
+  __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int s = blockIdx.z, kvh = blockIdx.y;
+  const int row0 = p.cu_seqlens_q[s];
+  const int qlen = p.cu_seqlens_q[s + 1] - row0;
+  if (qlen < p.qlen_lo || qlen > p.qlen_hi) return;
+  const int tq0 = (blockIdx.x * WAVES + wave) * (2 * NT);
+  if (tq0 >= qlen) return;
+  const int L = p.seq_lens[s];
+  if (L < qlen) return;
+  const int pos0 = L - qlen;
+  const int tq_last = min(tq0 + 2 * NT, qlen) - 1;
+  const int pos_first = pos0 + tq0, pos_last = pos0 + tq_last;
+  const int lo_first = p.window > 0 ? max(0, pos_first - p.window + 1) : 0;
+  const int lo_last = p.window > 0 ? max(0, pos_last - p.window + 1) : 0;
+
+  Frag8 qf[NT][2];
+  RowInfo ri[NT];
+  load_q<NT>(p, row0, qlen, tq0, kvh, pos0, qf, ri);
+  float m[NT], lsum[NT];
+  f32x4 acc[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    m[nt] = kNegBig;
+    lsum[nt] = 0.f;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  attend<NT, FP8>(p, s, kvh, lo_first & ~(kBlock - 1), pos_last + 1, L, pos_first, lo_last, qf,
+                  ri, lds + wave * kWaveLdsBytes, m, lsum, acc);
+  finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lsum, acc);
+}
+
+// ---------------------------------------------------------------------------------------
+// Cross-partition merge.  grid = (Hq / 4, num_seqs * ws_rows); one wave per (row, head),
+// lane = output dim.  Sequences finished by the split-KV kernel itself (one partition) and
+// sequences outside [qlen_lo, qlen_hi] are skipped.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
+  const int lane = threadIdx.x & 63;
+  const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int wsrow = blockIdx.y;
+  const int s = wsrow / p.ws_rows, t = wsrow % p.ws_rows;
+  int row0 = s, qlen = 1;
+  if (p.cu_seqlens_q) {
+    row0 = p.cu_seqlens_q[s];
+    qlen = p.cu_seqlens_q[s + 1] - row0;
+  }
+  if (qlen < p.qlen_lo || qlen > p.qlen_hi || t >= qlen) return;
+  const int L = p.seq_lens[s];
+  if (L < qlen) return;
+  const int kb = kv_begin(L, qlen, p.window);
+  const int nparts = min((L - kb + p.partition - 1) / p.partition, p.nparts_max);
+  if (nparts <= 1) return;
+
+  const size_t base = ((size_t)wsrow * p.num_q_heads + head) * p.nparts_max;
+  const float sink = p.sinks ? p.sinks[head] : -INFINITY;
+  float M = sink;
+  for (int c = lane; c < nparts; c += 64) {
+    const float2 ml = *(const float2 *)(p.ws_ml + (base + c) * 2);
+    if (ml.y > 0.f) M = fmaxf(M, ml.x);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
+  float den = fast_exp2((sink - M) * kLog2e);
+  float o = 0.f;
+  for (int c = 0; c < nparts; ++c) {
+    const float2 ml = *(const float2 *)(p.ws_ml + (base + c) * 2);
+    if (!(ml.y > 0.f)) continue;
+    const float w = fast_exp2((ml.x - M) * kLog2e);
+    den += ml.y * w;
+    o += p.ws_acc[(base + c) * kHeadDim + lane] * w;
+  }
+  const size_t orow = (size_t)(row0 + t) * p.num_q_heads + head;
+  const float val = o / den;
+  const uint32_t pk = pack_bf16(val, 0.f);
+  p.out[orow * kHeadDim + lane] = (uint16_t)(pk & 0xffffu);
+  if (p.lse && lane == 0) p.lse[orow] = M + __log2f(den) * kLn2;
+}
+
+// ---------------------------------------------------------------------------------------
+// Slot-mapped KV write.  grid = num_tokens, block = 128: thread e moves 8 elements of the
+// token's K row (first Hkv*8 threads) or V row (next Hkv*8 threads).
+// ---------------------------------------------------------------------------------------
+// Software round-to-nearest-even onto the OCP e4m3fn grid, saturating at +-448; NaN -> 0x7F.
+__device__ __forceinline__ uint32_t fp8_e4m3_encode(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return 0x7Fu;
+  if (a >= 0x43E00000u) return sign | 0x7Eu;  // |x| >= 448
+  if (a >= (121u << 23)) {                    // normal in e4m3: |x| >= 2^-6
+    uint32_t r = a + 0x7FFFFu + ((a >> 20) & 1u);
+    r >>= 20;  // exponent and 3 mantissa bits, carry propagated
+    return sign | (r - (120u << 3));
+  }
+  // subnormal: multiples of 2^-9; 8 rounds up into the smallest normal (0x08)
+  const float y = __uint_as_float(a) * 512.0f;
+  return sign | (uint32_t)__float2int_rn(y);
+}
+
+template <bool FP8>
+__global__ __launch_bounds__(128) void kv_write_kernel(const uint16_t *__restrict__ k_new,
+                                                       const uint16_t *__restrict__ v_new,
+                                                       uint8_t *__restrict__ k_cache,
+                                                       uint8_t *__restrict__ v_cache,
+                                                       const int64_t *__restrict__ slot_mapping,
+                                                       const float *__restrict__ k_scale,
+                                                       const float *__restrict__ v_scale,
+                                                       const int Hkv, const int64_t num_slots) {
+  const int t = blockIdx.x;
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0 || slot >= num_slots) return;
+  const int per = Hkv * (kHeadDim / 8);  // 16-byte groups per row
+  for (int e = threadIdx.x; e < 2 * per; e += blockDim.x) {
+    const bool is_v = e >= per;
+    const int idx = is_v ? e - per : e;
+    const uint16_t *src = (is_v ? v_new : k_new) + ((size_t)t * per + idx) * 8;
+    uint8_t *dst_base = is_v ? v_cache : k_cache;
+    const u32x4 raw = *(const u32x4 *)src;
+    if constexpr (FP8) {
+      const float sc = (is_v ? v_scale : k_scale)[idx / (kHeadDim / 8)];
+      uint32_t o[2] = {0, 0};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const uint32_t h = (raw[j >> 1] >> ((j & 1) * 16)) & 0xffffu;
+        const float x = __fdiv_rn(bf16_bits_to_f32(h), sc);
+        o[j >> 2] |= fp8_e4m3_encode(x) << ((j & 3) * 8);
+      }
+      *(u32x2 *)(dst_base + ((size_t)slot * per + idx) * 8) = u32x2{o[0], o[1]};
+    } else {
+      *(u32x4 *)(dst_base + ((size_t)slot * per + idx) * 16) = raw;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// Host-side launchers (called from the C ABI after validation).
+// ---------------------------------------------------------------------------------------
+template <int NT, bool FP8>
+static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
+  const int Hkv = p.num_kv_heads;
+  const int waves = Hkv >= 8 ? 8 : Hkv;
+  dim3 grid(p.nparts_max, Hkv / waves, p.num_seqs);
+  switch (waves) {
+    case 8: splitkv_kernel<NT, FP8, 8><<<grid, 512, 0, st>>>(p); break;
+    case 4: splitkv_kernel<NT, FP8, 4><<<grid, 256, 0, st>>>(p); break;
+    case 2: splitkv_kernel<NT, FP8, 2><<<grid, 128, 0, st>>>(p); break;
+    default: splitkv_kernel<NT, FP8, 1><<<grid, 64, 0, st>>>(p); break;
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
+  if (fp8) {
+    if (ntiles == 1) return launch_splitkv_t<1, true>(p, st);
+    return launch_splitkv_t<3, true>(p, st);
+  }
+  if (ntiles == 1) return launch_splitkv_t<1, false>(p, st);
+  return launch_splitkv_t<3, false>(p, st);
+}
+
+hipError_t launch_tile(const AttnParams &p, int max_q_len, bool fp8, hipStream_t st) {
+  constexpr int NT = 4, WAVES = 4;
+  const int tokens_per_wg = WAVES * 2 * NT;
+  dim3 grid((max_q_len + tokens_per_wg - 1) / tokens_per_wg, p.num_kv_heads, p.num_seqs);
+  if (fp8)
+    tile_kernel<NT, true, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
+  else
+    tile_kernel<NT, false, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
+  return hipGetLastError();
+}
+
+hipError_t launch_merge(const AttnParams &p, hipStream_t st) {
+  dim3 grid(p.num_q_heads / 4, p.num_seqs * p.ws_rows);
+  lse_merge_kernel<<<grid, 256, 0, st>>>(p);
+  return hipGetLastError();
+}
+
+hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
+                           uint8_t *v_cache, const int64_t *slot_mapping, const float *k_scale,
+                           const float *v_scale, int Hkv, int64_t num_slots, int num_tokens,
+                           bool fp8, hipStream_t st) {
+  if (num_tokens == 0) return hipSuccess;
+  if (fp8)
+    kv_write_kernel<true><<<num_tokens, 128, 0, st>>>(k_new, v_new, k_cache, v_cache,
+                                                      slot_mapping, k_scale, v_scale, Hkv,
+                                                      num_slots);
+  else
+    kv_write_kernel<false><<<num_tokens, 128, 0, st>>>(k_new, v_new, k_cache, v_cache,
+                                                       slot_mapping, k_scale, v_scale, Hkv,
+                                                       num_slots);
+  return hipGetLastError();
+}
+
+}  // namespace eid

@@ -1,0 +1,285 @@
+// C ABI of the paged sink-attention library: argument validation (no HIP calls), launch
+// planning (partition size, workspace layout) and dispatch to the gfx950 kernels.
+#include <hip/hip_runtime.h>
+
+#include "../../include/eidola_attn.h"
+#include "eid_params.h"
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+namespace eid {
+hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
+hipError_t launch_tile(const AttnParams &p, int max_q_len, bool fp8, hipStream_t st);
+hipError_t launch_merge(const AttnParams &p, hipStream_t st);
+hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
+                           uint8_t *v_cache, const int64_t *slot_mapping, const float *k_scale,
+                           const float *v_scale, int Hkv, int64_t num_slots, int num_tokens,
+                           bool fp8, hipStream_t st);
+}  // namespace eid
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int32_t fail(eid_status st, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  va_end(ap);
+  return (int32_t)st;
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Geometry checks shared by every entry point.
+int32_t check_geometry(const eid_attn_desc *d) {
+  if (!d) return fail(EID_ERR_INVALID_ARG, "desc is NULL");
+  if (d->struct_size != sizeof(eid_attn_desc))
+    return fail(EID_ERR_INVALID_ARG, "desc.struct_size %u != %zu", d->struct_size,
+                sizeof(eid_attn_desc));
+  if (d->head_dim != eid::kHeadDim)
+    return fail(EID_ERR_UNSUPPORTED, "head_dim %d unsupported (64 only)", d->head_dim);
+  if (d->block_size != eid::kBlock)
+    return fail(EID_ERR_UNSUPPORTED, "block_size %d unsupported (16 only)", d->block_size);
+  if (d->num_kv_heads <= 0 || d->num_q_heads <= 0)
+    return fail(EID_ERR_INVALID_ARG, "head counts must be positive");
+  if (d->num_q_heads != eid::kGroup * d->num_kv_heads)
+    return fail(EID_ERR_UNSUPPORTED, "num_q_heads %d must be 8 * num_kv_heads %d",
+                d->num_q_heads, d->num_kv_heads);
+  const int h = d->num_kv_heads;
+  if (!(h == 1 || h == 2 || h == 4 || h % 8 == 0))
+    return fail(EID_ERR_UNSUPPORTED, "num_kv_heads %d must be 1, 2, 4 or a multiple of 8", h);
+  if (d->kv_dtype != EID_KV_BF16 && d->kv_dtype != EID_KV_FP8_E4M3)
+    return fail(EID_ERR_INVALID_ARG, "kv_dtype %d unknown", d->kv_dtype);
+  if (d->num_blocks <= 0) return fail(EID_ERR_INVALID_ARG, "num_blocks must be positive");
+  return EID_OK;
+}
+
+int32_t check_attn_desc(const eid_attn_desc *d) {
+  int32_t rc = check_geometry(d);
+  if (rc) return rc;
+  if (d->num_seqs <= 0 || d->num_q_tokens <= 0)
+    return fail(EID_ERR_INVALID_ARG, "num_seqs and num_q_tokens must be positive");
+  if (d->num_seqs > 65535) return fail(EID_ERR_UNSUPPORTED, "num_seqs > 65535");
+  if (d->max_q_len <= 0 || d->max_q_len > d->num_q_tokens)
+    return fail(EID_ERR_INVALID_ARG, "max_q_len %d out of range", d->max_q_len);
+  if (d->num_q_tokens < d->num_seqs)
+    return fail(EID_ERR_INVALID_ARG, "num_q_tokens %d < num_seqs %d", d->num_q_tokens,
+                d->num_seqs);
+  if (d->max_kv_len <= 0) return fail(EID_ERR_INVALID_ARG, "max_kv_len must be positive");
+  if ((int64_t)d->max_blocks_per_seq * d->block_size < d->max_kv_len)
+    return fail(EID_ERR_INVALID_ARG, "max_blocks_per_seq %d cannot hold max_kv_len %d",
+                d->max_blocks_per_seq, d->max_kv_len);
+  if (!(d->softmax_scale > 0.f) || !std::isfinite(d->softmax_scale))
+    return fail(EID_ERR_INVALID_ARG, "softmax_scale must be finite and positive");
+  if (d->window < 0) return fail(EID_ERR_INVALID_ARG, "window must be >= 0");
+  if (d->partition_size != 0 &&
+      (d->partition_size < 64 || d->partition_size > 4096 || d->partition_size % 64 != 0))
+    return fail(EID_ERR_INVALID_ARG, "partition_size %d must be 0 or a multiple of 64 in [64,4096]",
+                d->partition_size);
+  return EID_OK;
+}
+
+struct Plan {
+  int32_t partition, nparts_max, ws_rows;
+  size_t ml_bytes, acc_bytes;
+};
+
+// Longest key span a split-KV sequence can have (from its first visible page to its end).
+int32_t max_span(const eid_attn_desc *d) {
+  if (d->window > 0) {
+    const int64_t w = (int64_t)d->window + eid::kShortQMax + eid::kBlock - 1;
+    return (int32_t)(w < d->max_kv_len ? w : d->max_kv_len);
+  }
+  return d->max_kv_len;
+}
+
+Plan make_plan(const eid_attn_desc *d) {
+  Plan pl;
+  const int32_t span = max_span(d);
+  int32_t P = d->partition_size;
+  if (P == 0) {
+    // Aim at ~8 workgroups per CU if every sequence were max length.
+    const int64_t target_wgs = 2048;
+    int64_t want = ((int64_t)span * d->num_seqs + target_wgs - 1) / target_wgs;
+    want = (want + 63) / 64 * 64;
+    if (want < 128) want = 128;
+    if (want > 1024) want = 1024;
+    P = (int32_t)want;
+  }
+  pl.partition = P;
+  pl.nparts_max = (span + P - 1) / P;
+  pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
+  const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
+  pl.ml_bytes = (cells * 2 * sizeof(float) + 255) / 256 * 256;
+  pl.acc_bytes = cells * eid::kHeadDim * sizeof(float);
+  return pl;
+}
+
+int32_t check_attn_args(const eid_attn_desc *d, const eid_attn_args *a, bool need_q,
+                        bool need_cu) {
+  if (!a) return fail(EID_ERR_INVALID_ARG, "args is NULL");
+  if (need_q && (!a->q || !a->k_cache || !a->v_cache || !a->block_table))
+    return fail(EID_ERR_INVALID_ARG, "q, k_cache, v_cache and block_table must be non-NULL");
+  if (!a->out || !a->seq_lens) return fail(EID_ERR_INVALID_ARG, "out and seq_lens must be non-NULL");
+  if (need_cu && !a->cu_seqlens_q) return fail(EID_ERR_INVALID_ARG, "cu_seqlens_q is NULL");
+  if (!aligned16(a->q) || !aligned16(a->out) || !aligned16(a->k_cache) || !aligned16(a->v_cache))
+    return fail(EID_ERR_INVALID_ARG, "q, out, k_cache and v_cache must be 16-byte aligned");
+  if (d->kv_dtype == EID_KV_FP8_E4M3 && need_q && (!a->k_scale || !a->v_scale))
+    return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
+  const Plan pl = make_plan(d);
+  if (!a->workspace || a->workspace_bytes < pl.ml_bytes + pl.acc_bytes)
+    return fail(EID_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given",
+                pl.ml_bytes + pl.acc_bytes, a->workspace ? a->workspace_bytes : (size_t)0);
+  if ((reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0)
+    return fail(EID_ERR_WORKSPACE, "workspace must be 256-byte aligned");
+  return EID_OK;
+}
+
+eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, const Plan &pl) {
+  eid::AttnParams p;
+  std::memset(&p, 0, sizeof p);
+  p.q = static_cast<const uint16_t *>(a->q);
+  p.out = static_cast<uint16_t *>(a->out);
+  p.lse = a->lse;
+  p.k_cache = static_cast<const uint8_t *>(a->k_cache);
+  p.v_cache = static_cast<const uint8_t *>(a->v_cache);
+  p.block_table = a->block_table;
+  p.cu_seqlens_q = a->cu_seqlens_q;
+  p.seq_lens = a->seq_lens;
+  p.sinks = a->sinks;
+  p.k_scale = a->k_scale;
+  p.v_scale = a->v_scale;
+  p.ws_ml = static_cast<float *>(a->workspace);
+  p.ws_acc = reinterpret_cast<float *>(static_cast<uint8_t *>(a->workspace) + pl.ml_bytes);
+  p.num_seqs = d->num_seqs;
+  p.num_q_heads = d->num_q_heads;
+  p.num_kv_heads = d->num_kv_heads;
+  p.max_blocks_per_seq = d->max_blocks_per_seq;
+  p.window = d->window;
+  p.partition = pl.partition;
+  p.nparts_max = pl.nparts_max;
+  p.ws_rows = pl.ws_rows;
+  p.softmax_scale = d->softmax_scale;
+  return p;
+}
+
+int32_t hip_fail(hipError_t e, const char *what) {
+  return fail(EID_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace
+
+extern "C" {
+
+uint32_t eid_version(void) { return (EID_VERSION_MAJOR << 16) | EID_VERSION_MINOR; }
+
+const char *eid_last_error(void) { return g_err; }
+
+int32_t eid_partition_size(const eid_attn_desc *desc) {
+  if (check_attn_desc(desc)) return 0;
+  return make_plan(desc).partition;
+}
+
+size_t eid_workspace_bytes(const eid_attn_desc *desc) {
+  if (check_attn_desc(desc)) return 0;
+  const Plan pl = make_plan(desc);
+  return pl.ml_bytes + pl.acc_bytes;
+}
+
+int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v_new,
+                     void *k_cache, void *v_cache, const int64_t *slot_mapping,
+                     int32_t num_tokens, const float *k_scale, const float *v_scale,
+                     void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_geometry(desc)) return rc;
+  if (num_tokens < 0) return fail(EID_ERR_INVALID_ARG, "num_tokens %d < 0", num_tokens);
+  if (num_tokens == 0) return EID_OK;
+  if (!k_new || !v_new || !k_cache || !v_cache || !slot_mapping)
+    return fail(EID_ERR_INVALID_ARG, "k_new, v_new, k_cache, v_cache, slot_mapping must be non-NULL");
+  if (!aligned16(k_new) || !aligned16(v_new) || !aligned16(k_cache) || !aligned16(v_cache))
+    return fail(EID_ERR_INVALID_ARG, "k_new, v_new, k_cache and v_cache must be 16-byte aligned");
+  const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  if (fp8 && (!k_scale || !v_scale)) return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
+  hipError_t e = eid::launch_kv_write(
+      static_cast<const uint16_t *>(k_new), static_cast<const uint16_t *>(v_new),
+      static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), slot_mapping, k_scale,
+      v_scale, desc->num_kv_heads, desc->num_blocks * desc->block_size, num_tokens, fp8,
+      static_cast<hipStream_t>(hip_stream));
+  if (e != hipSuccess) return hip_fail(e, "kv_write launch");
+  return EID_OK;
+}
+
+int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_attn_desc(desc)) return rc;
+  if (desc->max_q_len != 1 || desc->num_q_tokens != desc->num_seqs)
+    return fail(EID_ERR_INVALID_ARG, "decode needs max_q_len == 1 and num_q_tokens == num_seqs");
+  if (int32_t rc = check_attn_args(desc, args, true, false)) return rc;
+  const Plan pl = make_plan(desc);
+  eid::AttnParams p = make_params(desc, args, pl);
+  p.cu_seqlens_q = nullptr;  // one row per sequence by contract
+  p.qlen_lo = 1;
+  p.qlen_hi = 1;
+  hipStream_t st = static_cast<hipStream_t>(hip_stream);
+  const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  hipError_t e = eid::launch_splitkv(p, 1, fp8, st);
+  if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  if (pl.nparts_max > 1) {
+    e = eid::launch_merge(p, st);
+    if (e != hipSuccess) return hip_fail(e, "merge launch");
+  }
+  return EID_OK;
+}
+
+int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_attn_desc(desc)) return rc;
+  if (int32_t rc = check_attn_args(desc, args, true, true)) return rc;
+  const Plan pl = make_plan(desc);
+  eid::AttnParams p = make_params(desc, args, pl);
+  hipStream_t st = static_cast<hipStream_t>(hip_stream);
+  const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  hipError_t e;
+  // q_len 1..2: one 16-row tile per KV head
+  p.qlen_lo = 1;
+  p.qlen_hi = 2;
+  e = eid::launch_splitkv(p, 1, fp8, st);
+  if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  if (desc->max_q_len > 2) {  // q_len 3..6: three tiles
+    p.qlen_lo = 3;
+    p.qlen_hi = eid::kShortQMax;
+    e = eid::launch_splitkv(p, 3, fp8, st);
+    if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
+  }
+  if (desc->max_q_len > eid::kShortQMax) {  // long chunks: MFMA tile kernel
+    p.qlen_lo = eid::kShortQMax + 1;
+    p.qlen_hi = 0x7fffffff;
+    e = eid::launch_tile(p, desc->max_q_len, fp8, st);
+    if (e != hipSuccess) return hip_fail(e, "tile launch");
+  }
+  if (pl.nparts_max > 1) {
+    p.qlen_lo = 1;
+    p.qlen_hi = eid::kShortQMax;
+    e = eid::launch_merge(p, st);
+    if (e != hipSuccess) return hip_fail(e, "merge launch");
+  }
+  return EID_OK;
+}
+
+int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_attn_desc(desc)) return rc;
+  if (int32_t rc = check_attn_args(desc, args, false, false)) return rc;
+  const Plan pl = make_plan(desc);
+  eid::AttnParams p = make_params(desc, args, pl);
+  p.qlen_lo = 1;
+  p.qlen_hi = eid::kShortQMax;
+  hipError_t e = eid::launch_merge(p, static_cast<hipStream_t>(hip_stream));
+  if (e != hipSuccess) return hip_fail(e, "merge launch");
+  return EID_OK;
+}
+
+}  // extern "C"

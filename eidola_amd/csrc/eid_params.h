@@ -1,0 +1,44 @@
+// Host/device launch descriptors of the attention kernels (internal to the library).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+namespace eid {
+
+constexpr int kHeadDim = 64;
+constexpr int kBlock = 16;        // tokens per KV page
+constexpr int kGroup = 8;         // query heads per KV head
+constexpr int kShortQMax = 6;     // q_len handled by the split-KV kernel (6*8 = 48 rows = 3 tiles)
+constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the split-KV loop
+
+struct AttnParams {
+  const uint16_t *q;
+  uint16_t *out;
+  float *lse;
+  const uint8_t *k_cache;
+  const uint8_t *v_cache;
+  const int32_t *block_table;
+  const int32_t *cu_seqlens_q;  // may be null: q_len == 1 everywhere
+  const int32_t *seq_lens;
+  const float *sinks;    // may be null
+  const float *k_scale;  // fp8 only
+  const float *v_scale;  // fp8 only
+  float *ws_ml;          // [num_seqs*ws_rows][Hq][nparts_max][2]  (m natural-log units, l)
+  float *ws_acc;         // [num_seqs*ws_rows][Hq][nparts_max][64] (sum e^(s-m) v, v_scale applied)
+  int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;
+  int32_t window, partition, nparts_max, ws_rows;
+  int32_t qlen_lo, qlen_hi;  // this launch serves sequences with qlen_lo <= q_len <= qlen_hi
+  float softmax_scale;
+};
+
+// First key visible to any query row of a sequence, rounded down to a page boundary.
+__host__ __device__ inline int kv_begin(int seq_len, int q_len, int window) {
+  int p0 = seq_len - q_len;
+  if (p0 < 0) p0 = 0;
+  int lo = window > 0 ? p0 - window + 1 : 0;
+  if (lo < 0) lo = 0;
+  return lo & ~(kBlock - 1);
+}
+
+}  // namespace eid

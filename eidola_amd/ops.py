@@ -1,0 +1,228 @@
+"""Operator-level host API over the C ABI: tensors in, status-checked launches out.
+
+Every function takes torch tensors that already live on the GPU, checks dtype/shape/
+contiguity on the host, and passes raw device pointers plus the current HIP stream to the
+library.  Nothing here computes attention: if the HIP library is absent the call raises.
+"""
+import ctypes as C
+import math
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+from ._lib import AttnArgs, AttnDesc, KV_BF16, KV_FP8_E4M3, check, load_library
+
+
+@dataclass
+class AttnGeometry:
+    """Static shape of one attention layer and its paged KV cache."""
+    num_q_heads: int = 64
+    num_kv_heads: int = 8
+    head_dim: int = 64
+    block_size: int = 16
+    softmax_scale: float = 0.125
+    window: int = 0          # 0 = full causal
+    kv_dtype: int = KV_BF16
+    partition_size: int = 0  # 0 = library picks
+
+
+def make_desc(geom, *, num_seqs, num_q_tokens, max_q_len, max_kv_len, max_blocks_per_seq,
+              num_blocks):
+    d = AttnDesc()
+    d.struct_size = C.sizeof(AttnDesc)
+    d.num_seqs = num_seqs
+    d.num_q_tokens = num_q_tokens
+    d.max_q_len = max_q_len
+    d.max_kv_len = max_kv_len
+    d.num_q_heads = geom.num_q_heads
+    d.num_kv_heads = geom.num_kv_heads
+    d.head_dim = geom.head_dim
+    d.block_size = geom.block_size
+    d.max_blocks_per_seq = max_blocks_per_seq
+    d.num_blocks = num_blocks
+    d.softmax_scale = geom.softmax_scale
+    d.window = geom.window
+    d.kv_dtype = geom.kv_dtype
+    d.partition_size = geom.partition_size
+    return d
+
+
+def workspace_bytes(desc):
+    return load_library().eid_workspace_bytes(C.byref(desc))
+
+
+def partition_size(desc):
+    return load_library().eid_partition_size(C.byref(desc))
+
+
+def _ptr(t):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _kv_torch_dtype(kv_dtype):
+    return torch.bfloat16 if kv_dtype == KV_BF16 else torch.uint8
+
+
+def _require(t, name, dtype, ndim=None):
+    if t is None:
+        raise ValueError(f"{name} is None")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if ndim is not None and t.dim() != ndim:
+        raise ValueError(f"{name} must have {ndim} dims, got {t.dim()}")
+
+
+def _cache_view(t, geom, name):
+    """Accept fp8 caches as uint8 or torch.float8_e4m3fn storage."""
+    if geom.kv_dtype == KV_FP8_E4M3 and t.dtype == torch.float8_e4m3fn:
+        t = t.view(torch.uint8)
+    _require(t, name, _kv_torch_dtype(geom.kv_dtype), 4)
+    if tuple(t.shape[1:]) != (geom.block_size, geom.num_kv_heads, geom.head_dim):
+        raise ValueError(f"{name} must be [num_blocks, {geom.block_size}, {geom.num_kv_heads}, "
+                         f"{geom.head_dim}], got {tuple(t.shape)}")
+    return t
+
+
+def kv_write(geom, k_new, v_new, k_cache, v_cache, slot_mapping, k_scale=None, v_scale=None):
+    """Stage K1: cache_flat[slot_mapping[t]] = k_new[t] (bit copy, or fp8 quantise)."""
+    _require(k_new, "k_new", torch.bfloat16, 3)
+    _require(v_new, "v_new", torch.bfloat16, 3)
+    k_cache = _cache_view(k_cache, geom, "k_cache")
+    v_cache = _cache_view(v_cache, geom, "v_cache")
+    _require(slot_mapping, "slot_mapping", torch.int64, 1)
+    T = k_new.shape[0]
+    if tuple(k_new.shape) != (T, geom.num_kv_heads, geom.head_dim) or k_new.shape != v_new.shape:
+        raise ValueError("k_new / v_new must be [T, num_kv_heads, head_dim]")
+    if slot_mapping.shape[0] != T:
+        raise ValueError("slot_mapping must have one entry per new token")
+    if k_cache.shape != v_cache.shape:
+        raise ValueError("k_cache and v_cache shapes differ")
+    if geom.kv_dtype == KV_FP8_E4M3:
+        _require(k_scale, "k_scale", torch.float32, 1)
+        _require(v_scale, "v_scale", torch.float32, 1)
+    desc = make_desc(geom, num_seqs=1, num_q_tokens=1, max_q_len=1, max_kv_len=1,
+                     max_blocks_per_seq=1, num_blocks=k_cache.shape[0])
+    check(load_library().eid_kv_write(C.byref(desc), _ptr(k_new), _ptr(v_new), _ptr(k_cache),
+                                      _ptr(v_cache), _ptr(slot_mapping), T, _ptr(k_scale),
+                                      _ptr(v_scale), _stream()))
+
+
+def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q,
+               max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace,
+               return_lse):
+    _require(q, "q", torch.bfloat16, 3)
+    k_cache = _cache_view(k_cache, geom, "k_cache")
+    v_cache = _cache_view(v_cache, geom, "v_cache")
+    _require(block_table, "block_table", torch.int32, 2)
+    _require(seq_lens, "seq_lens", torch.int32, 1)
+    S = seq_lens.shape[0]
+    T = q.shape[0]
+    if tuple(q.shape[1:]) != (geom.num_q_heads, geom.head_dim):
+        raise ValueError("q must be [T, num_q_heads, head_dim]")
+    if block_table.shape[0] != S:
+        raise ValueError("block_table must have one row per sequence")
+    if cu_seqlens_q is not None:
+        _require(cu_seqlens_q, "cu_seqlens_q", torch.int32, 1)
+        if cu_seqlens_q.shape[0] != S + 1:
+            raise ValueError("cu_seqlens_q must have num_seqs + 1 entries")
+    if sinks is not None:
+        _require(sinks, "sinks", torch.float32, 1)
+    if geom.kv_dtype == KV_FP8_E4M3:
+        _require(k_scale, "k_scale", torch.float32, 1)
+        _require(v_scale, "v_scale", torch.float32, 1)
+    desc = make_desc(geom, num_seqs=S, num_q_tokens=T, max_q_len=max_q_len,
+                     max_kv_len=max_kv_len, max_blocks_per_seq=block_table.shape[1],
+                     num_blocks=k_cache.shape[0])
+    if out is None:
+        out = torch.empty_like(q)
+    else:
+        _require(out, "out", torch.bfloat16, 3)
+    if return_lse and lse is None:
+        lse = torch.empty((T, geom.num_q_heads), dtype=torch.float32, device=q.device)
+    lib = load_library()
+    need = lib.eid_workspace_bytes(C.byref(desc))
+    if need == 0:
+        check(getattr(lib, fn_name)(C.byref(desc), C.byref(AttnArgs()), None))
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    args = AttnArgs()
+    args.q = q.data_ptr()
+    args.out = out.data_ptr()
+    args.lse = lse.data_ptr() if lse is not None else None
+    args.k_cache = k_cache.data_ptr()
+    args.v_cache = v_cache.data_ptr()
+    args.block_table = block_table.data_ptr()
+    args.cu_seqlens_q = cu_seqlens_q.data_ptr() if cu_seqlens_q is not None else None
+    args.seq_lens = seq_lens.data_ptr()
+    args.sinks = sinks.data_ptr() if sinks is not None else None
+    args.k_scale = k_scale.data_ptr() if k_scale is not None else None
+    args.v_scale = v_scale.data_ptr() if v_scale is not None else None
+    args.workspace = workspace.data_ptr()
+    args.workspace_bytes = workspace.numel() * workspace.element_size()
+    check(getattr(lib, fn_name)(C.byref(desc), C.byref(args), _stream()))
+    return (out, lse) if return_lse else out
+
+
+def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, sinks=None,
+                k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
+                return_lse=False):
+    """Stages K2+K4: one query row per sequence (q is [num_seqs, Hq, D])."""
+    return _attn_call("eid_attn_decode", geom, q, k_cache, v_cache, block_table, seq_lens, None,
+                      1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse)
+
+
+def attn_varlen(geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, *, max_q_len,
+                max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
+                workspace=None, return_lse=False):
+    """Stages K2/K3+K4 on a ragged cu_seqlens batch (prefill chunks, verify rows, decodes)."""
+    return _attn_call("eid_attn_varlen", geom, q, k_cache, v_cache, block_table, seq_lens,
+                      cu_seqlens_q, max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse,
+                      workspace, return_lse)
+
+
+def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_len, max_kv_len,
+              max_blocks_per_seq, num_blocks, sinks=None, out=None, lse=None):
+    """Stage K4 alone over partials already present in `workspace` (see workspace_layout)."""
+    S = seq_lens.shape[0]
+    desc = make_desc(geom, num_seqs=S, num_q_tokens=num_q_tokens, max_q_len=max_q_len,
+                     max_kv_len=max_kv_len, max_blocks_per_seq=max_blocks_per_seq,
+                     num_blocks=num_blocks)
+    if out is None:
+        out = torch.zeros((num_q_tokens, geom.num_q_heads, geom.head_dim), dtype=torch.bfloat16,
+                          device=workspace.device)
+    args = AttnArgs()
+    args.out = out.data_ptr()
+    args.lse = lse.data_ptr() if lse is not None else None
+    args.cu_seqlens_q = cu_seqlens_q.data_ptr() if cu_seqlens_q is not None else None
+    args.seq_lens = seq_lens.data_ptr()
+    args.sinks = sinks.data_ptr() if sinks is not None else None
+    args.workspace = workspace.data_ptr()
+    args.workspace_bytes = workspace.numel() * workspace.element_size()
+    check(load_library().eid_lse_merge(C.byref(desc), C.byref(args), _stream()))
+    return out
+
+
+def workspace_layout(desc):
+    """(partition, nparts_max, ws_rows, ml_bytes): the split-KV workspace holds
+    ml  float32 [num_seqs*ws_rows, Hq, nparts_max, 2]  (m in natural-log units, l), then at
+    byte offset ml_bytes
+    acc float32 [num_seqs*ws_rows, Hq, nparts_max, 64] (sum of e^(s-m) * v)."""
+    P = partition_size(desc)
+    if desc.window > 0:
+        span = min(desc.max_kv_len, desc.window + 6 + desc.block_size - 1)
+    else:
+        span = desc.max_kv_len
+    nparts = (span + P - 1) // P
+    ws_rows = min(desc.max_q_len, 6)
+    cells = desc.num_seqs * ws_rows * desc.num_q_heads * nparts
+    ml_bytes = (cells * 8 + 255) // 256 * 256
+    return P, nparts, ws_rows, ml_bytes

@@ -1,0 +1,153 @@
+/*
+ * eidola_attn.h — C ABI of the MI355X (gfx950) ragged-batch paged sink-attention path.
+ *
+ * Reference interface replaced: NONE EXISTS.  eidola-ai/eidola performs no inference
+ * itself; its only seam towards an inference engine is an OpenAI-compatible HTTP
+ * boundary (crates/eidola-server/src/backend.rs:87-108 `trait ChatBackend`,
+ * crates/eidola-app-core/src/local_models.rs:1612-1626 engine spawn,
+ * crates/eidola-app-core/src/lib.rs:6616-6623 HTTP POST).  No tensor, pointer or shape
+ * crosses it.  Every entry point below is therefore defined by this library; each
+ * comment says which stage of the path it is and which engine-side call site would
+ * bind it.
+ *
+ * Conventions
+ *  - All tensor pointers are DEVICE pointers owned by the caller.  The library
+ *    allocates nothing and keeps no global mutable state except a thread-local
+ *    error string.
+ *  - All work is enqueued asynchronously on the caller's `hipStream_t`
+ *    (passed as `void *`; NULL = the default stream).
+ *  - Every function returns an `eid_status` (0 = OK, negative = error) and never
+ *    throws or aborts.  Argument validation runs before the first HIP call, so
+ *    invalid-argument paths can be exercised on a host without a GPU.
+ *
+ * Geometry supported by this version: head_dim 64, block_size 16,
+ * num_q_heads = 8 * num_kv_heads (GQA 8:1), bf16 Q/out, bf16 or fp8-e4m3fn KV.
+ *
+ * Tensor layouts (row-major, innermost last)
+ *   q, out            [num_q_tokens, num_q_heads, 64]  bf16   ragged by cu_seqlens_q
+ *   k_new, v_new      [num_tokens,   num_kv_heads, 64] bf16
+ *   k_cache, v_cache  [num_blocks, 16, num_kv_heads, 64]  bf16 or fp8-e4m3fn
+ *   slot_mapping      [num_tokens] int64   slot = block*16 + offset, -1 = skip
+ *   block_table       [num_seqs, max_blocks_per_seq] int32
+ *   cu_seqlens_q      [num_seqs + 1] int32
+ *   seq_lens          [num_seqs] int32   KV length AFTER this step's append
+ *   sinks             [num_q_heads] fp32 (NULL = no sink, i.e. -inf)
+ *   k_scale, v_scale  [num_kv_heads] fp32 (fp8 only)
+ *   lse               [num_q_tokens, num_q_heads] fp32 (optional) = m + ln(denominator)
+ */
+#ifndef EIDOLA_ATTN_H
+#define EIDOLA_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define EID_VERSION_MAJOR 0
+#define EID_VERSION_MINOR 1
+
+typedef enum {
+  EID_OK = 0,
+  EID_ERR_INVALID_ARG = -1, /* null pointer, bad shape, misalignment, bad struct_size */
+  EID_ERR_UNSUPPORTED = -2, /* geometry or dtype outside what this version builds    */
+  EID_ERR_WORKSPACE = -3,   /* workspace NULL or smaller than eid_workspace_bytes()  */
+  EID_ERR_HIP = -4          /* a HIP runtime call or kernel launch failed            */
+} eid_status;
+
+typedef enum { EID_KV_BF16 = 0, EID_KV_FP8_E4M3 = 1 } eid_kv_dtype;
+
+/* Shapes and scalars.  Plain data; `struct_size` must be sizeof(eid_attn_desc). */
+typedef struct eid_attn_desc {
+  uint32_t struct_size;
+  int32_t num_seqs;
+  int32_t num_q_tokens;       /* total rows of q / out                                   */
+  int32_t max_q_len;          /* max over sequences of cu_seqlens_q[s+1]-cu_seqlens_q[s] */
+  int32_t max_kv_len;         /* max over sequences of seq_lens[s]                       */
+  int32_t num_q_heads;        /* 64 */
+  int32_t num_kv_heads;       /* 8  */
+  int32_t head_dim;           /* 64 */
+  int32_t block_size;         /* 16 */
+  int32_t max_blocks_per_seq; /* row stride of block_table                               */
+  int64_t num_blocks;         /* blocks in each of k_cache / v_cache                     */
+  float softmax_scale;        /* 1/sqrt(head_dim) normally                               */
+  int32_t window;             /* 0 = full causal; W>0: row at position p sees p-W+1..p   */
+  int32_t kv_dtype;           /* eid_kv_dtype                                            */
+  int32_t partition_size;     /* split-KV partition in tokens; 0 = library picks; else a
+                                 multiple of 64 in [64, 4096]                            */
+} eid_attn_desc;
+
+/* Device pointers, all caller-owned. */
+typedef struct eid_attn_args {
+  const void *q;
+  void *out;
+  float *lse; /* may be NULL */
+  const void *k_cache;
+  const void *v_cache;
+  const int32_t *block_table;
+  const int32_t *cu_seqlens_q; /* may be NULL for eid_attn_decode (q_len == 1 for all) */
+  const int32_t *seq_lens;
+  const float *sinks;   /* may be NULL */
+  const float *k_scale; /* fp8 only */
+  const float *v_scale; /* fp8 only */
+  void *workspace;      /* >= eid_workspace_bytes(desc), 256-byte aligned */
+  size_t workspace_bytes;
+} eid_attn_args;
+
+/*
+ * Stage K1 — slot-mapped KV-cache write ("reshape and cache").
+ * cache_flat[slot_mapping[t], h, :] = f(k_new[t, h, :]) for every t with slot >= 0.
+ * bf16: bit copy.  fp8: RNE_e4m3fn(clamp(fp32(x) / scale[h], -448, 448)), NaN -> 0x7F.
+ * Only desc->num_kv_heads, head_dim, block_size, num_blocks, kv_dtype are read.
+ * Reference counterpart: none.  Engine call site: once per layer per step, after the
+ * QKV projection and before attention, on the same stream.
+ */
+int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v_new,
+                     void *k_cache, void *v_cache, const int64_t *slot_mapping,
+                     int32_t num_tokens, const float *k_scale, const float *v_scale,
+                     void *hip_stream);
+
+/*
+ * Stages K2+K4 — decode attention: every sequence contributes exactly one query row
+ * (num_q_tokens == num_seqs, max_q_len == 1).  Split-KV over partitions of
+ * `partition_size` tokens with the per-head sink folded into the denominator once, in
+ * the merge.  Reference counterpart: none.  Engine call site: per layer per decode step.
+ */
+int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args,
+                        void *hip_stream);
+
+/*
+ * Stages K2/K3+K4 — ragged attention in cu_seqlens layout: chunked prefill, speculative
+ * verify and mixed prefill+decode batches.  Query row i of sequence s sits at absolute
+ * position seq_lens[s] - q_len_s + i and sees keys 0..position (clipped by `window`).
+ * Sequences with q_len <= 6 run on the bandwidth-bound split-KV kernel; longer chunks
+ * run on the bf16-MFMA tile kernel.  Reference counterpart: none.
+ */
+int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
+                        void *hip_stream);
+
+/*
+ * Stage K4 alone — merge the split-KV partials found in args->workspace (as laid out by
+ * the split-KV kernel for this desc) into args->out / args->lse.  Exposed for tests.
+ */
+int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
+                      void *hip_stream);
+
+/* Bytes of workspace eid_attn_decode / eid_attn_varlen / eid_lse_merge need for desc.
+ * Returns 0 for an invalid desc. */
+size_t eid_workspace_bytes(const eid_attn_desc *desc);
+
+/* The partition size (tokens) the library will use for desc (resolves the 0 default). */
+int32_t eid_partition_size(const eid_attn_desc *desc);
+
+/* Thread-local description of the last error on this thread; "" if none. */
+const char *eid_last_error(void);
+
+/* (major << 16) | minor */
+uint32_t eid_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* EIDOLA_ATTN_H */

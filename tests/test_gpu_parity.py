@@ -1,0 +1,363 @@
+"""GPU parity tests: the HIP path, called through the C ABI, against the CPU oracle.
+
+Bars: KV writes bit-exact; attention outputs within max-abs 2e-2 / mean-abs 2e-3 of the
+fp64 oracle (bf16 output, fp32 accumulation).  Parity is against this repository's own
+oracle: the reference holds no implementation of this path."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import eidola_amd as ea
+from eidola_amd import KV_BF16, KV_FP8_E4M3, synth
+from eidola_amd.ops import workspace_layout
+
+from helpers import (make_batch, desc_of, logical_tensors, cpu_caches, oracle_out, fp8_scales,
+                     all_slots, empty_caches, assert_close)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def G():
+    import gpu_helpers
+    assert torch.cuda.is_available()
+    ea.load_library()       # raises if the HIP extension has not been built
+    return gpu_helpers
+
+
+# ---------------------------------------------------------------- K1: kv_write
+def test_kv_write_bf16_bit_exact_with_skips_and_poison(G):
+    b = make_batch([37, 128, 511, 1000, 5], [1, 1, 1, 1, 1], num_blocks=200)
+    q, k, v, _ = logical_tensors(b)
+    sm = all_slots(b)
+    sm[::17] = -1
+    kc, vc = empty_caches(b)
+    oracle.kv_write(desc_of(b), k, v, kc, vc, sm)
+    kc_d, vc_d = G.cache_dev(empty_caches(b)[0]), G.cache_dev(empty_caches(b)[1])
+    ea.kv_write(b.geom, G.bf16_dev(k), G.bf16_dev(v), kc_d, vc_d, G.dev(sm))
+    torch.cuda.synchronize()
+    assert np.array_equal(G.cache_host(kc_d), kc)
+    assert np.array_equal(G.cache_host(vc_d), vc)
+
+
+def test_kv_write_empty_and_all_skipped(G):
+    b = make_batch([16], [1])
+    kc, vc = empty_caches(b)
+    kc_d, vc_d = G.cache_dev(kc), G.cache_dev(vc)
+    z = torch.empty((0, 8, 64), dtype=torch.bfloat16, device=G.DEV)
+    ea.kv_write(b.geom, z, z, kc_d, vc_d, torch.empty(0, dtype=torch.int64, device=G.DEV))
+    q, k, v, _ = logical_tensors(b)
+    ea.kv_write(b.geom, G.bf16_dev(k), G.bf16_dev(v), kc_d, vc_d,
+                torch.full((16,), -1, dtype=torch.int64, device=G.DEV))
+    torch.cuda.synchronize()
+    assert np.array_equal(G.cache_host(kc_d), kc) and np.array_equal(G.cache_host(vc_d), vc)
+
+
+@pytest.mark.parametrize("scale", [1.0, 0.0078125, 3.7e-3, 0.013671875, 123.456])
+def test_kv_write_fp8_exhaustive_over_all_bf16_inputs(G, scale):
+    """Every one of the 65,536 bf16 bit patterns, as K and (bit-reversed order) as V."""
+    n_tok = 65536 // (8 * 64)
+    b = make_batch([n_tok], [1], kv_dtype=KV_FP8_E4M3, shuffle=True)
+    k = np.arange(65536, dtype=np.uint32).astype(np.uint16).reshape(n_tok, 8, 64)
+    v = k[::-1].copy()
+    ks = np.full(8, scale, np.float32) * np.array([1, 2, 0.5, 1, 3, 1, 7, 1], np.float32)
+    vs = ks[::-1].copy()
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    torch.cuda.synchronize()
+    assert np.array_equal(G.cache_host(kc_d), kc)
+    assert np.array_equal(G.cache_host(vc_d), vc)
+
+
+# ---------------------------------------------------------------- config 1 (plumbing)
+def test_config1_plumbing_decode(G):
+    b = synth.config1()
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    assert np.array_equal(G.cache_host(kc_d), kc) and np.array_equal(G.cache_host(vc_d), vc)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+    assert_close(out, ref, "config1")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+# ---------------------------------------------------------------- decode, ragged edge cases
+@pytest.mark.parametrize("window", [0, 1, 16, 128])
+@pytest.mark.parametrize("partition", [0, 64, 128, 512])
+def test_decode_ragged_edges(G, window, partition):
+    seq_lens = [1, 2, 15, 16, 17, 63, 64, 65, 127, 128, 129, 500, 1024, 1500]
+    b = make_batch(seq_lens, [1] * len(seq_lens), window=window, partition=partition)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+    assert_close(out, ref, f"decode w={window} P={partition}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+def test_decode_without_sinks_and_with_extreme_sinks(G):
+    b = make_batch([300, 40, 700], [1, 1, 1], partition=128)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    for sk in (None, np.full(64, 30.0, np.float32), np.full(64, -30.0, np.float32)):
+        ref, _ = oracle_out(b, q, kc, vc, sk)
+        out = G.run_attn(b, q, kc_d, vc_d, sk)
+        assert_close(out, ref, f"sinks={None if sk is None else sk[0]}")
+
+
+def test_decode_two_kv_heads(G):
+    b = make_batch([200, 33], [1, 1], num_kv_heads=2, partition=64)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "Hkv=2")
+
+
+def test_decode_is_invariant_under_page_permutation_bitwise(G):
+    seq_lens = [700, 45, 1030]
+    a = make_batch(seq_lens, [1, 1, 1], seed=21, partition=256)
+    c = make_batch(seq_lens, [1, 1, 1], seed=22, num_blocks=400, partition=256)
+    q, k, v, sinks = logical_tensors(a, seed=5)
+    outs = []
+    for b in (a, c):
+        kc_d, vc_d = G.gpu_caches(b, k, v)
+        outs.append(G.run_attn(b, q, kc_d, vc_d, sinks))
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_garbage_beyond_sequence_end_is_never_used(G):
+    """Slots past seq_len inside the last page hold NaN patterns (poison) in K and V."""
+    b = make_batch([33, 100], [1, 1])
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)              # unwritten slots stay 0x7FC1 (NaN)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "poison tail")
+
+
+# ---------------------------------------------------------------- varlen: verify rows
+@pytest.mark.parametrize("window", [0, 128])
+@pytest.mark.parametrize("partition", [0, 512])
+def test_verify_five_rows(G, window, partition):
+    seq_lens = [5, 21, 130, 517, 1029, 2300]
+    b = make_batch(seq_lens, [5] * len(seq_lens), window=window, partition=partition)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+    assert_close(out, ref, f"verify w={window} P={partition}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+def test_verify_row_equals_decode_row(G):
+    L = 777
+    b5 = make_batch([L], [5], partition=256)
+    q, k, v, sinks = logical_tensors(b5)
+    kc_d, vc_d = G.gpu_caches(b5, k, v)
+    out5 = synth.bf16_bits_to_f32(G.run_attn(b5, q, kc_d, vc_d, sinks))
+    for t in (0, 4):
+        b1 = make_batch([L - 4 + t], [1], partition=256)
+        k1, v1 = k[:L - 4 + t], v[:L - 4 + t]
+        kc1, vc1 = G.gpu_caches(b1, k1, v1)
+        out1 = synth.bf16_bits_to_f32(G.run_attn(b1, q[t:t + 1], kc1, vc1, sinks))
+        assert np.abs(out5[t] - out1[0]).max() <= 1e-2
+
+
+@pytest.mark.parametrize("window", [0, 40])
+def test_varlen_mixed_short_lengths(G, window):
+    seq_lens = [9, 64, 300, 31, 1000, 6, 450]
+    q_lens = [1, 2, 3, 4, 5, 6, 1]
+    b = make_batch(seq_lens, q_lens, window=window, partition=128)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, f"mixed short w={window}")
+
+
+# ---------------------------------------------------------------- varlen: prefill chunks
+@pytest.mark.parametrize("window", [0, 128])
+def test_prefill_chunks_and_decodes_mixed(G, window):
+    seq_lens = [7, 40, 100 + 64, 512, 300 + 512, 1, 200, 33]
+    q_lens = [7, 40, 64, 512, 512, 1, 1, 5]
+    b = make_batch(seq_lens, q_lens, window=window)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+    assert_close(out, ref, f"prefill mixed w={window}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+def test_varlen_at_qlen1_equals_decode_entry_point(G):
+    b = make_batch([100, 1000, 17], [1, 1, 1], partition=128)
+    q, k, v, sinks = logical_tensors(b)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    a = G.run_attn(b, q, kc_d, vc_d, sinks, decode=True)
+    c = G.run_attn(b, q, kc_d, vc_d, sinks, decode=False)
+    assert np.array_equal(a, c)
+
+
+# ---------------------------------------------------------------- fp8 KV
+@pytest.mark.parametrize("q_len", [1, 5, 48])
+def test_fp8_kv_attention(G, q_len):
+    seq_lens = [130, 64, 900, 2100]
+    b = make_batch(seq_lens, [q_len] * 4, kv_dtype=KV_FP8_E4M3, partition=256)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    assert np.array_equal(G.cache_host(kc_d), kc) and np.array_equal(G.cache_host(vc_d), vc)
+    ref, _ = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs), ref, f"fp8 q_len={q_len}")
+
+
+def test_fp8_every_code_dequantises_exactly(G):
+    """One-key attention returns v0 * sigmoid(s0 - sink): with a huge negative sink the
+    output is the dequantised V row itself, for all 254 finite codes."""
+    n_tok = 4
+    b = make_batch([1] * n_tok, [1] * n_tok, kv_dtype=KV_FP8_E4M3)
+    codes = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    vc = np.zeros((b.num_blocks, 16, 8, 64), np.uint8)
+    kc = np.zeros_like(vc)
+    flat = vc.reshape(-1, 8 * 64)
+    for s in range(n_tok):
+        slot = int(b.all_slots(s)[0])
+        flat[slot] = np.resize(np.roll(codes, 64 * s), 512)
+    vs = np.ones(8, np.float32)
+    q = np.zeros((n_tok, 64, 64), np.uint16)
+    sinks = np.full(64, -100.0, np.float32)
+    out = G.run_attn(b, q, G.cache_dev(kc), G.cache_dev(vc), sinks, vs, vs)
+    got = synth.bf16_bits_to_f32(out).reshape(n_tok, 8, 8, 64)
+    for s in range(n_tok):
+        want = oracle.fp8_decode(flat[int(b.all_slots(s)[0])]).reshape(8, 1, 64)
+        assert np.array_equal(got[s], np.broadcast_to(want, (8, 8, 64)))
+
+
+# ---------------------------------------------------------------- K4 alone
+def test_lse_merge_entry_point_against_oracle_merge(G):
+    seq_lens, q_lens = [700, 1300, 90], [5, 5, 5]
+    b = make_batch(seq_lens, q_lens, partition=128)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    d = desc_of(b)
+    P, nparts, ws_rows, ml_bytes = workspace_layout(d)
+    assert P == 128 and ws_rows == 5
+    ml, acc = oracle.splitkv_f64(d, P, nparts, q, kc, vc, b.block_table, b.seq_lens, b.cu_seqlens_q)
+    ref, ref_lse = oracle.lse_merge_f64(ml, acc, sinks)
+    full, _ = oracle_out(b, q, kc, vc, sinks)
+    assert np.allclose(ref, full, rtol=1e-10, atol=1e-13)
+    # workspace rows are (sequence, row-in-sequence); here every sequence has ws_rows rows
+    ws = np.zeros(ea.workspace_bytes(d), np.uint8)
+    ws[:ml.size * 4] = ml.astype(np.float32).reshape(-1).view(np.uint8)
+    ws[ml_bytes:ml_bytes + acc.size * 4] = acc.astype(np.float32).reshape(-1).view(np.uint8)
+    ws_d = torch.from_numpy(ws).to(G.DEV)
+    lse_d = torch.zeros((15, 64), dtype=torch.float32, device=G.DEV)
+    out = ea.ops.lse_merge(b.geom, ws_d, G.dev(b.seq_lens), G.dev(b.cu_seqlens_q),
+                           num_q_tokens=15, max_q_len=5, max_kv_len=1300,
+                           max_blocks_per_seq=b.block_table.shape[1], num_blocks=b.num_blocks,
+                           sinks=G.dev(sinks), lse=lse_d)
+    torch.cuda.synchronize()
+    # sequence 2 (90 tokens) has one partition: the merge leaves its rows to the main kernel
+    assert_close(G.bits_host(out)[:10], ref[:10], "merge")
+    assert np.allclose(lse_d.cpu().numpy()[:10], ref_lse[:10], atol=1e-4)
+    assert (G.bits_host(out)[10:] == 0).all()
+
+
+# ---------------------------------------------------------------- benchmark configurations
+def _sample_check(G, b, q_d, kc_d, vc_d, sinks, out_d, seqs, what, ks=None, vs=None):
+    sub, kc, vc = G.compact_to_cpu(b, kc_d, vc_d, seqs)
+    rows = G.rows_of(b, seqs)
+    qb = G.bits_host(q_d)[rows]
+    ref, _ = oracle.attn_f64(desc_of(sub), qb, kc, vc, sub.block_table, sub.seq_lens,
+                             sub.cu_seqlens_q, sinks, ks, vs)
+    return assert_close(G.bits_host(out_d)[rows], ref, what)
+
+
+def _gpu_inputs(G, b, pool_seed=7):
+    g = b.geom
+    dt = torch.uint8 if g.kv_dtype == KV_FP8_E4M3 else torch.bfloat16
+    kc_d = torch.empty((b.num_blocks, 16, 8, 64), dtype=dt, device=G.DEV)
+    vc_d = torch.empty_like(kc_d)
+    ks, vs = synth.fill_pool_gpu(g, kc_d, vc_d, pool_seed)
+    q = synth.normal_bf16((b.num_q_tokens, 64, 64), b.seed, synth.TID_Q)
+    sinks = synth.bf16_bits_to_f32(synth.normal_bf16((64,), b.seed, synth.TID_SINK))
+    return G.bf16_dev(q), kc_d, vc_d, sinks, ks, vs
+
+
+@pytest.mark.parametrize("window", [0, 128])
+def test_config2_full_size(G, window):
+    b = synth.config2(window=window)
+    assert b.num_seqs == 64 and b.block_table.shape[1] == 512
+    q_d, kc_d, vc_d, sinks, _, _ = _gpu_inputs(G, b)
+    args = (b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens))
+    out = ea.attn_decode(*args, max_kv_len=b.max_kv_len, sinks=G.dev(sinks))
+    torch.cuda.synchronize()
+    order = np.argsort(b.seq_lens)
+    seqs = [int(order[0]), int(order[31]), int(order[-1])] + list(range(4))
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, seqs, f"config2 w={window}")
+    # size-independent properties: partition size does not matter beyond fp32 round-off
+    o = synth.bf16_bits_to_f32(G.bits_host(out))
+    assert np.isfinite(o).all()
+    for P in (128, 1024):
+        g2 = b.with_geom(partition_size=P).geom
+        o2 = ea.attn_decode(g2, *args[1:], max_kv_len=b.max_kv_len, sinks=G.dev(sinks))
+        torch.cuda.synchronize()
+        assert np.abs(synth.bf16_bits_to_f32(G.bits_host(o2)) - o).max() <= 4e-3
+
+
+def test_config3_mixed_full_size(G):
+    b = synth.config3()
+    assert b.num_q_tokens == 4216 and b.num_seqs == 128
+    q_d, kc_d, vc_d, sinks, _, _ = _gpu_inputs(G, b)
+    # slot-mapped write of every new token precedes attention
+    k_new = synth.normal_bf16((4216, 8, 64), b.seed, synth.TID_K)
+    v_new = synth.normal_bf16((4216, 8, 64), b.seed, synth.TID_V)
+    ea.kv_write(b.geom, G.bf16_dev(k_new), G.bf16_dev(v_new), kc_d, vc_d, G.dev(b.slot_mapping))
+    flat = kc_d.view(-1, 8, 64)
+    got = G.bits_host(flat[torch.from_numpy(b.slot_mapping).to(G.DEV)])
+    assert np.array_equal(got, k_new)
+    out = ea.attn_varlen(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                         G.dev(b.cu_seqlens_q), max_q_len=512, max_kv_len=b.max_kv_len,
+                         sinks=G.dev(sinks))
+    torch.cuda.synchronize()
+    assert np.isfinite(synth.bf16_bits_to_f32(G.bits_host(out))).all()
+    pre = int(np.argmin(b.seq_lens[:8]))
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [pre, 8, 9, 60, 127], "config3")
+
+
+def test_config4_fp8_full_size(G):
+    b = synth.config4()
+    assert b.num_seqs == 256 and 128 <= b.seq_lens.min() and b.seq_lens.max() <= 32768
+    q_d, kc_d, vc_d, sinks, ks, vs = _gpu_inputs(G, b)
+    out = ea.attn_decode(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                         max_kv_len=b.max_kv_len, sinks=G.dev(sinks), k_scale=ks, v_scale=vs)
+    torch.cuda.synchronize()
+    order = np.argsort(b.seq_lens)
+    seqs = [int(order[0]), int(order[128]), int(order[-1]), 0, 1]
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, seqs, "config4",
+                  ks.cpu().numpy(), vs.cpu().numpy())
+
+
+@pytest.mark.parametrize("layer", [0, 1])
+def test_config5_verify_full_size(G, layer):
+    b = synth.config5(layer=layer)
+    assert b.num_q_tokens == 640 and b.geom.partition_size == 512
+    q_d, kc_d, vc_d, sinks, _, _ = _gpu_inputs(G, b, pool_seed=9 + layer)
+    out = ea.attn_varlen(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                         G.dev(b.cu_seqlens_q), max_q_len=5, max_kv_len=b.max_kv_len,
+                         sinks=G.dev(sinks))
+    torch.cuda.synchronize()
+    assert np.isfinite(synth.bf16_bits_to_f32(G.bits_host(out))).all()
+    order = np.argsort(b.seq_lens)
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [int(order[0]), int(order[64]), int(order[-1])],
+                  f"config5 layer {layer}")
