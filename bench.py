@@ -1,0 +1,271 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged sink-attention hot path on one MI355X.
+
+A step = one pass of the hot path over one synthetic batch of BASELINE.json's decode
+configuration (configs[1], full-attention variant): the slot-mapped KV write of the 64 new
+tokens followed by split-KV decode attention + merge, all inputs resident in HBM.  Page
+sets rotate between steps so the 256 MB Infinity Cache cannot serve the KV stream.
+
+Prints ONE JSON line on stdout.  `--all` additionally measures the other configurations
+and writes them (one JSON object per line) to the file given by --report.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+METRIC = "paged sink-attn decode HBM GB/s (% peak) + ragged-batch tokens/s, 1 GPU"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def event_ms(fn, iters, torch):
+    """Average milliseconds per call of fn over `iters` back-to-back calls (HIP events on
+    torch's current stream, which is the stream every launch here uses)."""
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for i in range(iters):
+        fn(i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+class Workload:
+    """One configuration materialised on the GPU with `nsets` disjoint page sets."""
+
+    def __init__(self, make_batch, nsets, pool_seed, torch, ea, synth, kind):
+        self.kind = kind  # "decode" or "varlen"
+        dev = "cuda:0"
+        b0 = make_batch(0)
+        nblk = int(((b0.seq_lens.astype("int64") + 15) // 16).sum())
+        self.batches = [b0] + [make_batch(r * nblk) for r in range(1, nsets)]
+        g = b0.geom
+        self.geom = g
+        dt = torch.uint8 if g.kv_dtype == ea.KV_FP8_E4M3 else torch.bfloat16
+        self.k_cache = torch.empty((b0.num_blocks, 16, g.num_kv_heads, 64), dtype=dt, device=dev)
+        self.v_cache = torch.empty_like(self.k_cache)
+        t0 = time.time()
+        self.k_scale, self.v_scale = synth.fill_pool_gpu(g, self.k_cache, self.v_cache, pool_seed)
+        torch.cuda.synchronize()
+        log(f"[bench] {b0.name}: pool of {b0.num_blocks} blocks filled in {time.time()-t0:.1f}s, "
+            f"{nsets} page sets of {nblk} blocks")
+        T = b0.num_q_tokens
+
+        def bf16(bits):
+            import numpy as np
+            return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).to(dev).view(torch.bfloat16)
+
+        self.q = bf16(synth.normal_bf16((T, g.num_q_heads, 64), b0.seed, synth.TID_Q))
+        self.k_new = bf16(synth.normal_bf16((T, g.num_kv_heads, 64), b0.seed, synth.TID_K))
+        self.v_new = bf16(synth.normal_bf16((T, g.num_kv_heads, 64), b0.seed, synth.TID_V))
+        self.sinks = torch.from_numpy(synth.bf16_bits_to_f32(
+            synth.normal_bf16((g.num_q_heads,), b0.seed, synth.TID_SINK))).to(dev)
+        self.seq_lens = torch.from_numpy(b0.seq_lens).to(dev)
+        self.cu = torch.from_numpy(b0.cu_seqlens_q).to(dev)
+        self.slots = [torch.from_numpy(b.slot_mapping).to(dev) for b in self.batches]
+        self.tables = [torch.from_numpy(b.block_table).to(dev) for b in self.batches]
+        fn = "eid_attn_decode" if kind == "decode" else "eid_attn_varlen"
+        ws = None
+        self.attn, self.merge = [], []
+        for bt in self.tables:
+            kw = dict(max_q_len=b0.max_q_len, max_kv_len=b0.max_kv_len, sinks=self.sinks,
+                      k_scale=self.k_scale, v_scale=self.v_scale, workspace=ws)
+            cu = self.cu if kind == "varlen" else None
+            c = ea.prepare(fn, g, self.q, self.k_cache, self.v_cache, bt, self.seq_lens, cu, **kw)
+            ws = c._keep[-1]
+            self.attn.append(c)
+            kw["workspace"] = ws
+            self.merge.append(ea.prepare("eid_lse_merge", g, self.q, self.k_cache, self.v_cache,
+                                         bt, self.seq_lens, cu, **kw))
+        self.ea = ea
+        self.n = nsets
+
+    def kv_write(self, i):
+        self.ea.kv_write(self.geom, self.k_new, self.v_new, self.k_cache, self.v_cache,
+                         self.slots[i % self.n], self.k_scale, self.v_scale)
+
+    def step(self, i):
+        self.kv_write(i)
+        self.attn[i % self.n]()
+
+
+def measure(w, steps, warmup, torch, synth, label):
+    b = w.batches[0]
+    for i in range(warmup):
+        w.step(i)
+    ms_step = event_ms(w.step, steps, torch)
+    ms_attn = event_ms(lambda i: w.attn[i % w.n](), steps, torch)
+    ms_merge = event_ms(lambda i: w.merge[i % w.n](), steps, torch)
+    ms_write = event_ms(w.kv_write, steps, torch)
+    work = synth.algorithmic_work(b)
+    work_w = synth.algorithmic_work(b, include_kv_write=True)
+    r = {
+        "config": label, "ms_per_step": ms_step, "ms_attn": ms_attn, "ms_merge": ms_merge,
+        "ms_kv_write": ms_write, "alg_bytes": work["bytes"], "alg_flops": work["flops"],
+        "q_tokens": work["q_tokens"], "ctx_tokens": work["ctx_tokens"],
+        "step_GBps": work_w["bytes"] / ms_step / 1e6,
+        "attn_GBps": work["bytes"] / ms_attn / 1e6,
+        "attn_TFLOPs": work["flops"] / ms_attn / 1e9,
+        "q_tokens_per_s": work["q_tokens"] / ms_step * 1e3,
+        "ctx_tokens_per_s": work["ctx_tokens"] / ms_step * 1e3,
+    }
+    log(f"[bench] {label}: step {ms_step*1e3:.1f} us (attn {ms_attn*1e3:.1f}, merge "
+        f"{ms_merge*1e3:.1f}, kv_write {ms_write*1e3:.1f}); attn {r['attn_GBps']:.0f} GB/s = "
+        f"{100*r['attn_GBps']/HBM_PEAK_GBS:.1f}% HBM, {r['attn_TFLOPs']:.1f} TFLOP/s")
+    return r
+
+
+def cpu_baseline(w, torch, synth, threads):
+    """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
+    one full pass over page set 0 of the decode configuration."""
+    import numpy as np
+    import oracle
+    import eidola_amd as ea
+    b = w.batches[0]
+    nblk = (b.seq_lens.astype(np.int64) + 15) // 16
+    pages = np.concatenate([b.block_table[s, :n] for s, n in enumerate(nblk)])
+    idx = torch.from_numpy(pages.astype(np.int64)).to("cuda:0")
+
+    def host(t):
+        t = t[idx].cpu().contiguous()
+        return t.numpy() if t.dtype == torch.uint8 else t.view(torch.int16).numpy().view(np.uint16)
+
+    kc, vc = host(w.k_cache), host(w.v_cache)
+    bt = np.zeros((b.num_seqs, int(nblk.max())), np.int32)
+    off = 0
+    for s, n in enumerate(nblk):
+        bt[s, :n] = np.arange(off, off + n)
+        off += int(n)
+    d = ea.make_desc(b.geom, num_seqs=b.num_seqs, num_q_tokens=b.num_q_tokens,
+                     max_q_len=b.max_q_len, max_kv_len=b.max_kv_len,
+                     max_blocks_per_seq=bt.shape[1], num_blocks=len(pages))
+    q = w.q.cpu().view(torch.int16).numpy().view(np.uint16)
+    sinks = w.sinks.cpu().numpy()
+    ks = w.k_scale.cpu().numpy() if w.k_scale is not None else None
+    vs = w.v_scale.cpu().numpy() if w.v_scale is not None else None
+    args = (d, q, kc, vc, bt, b.seq_lens, b.cu_seqlens_q, sinks, ks, vs)
+    oracle.attn_bf16(*args, num_threads=threads)           # warm-up (page-in, thread pool)
+    reps, t0 = 0, time.time()
+    while True:
+        out, _ = oracle.attn_bf16(*args, num_threads=threads)
+        reps += 1
+        if time.time() - t0 > 8.0 or reps >= 20:
+            break
+    dt = (time.time() - t0) / reps
+    # cross-check while we are here: GPU result of set 0 against the CPU path
+    gpu = w.attn[0]().cpu().view(torch.int16).numpy().view(np.uint16)
+    err = np.abs(synth.bf16_bits_to_f32(gpu).astype(np.float64)
+                 - synth.bf16_bits_to_f32(out).astype(np.float64))
+    work = synth.algorithmic_work(b)
+    return {"value": work["bytes"] / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"{reps} full passes of the same 64-sequence decode batch "
+                      f"({work['ctx_tokens']} context tokens), {dt:.2f} s each; "
+                      "CPU restatement of this repo (no reference CPU path exists)",
+            "tokens_per_s": work["q_tokens"] / dt,
+            "gpu_vs_cpu_max_abs_diff": float(err.max())}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--sets", type=int, default=8, help="disjoint page sets rotated between steps")
+    ap.add_argument("--all", action="store_true", help="also measure the other configurations")
+    ap.add_argument("--report", default=os.path.join(ROOT, "gpurun_out", "bench_all.jsonl"))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--partition", type=int, default=0)
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this path runs on ONE MI355X (no sharding, no collectives); "
+                 "--gpus must be 1")
+    import torch
+    import eidola_amd as ea
+    from eidola_amd import synth
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    ea.load_library()
+
+    w = Workload(lambda off: synth.config2(perm_offset=off).with_geom(partition_size=a.partition),
+                 a.sets, 7, torch, ea, synth, "decode")
+    r = measure(w, a.steps, a.warmup, torch, synth, "config2_decode_full")
+    split_ms = r["ms_attn"] - r["ms_merge"]
+    achieved = r["alg_bytes"] / split_ms / 1e6
+    line = {
+        "metric": METRIC, "value": r["step_GBps"], "unit": "GB/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (seeded ragged batch, N(0,1) bf16 Q/K/V and sinks, random-permuted pages)",
+        "config": {"workload": "configs[1] decode continuous batch, full attention: 64 seqs, "
+                               "ctx U[1,8192], Hq64/Hkv8/D64, block 16, 300k-block pool; "
+                               "step = kv_write(64 tokens) + split-KV decode + LSE merge",
+                   "partition_size": ea.partition_size(w.attn[0].desc),
+                   "page_sets_rotated": a.sets},
+        "pct_hbm_peak": 100 * r["step_GBps"] / HBM_PEAK_GBS,
+        "tokens_per_s": r["q_tokens_per_s"], "ctx_tokens_per_s": r["ctx_tokens_per_s"],
+        "breakdown_us": {"kv_write": r["ms_kv_write"] * 1e3, "attn_call": r["ms_attn"] * 1e3,
+                         "merge": r["ms_merge"] * 1e3},
+        "roofline": {"bound": "hbm", "kernel": "splitkv_kernel<1,bf16,8 waves>",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "alg_bytes_per_launch": r["alg_bytes"], "launch_us": split_ms * 1e3,
+                     "how": "HIP events: (eid_attn_decode call) minus (eid_lse_merge call)"},
+    }
+    extra = [r]
+    if a.all:
+        w = None
+        torch.cuda.empty_cache()
+        ww = Workload(lambda off: synth.config2(window=128, perm_offset=off), a.sets, 7, torch, ea,
+                      synth, "decode")
+        extra.append(measure(ww, a.steps, a.warmup, torch, synth, "config2_decode_w128"))
+        ww = None
+        torch.cuda.empty_cache()
+        w3 = Workload(lambda off: synth.config3(perm_offset=off), 4, 8, torch, ea, synth, "varlen")
+        r3 = measure(w3, max(20, a.steps // 4), a.warmup, torch, synth, "config3_mixed")
+        lw = synth.algorithmic_work(w3.batches[0], rows="long")
+        sw = synth.algorithmic_work(w3.batches[0], rows="short")
+        r3["prefill_flops"], r3["decode_rows_bytes"] = lw["flops"], sw["bytes"]
+        extra.append(r3)
+        w3 = None
+        torch.cuda.empty_cache()
+        w4 = Workload(lambda off: synth.config4(num_blocks=300_000, perm_offset=off), 3, 9, torch,
+                      ea, synth, "decode")
+        extra.append(measure(w4, max(20, a.steps // 2), a.warmup, torch, synth, "config4_fp8_decode"))
+        w4 = None
+        torch.cuda.empty_cache()
+        for layer in (0, 1):
+            w5 = Workload(lambda off: synth.config5(layer=layer, num_blocks=900_000, perm_offset=off),
+                          3, 10 + layer, torch, ea, synth, "varlen")
+            extra.append(measure(w5, max(10, a.steps // 10), max(3, a.warmup // 4), torch, synth,
+                                 f"config5_verify_layer{layer}"))
+            w5 = None
+            torch.cuda.empty_cache()
+        w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
+    if not a.no_cpu:
+        threads = min(16, os.cpu_count() or 1)
+        line["cpu_baseline"] = cpu_baseline(w, torch, synth, threads)
+    else:
+        line["cpu_baseline"] = None
+    try:
+        os.makedirs(os.path.dirname(a.report), exist_ok=True)
+        with open(a.report, "w") as f:
+            for e in extra:
+                f.write(json.dumps(e) + "\n")
+    except OSError:
+        pass
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -172,6 +172,59 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
     return (out, lse) if return_lse else out
 
 
+class PreparedCall:
+    """A validated (desc, args) pair bound to one entry point: calling it only crosses the
+    C ABI (no tensor checks, no allocation), for launch-rate-sensitive loops.  The tensors
+    are kept alive by the object."""
+
+    def __init__(self, fn_name, desc, args, keep, out, lse):
+        self._fn = getattr(load_library(), fn_name)
+        self.desc, self.args, self._keep, self.out, self.lse = desc, args, keep, out, lse
+        self._d, self._a = C.byref(desc), C.byref(args)
+
+    def __call__(self, stream=None):
+        st = _stream() if stream is None else C.c_void_p(stream)
+        rc = self._fn(self._d, self._a, st)
+        if rc:
+            check(rc)
+        return self.out
+
+
+def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, *,
+            max_q_len=1, max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
+            workspace=None):
+    """Build a PreparedCall for "eid_attn_decode" / "eid_attn_varlen" / "eid_lse_merge"."""
+    k_cache = _cache_view(k_cache, geom, "k_cache")
+    v_cache = _cache_view(v_cache, geom, "v_cache")
+    _require(q, "q", torch.bfloat16, 3)
+    _require(block_table, "block_table", torch.int32, 2)
+    _require(seq_lens, "seq_lens", torch.int32, 1)
+    desc = make_desc(geom, num_seqs=seq_lens.shape[0], num_q_tokens=q.shape[0],
+                     max_q_len=max_q_len, max_kv_len=max_kv_len,
+                     max_blocks_per_seq=block_table.shape[1], num_blocks=k_cache.shape[0])
+    need = load_library().eid_workspace_bytes(C.byref(desc))
+    if need == 0:
+        check(getattr(load_library(), fn_name)(C.byref(desc), C.byref(AttnArgs()), None))
+    if out is None:
+        out = torch.empty_like(q)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    args = AttnArgs()
+    args.q, args.out = q.data_ptr(), out.data_ptr()
+    args.lse = lse.data_ptr() if lse is not None else None
+    args.k_cache, args.v_cache = k_cache.data_ptr(), v_cache.data_ptr()
+    args.block_table, args.seq_lens = block_table.data_ptr(), seq_lens.data_ptr()
+    args.cu_seqlens_q = cu_seqlens_q.data_ptr() if cu_seqlens_q is not None else None
+    args.sinks = sinks.data_ptr() if sinks is not None else None
+    args.k_scale = k_scale.data_ptr() if k_scale is not None else None
+    args.v_scale = v_scale.data_ptr() if v_scale is not None else None
+    args.workspace = workspace.data_ptr()
+    args.workspace_bytes = workspace.numel()
+    keep = (q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, sinks, k_scale, v_scale,
+            workspace)
+    return PreparedCall(fn_name, desc, args, keep, out, lse)
+
+
 def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, sinks=None,
                 k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
                 return_lse=False):
