@@ -186,6 +186,8 @@ def main():
     ap.add_argument("--report", default=os.path.join(ROOT, "gpurun_out", "bench_all.jsonl"))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--partition", type=int, default=0)
+    ap.add_argument("--no-shuffle", action="store_true",
+                    help="experiment: physically contiguous pages instead of a shuffled pool")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this path runs on ONE MI355X (no sharding, no collectives); "
@@ -197,7 +199,8 @@ def main():
         sys.exit("bench.py needs a GPU")
     ea.load_library()
 
-    w = Workload(lambda off: synth.config2(perm_offset=off).with_geom(partition_size=a.partition),
+    w = Workload(lambda off: synth.config2(perm_offset=off, shuffle=not a.no_shuffle)
+                 .with_geom(partition_size=a.partition),
                  a.sets, 7, torch, ea, synth, "decode")
     r = measure(w, a.steps, a.warmup, torch, synth, "config2_decode_full")
     split_ms = r["ms_attn"] - r["ms_merge"]

@@ -78,6 +78,9 @@ _lib = None
 
 
 def lib_path():
+    override = os.environ.get("EID_ATTN_LIB")   # an alternative build of the same ABI
+    if override:
+        return override
     return os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
                         "libeidola_attn_hip.so")
 

@@ -53,13 +53,14 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
   const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
 
-  int ids = 0;
-  int ci = 0;
-  for (int tc = t_begin; tc < t_end; tc += kChunk, ++ci) {
-    if ((ci & 15) == 0) {  // page ids of the next 1024 tokens, one per lane
-      const int bi = tc / kBlock + lane;
-      ids = bi < nblk_total ? bt[bi] : 0;
-    }
+  // Page ids travel through scalar registers: the table row and the index are wave-uniform,
+  // so these are scalar loads that never share a wait counter with the K/V vector loads.
+  // The ids of chunk i+1 are fetched while chunk i is in flight.
+  int blk[4];
+#pragma unroll
+  for (int b = 0; b < 4; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
+
+  for (int tc = t_begin; tc < t_end; tc += kChunk) {
     const int nb = min(4, (t_end - tc + kBlock - 1) / kBlock);
 
     // ---- global loads: each lane takes 32 B (bf16) / 16 B (fp8) of one token row ----
@@ -72,9 +73,8 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         vraw[b][e] = u32x4{0, 0, 0, 0};
       }
       if (b < nb) {
-        const int blk = __builtin_amdgcn_readlane(ids, (ci & 15) * 4 + b);
-        const uint8_t *kp = p.k_cache + (size_t)blk * page_bytes + lane_off;
-        const uint8_t *vp = p.v_cache + (size_t)blk * page_bytes + lane_off;
+        const uint8_t *kp = p.k_cache + (size_t)blk[b] * page_bytes + lane_off;
+        const uint8_t *vp = p.v_cache + (size_t)blk[b] * page_bytes + lane_off;
 #pragma unroll
         for (int e = 0; e < kElt; ++e) {
           kraw[b][e] = ldg128(kp + 16 * e);
@@ -82,7 +82,22 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         }
       }
     }
+    if (tc + kChunk < t_end) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) blk[b] = bt[min((tc + kChunk) / kBlock + b, nblk_total - 1)];
+    }
 
+#if defined(EID_ABLATE) && EID_ABLATE == 1
+    {
+      u32x4 x = {0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int e = 0; e < kElt; ++e) x ^= kraw[b][e] ^ vraw[b][e];
+      acc[0][0][0] += __uint_as_float((x[0] ^ x[1] ^ x[2] ^ x[3]) & 0x3fffffffu);
+      continue;
+    }
+#endif
     // ---- V: zero rows past the sequence end, widen fp8, stage in LDS ----
     const bool tail = tc + kChunk > seq_len;
 #pragma unroll
@@ -267,28 +282,77 @@ __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, cons
   }
 }
 
+// Work-item lookup shared by the split-KV kernel: the launch serves the compacted list of
+// (sequence, partition) pairs of all sequences whose q_len lies in [qlen_lo, qlen_hi],
+// enumerated sequence-major.  Item `w` is found by a wave-wide prefix sum over the
+// per-sequence partition counts (64 sequences per pass).  Consecutive items go to
+// consecutive workgroup ids, which the hardware deals round-robin to the 8 XCDs, so every
+// XCD receives the same number of equal-sized items whatever the raggedness of the batch;
+// ids past the end of the list are the only ones that exit without work.
+struct WorkItem {
+  int seq, part, nparts, row0, qlen, seq_len;
+};
+
+__device__ __forceinline__ int wave_inclusive_scan(int v, const int lane) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int o = __shfl_up(v, off);
+    if (lane >= off) v += o;
+  }
+  return v;
+}
+
+__device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w, WorkItem &it) {
+  const int lane = threadIdx.x & 63;
+  int base = 0;
+  for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
+    const int s = s0 + lane;
+    int n = 0, row0 = 0, qlen = 0, L = 0;
+    if (s < p.num_seqs) {
+      L = p.seq_lens[s];
+      row0 = s;
+      qlen = 1;
+      if (p.cu_seqlens_q) {
+        row0 = p.cu_seqlens_q[s];
+        qlen = p.cu_seqlens_q[s + 1] - row0;
+      }
+      if (qlen >= p.qlen_lo && qlen <= p.qlen_hi && qlen <= p.ws_rows && L >= qlen)
+        n = min((L - kv_begin(L, qlen, p.window) + p.partition - 1) / p.partition, p.nparts_max);
+    }
+    const int incl = wave_inclusive_scan(n, lane);
+    const int total = __builtin_amdgcn_readlane(incl, 63);
+    if (w < base + total) {
+      const unsigned long long hit = __ballot(base + incl > w);
+      const int idx = __builtin_ctzll(hit);
+      it.seq = s0 + idx;
+      it.nparts = __builtin_amdgcn_readlane(n, idx);
+      it.part = w - (base + __builtin_amdgcn_readlane(incl, idx) - it.nparts);
+      it.row0 = __builtin_amdgcn_readlane(row0, idx);
+      it.qlen = __builtin_amdgcn_readlane(qlen, idx);
+      it.seq_len = __builtin_amdgcn_readlane(L, idx);
+      return true;
+    }
+    base += total;
+  }
+  return false;
+}
+
 // ---------------------------------------------------------------------------------------
-// Split-KV kernel.  grid = (nparts_max, Hkv / WAVES, num_seqs); wave w of a workgroup owns
-// KV head blockIdx.y*WAVES + w of partition blockIdx.x of sequence blockIdx.z, so the
-// workgroup as a whole streams whole 16-token pages (all KV heads) of its partition.
+// Split-KV kernel.  grid = (num_seqs * nparts_max, Hkv / WAVES); workgroup blockIdx.x takes
+// work item blockIdx.x (see find_work_item) and wave w of it owns KV head
+// blockIdx.y*WAVES + w, so the workgroup as a whole streams whole 16-token pages (all KV
+// heads) of its partition.
 // ---------------------------------------------------------------------------------------
 template <int NT, bool FP8, int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void splitkv_kernel(const AttnParams p) {
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int part = blockIdx.x, s = blockIdx.z;
   const int kvh = blockIdx.y * WAVES + wave;
-  int row0 = s, qlen = 1;
-  if (p.cu_seqlens_q) {
-    row0 = p.cu_seqlens_q[s];
-    qlen = p.cu_seqlens_q[s + 1] - row0;
-  }
-  if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows) return;
-  const int L = p.seq_lens[s];
-  if (L < qlen) return;
+  WorkItem it;
+  if (!find_work_item(p, blockIdx.x, it)) return;
+  const int s = it.seq, part = it.part, nparts = it.nparts;
+  const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
   const int kb = kv_begin(L, qlen, p.window);
-  const int nparts = (L - kb + p.partition - 1) / p.partition;
-  if (part >= nparts) return;
   const int t0 = kb + part * p.partition;
   const int t1 = min(t0 + p.partition, L);
   const int pos0 = L - qlen;
@@ -460,7 +524,7 @@ template <int NT, bool FP8>
 static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
   const int Hkv = p.num_kv_heads;
   const int waves = Hkv >= 8 ? 8 : Hkv;
-  dim3 grid(p.nparts_max, Hkv / waves, p.num_seqs);
+  dim3 grid(p.num_seqs * p.nparts_max, Hkv / waves);
   switch (waves) {
     case 8: splitkv_kernel<NT, FP8, 8><<<grid, 512, 0, st>>>(p); break;
     case 4: splitkv_kernel<NT, FP8, 4><<<grid, 256, 0, st>>>(p); break;

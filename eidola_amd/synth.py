@@ -121,13 +121,14 @@ class Batch:
 
 
 def build_block_table(seq_lens, num_blocks, seed, block_size=16, max_blocks_per_seq=None,
-                      perm_offset=0):
-    """Physical pages = consecutive slices of a seeded permutation of the pool."""
+                      perm_offset=0, shuffle=True):
+    """Physical pages = consecutive slices of a seeded permutation of the pool
+    (shuffle=False: of 0..num_blocks-1 in order, for locality experiments)."""
     nblk = (np.asarray(seq_lens, dtype=np.int64) + block_size - 1) // block_size
     total = int(nblk.sum())
     if perm_offset + total > num_blocks:
         raise ValueError(f"pool of {num_blocks} blocks cannot hold {perm_offset + total}")
-    perm = permutation(num_blocks, seed, TID_PERM)
+    perm = permutation(num_blocks, seed, TID_PERM) if shuffle else np.arange(num_blocks, dtype=np.int32)
     mb = int(max_blocks_per_seq or nblk.max())
     if mb < nblk.max():
         raise ValueError("max_blocks_per_seq too small")
@@ -151,13 +152,13 @@ def config1():
     return Batch("config1_plumbing", _geom(), L, np.ones(4, dtype=np.int32), bt, 128, 0)
 
 
-def config2(window=0, scale=1.0, num_blocks=300_000, perm_offset=0):
+def config2(window=0, scale=1.0, num_blocks=300_000, perm_offset=0, shuffle=True):
     """Decode continuous batch: 64 sequences, contexts U{1..8192*scale}."""
     seed = 2
     hi = max(1, int(8192 * scale))
     L = randint(64, 1, hi, seed, TID_LEN)
     bt = build_block_table(L, num_blocks, seed, max_blocks_per_seq=max(1, (hi + 15) // 16),
-                           perm_offset=perm_offset)
+                           perm_offset=perm_offset, shuffle=shuffle)
     name = f"config2_decode_{'w%d' % window if window else 'full'}"
     return Batch(name, _geom(window=window), L, np.ones(64, dtype=np.int32), bt, num_blocks, seed)
 
