@@ -15,6 +15,9 @@
 #include "eid_device.h"
 #include "eid_params.h"
 
+#include <cstdio>
+#include <cstdlib>
+
 namespace eid {
 
 constexpr int kVRowBytes = 144;                 // 128 B of bf16 + 16 B pad (bank spread)
@@ -87,17 +90,6 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
       for (int b = 0; b < 4; ++b) blk[b] = bt[min((tc + kChunk) / kBlock + b, nblk_total - 1)];
     }
 
-#if defined(EID_ABLATE) && EID_ABLATE == 1
-    {
-      u32x4 x = {0, 0, 0, 0};
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int e = 0; e < kElt; ++e) x ^= kraw[b][e] ^ vraw[b][e];
-      acc[0][0][0] += __uint_as_float((x[0] ^ x[1] ^ x[2] ^ x[3]) & 0x3fffffffu);
-      continue;
-    }
-#endif
     // ---- V: zero rows past the sequence end, widen fp8, stage in LDS ----
     const bool tail = tc + kChunk > seq_len;
 #pragma unroll
@@ -302,23 +294,67 @@ __device__ __forceinline__ int wave_inclusive_scan(int v, const int lane) {
   return v;
 }
 
-__device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w, WorkItem &it) {
+// Per-lane view of one sequence for the planning passes: partitions are counted from the
+// first visible page (kv_begin) to the end of the sequence.
+struct SeqView {
+  int span, row0, qlen, seq_len;
+};
+
+__device__ __forceinline__ SeqView view_seq(const AttnParams &p, const int s) {
+  SeqView v{0, 0, 0, 0};
+  if (s < p.num_seqs) {
+    v.seq_len = p.seq_lens[s];
+    v.row0 = s;
+    v.qlen = 1;
+    if (p.cu_seqlens_q) {
+      v.row0 = p.cu_seqlens_q[s];
+      v.qlen = p.cu_seqlens_q[s + 1] - v.row0;
+    }
+    if (v.qlen >= p.qlen_lo && v.qlen <= p.qlen_hi && v.qlen <= p.ws_rows && v.seq_len >= v.qlen)
+      v.span = v.seq_len - kv_begin(v.seq_len, v.qlen, p.window);
+  }
+  return v;
+}
+
+// Partition size of this launch.  Fixed when the caller gave one.  Otherwise every wave
+// derives the same value from the batch itself: the smallest multiple of 64 (>= the
+// planning minimum that sized the workspace) for which the item list fits in a whole
+// number R of device fills, R being the fewest fills that keep a partition <= the cap:
+//   items <= total/P + active <= target_items * R.
+__device__ __forceinline__ int effective_partition(const AttnParams &p) {
+  if (!p.dynamic_partition) return p.partition;
+  const int lane = threadIdx.x & 63;
+  long long total = 0;
+  int active = 0;
+  for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
+    const SeqView v = view_seq(p, s0 + lane);
+    total += v.span;
+    active += v.span > 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    total += __shfl_xor(total, off);
+    active += __shfl_xor(active, off);
+  }
+  const long long T = max(p.target_items, 1);
+  const long long R = max(1LL, (total / kDynPartitionCap + active + T - 1) / T);
+  const long long denom = max(1LL, T * R - active);
+  long long P = ((total + denom - 1) / denom + 63) / 64 * 64;
+  P = max(P, (long long)p.partition);
+  return (int)min(P, 1LL << 20);
+}
+
+__device__ __forceinline__ int num_partitions(const AttnParams &p, const int span, const int P) {
+  return min((span + P - 1) / P, p.nparts_max);
+}
+
+__device__ __forceinline__ bool find_work_item(const AttnParams &p, const int P, const int w,
+                                               WorkItem &it) {
   const int lane = threadIdx.x & 63;
   int base = 0;
   for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
-    const int s = s0 + lane;
-    int n = 0, row0 = 0, qlen = 0, L = 0;
-    if (s < p.num_seqs) {
-      L = p.seq_lens[s];
-      row0 = s;
-      qlen = 1;
-      if (p.cu_seqlens_q) {
-        row0 = p.cu_seqlens_q[s];
-        qlen = p.cu_seqlens_q[s + 1] - row0;
-      }
-      if (qlen >= p.qlen_lo && qlen <= p.qlen_hi && qlen <= p.ws_rows && L >= qlen)
-        n = min((L - kv_begin(L, qlen, p.window) + p.partition - 1) / p.partition, p.nparts_max);
-    }
+    const SeqView v = view_seq(p, s0 + lane);
+    const int n = num_partitions(p, v.span, P);
     const int incl = wave_inclusive_scan(n, lane);
     const int total = __builtin_amdgcn_readlane(incl, 63);
     if (w < base + total) {
@@ -327,9 +363,9 @@ __device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w,
       it.seq = s0 + idx;
       it.nparts = __builtin_amdgcn_readlane(n, idx);
       it.part = w - (base + __builtin_amdgcn_readlane(incl, idx) - it.nparts);
-      it.row0 = __builtin_amdgcn_readlane(row0, idx);
-      it.qlen = __builtin_amdgcn_readlane(qlen, idx);
-      it.seq_len = __builtin_amdgcn_readlane(L, idx);
+      it.row0 = __builtin_amdgcn_readlane(v.row0, idx);
+      it.qlen = __builtin_amdgcn_readlane(v.qlen, idx);
+      it.seq_len = __builtin_amdgcn_readlane(v.seq_len, idx);
       return true;
     }
     base += total;
@@ -348,13 +384,14 @@ __global__ __launch_bounds__(WAVES * 64) void splitkv_kernel(const AttnParams p)
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.y * WAVES + wave;
+  const int P = effective_partition(p);
   WorkItem it;
-  if (!find_work_item(p, blockIdx.x, it)) return;
+  if (!find_work_item(p, P, blockIdx.x, it)) return;
   const int s = it.seq, part = it.part, nparts = it.nparts;
   const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
   const int kb = kv_begin(L, qlen, p.window);
-  const int t0 = kb + part * p.partition;
-  const int t1 = min(t0 + p.partition, L);
+  const int t0 = kb + part * P;
+  const int t1 = min(t0 + P, L);
   const int pos0 = L - qlen;
   const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
 
@@ -416,8 +453,10 @@ __global__ __launch_bounds__(WAVES * 64) void tile_kernel(const AttnParams p) {
 
 // ---------------------------------------------------------------------------------------
 // Cross-partition merge.  grid = (Hq / 4, num_seqs * ws_rows); one wave per (row, head),
-// lane = output dim.  Sequences finished by the split-KV kernel itself (one partition) and
-// sequences outside [qlen_lo, qlen_hi] are skipped.
+// lane = output dim.  The (m, l) pairs of up to 64 partitions are fetched one per lane, the
+// weights e^(m_c - M) are formed lane-parallel, and the accumulator rows are then streamed
+// with independent loads.  Sequences finished by the split-KV kernel itself (one
+// partition) and sequences outside [qlen_lo, qlen_hi] are skipped.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   const int lane = threadIdx.x & 63;
@@ -429,15 +468,16 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
     row0 = p.cu_seqlens_q[s];
     qlen = p.cu_seqlens_q[s + 1] - row0;
   }
-  if (qlen < p.qlen_lo || qlen > p.qlen_hi || t >= qlen) return;
+  if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
   const int L = p.seq_lens[s];
   if (L < qlen) return;
-  const int kb = kv_begin(L, qlen, p.window);
-  const int nparts = min((L - kb + p.partition - 1) / p.partition, p.nparts_max);
+  const int P = effective_partition(p);
+  const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
   if (nparts <= 1) return;
 
   const size_t base = ((size_t)wsrow * p.num_q_heads + head) * p.nparts_max;
   const float sink = p.sinks ? p.sinks[head] : -INFINITY;
+  // pass 1: global maximum over non-empty partitions and the sink
   float M = sink;
   for (int c = lane; c < nparts; c += 64) {
     const float2 ml = *(const float2 *)(p.ws_ml + (base + c) * 2);
@@ -445,18 +485,38 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
-  float den = fast_exp2((sink - M) * kLog2e);
-  float o = 0.f;
-  for (int c = 0; c < nparts; ++c) {
-    const float2 ml = *(const float2 *)(p.ws_ml + (base + c) * 2);
-    if (!(ml.y > 0.f)) continue;
-    const float w = fast_exp2((ml.x - M) * kLog2e);
-    den += ml.y * w;
-    o += p.ws_acc[(base + c) * kHeadDim + lane] * w;
+  // pass 2: weights per lane, accumulator rows with four loads in flight
+  float den = 0.f, o = 0.f;
+  for (int c0 = 0; c0 < nparts; c0 += 64) {
+    float w = 0.f, lw = 0.f;
+    if (c0 + lane < nparts) {
+      const float2 ml = *(const float2 *)(p.ws_ml + (base + c0 + lane) * 2);
+      if (ml.y > 0.f) {
+        w = fast_exp2((ml.x - M) * kLog2e);
+        lw = ml.y * w;
+      }
+    }
+    den += lw;
+    const int n = min(64, nparts - c0);
+    const float *a = p.ws_acc + (base + c0) * kHeadDim + lane;
+    int c = 0;
+    for (; c + 4 <= n; c += 4) {
+      const float a0 = a[(c + 0) * kHeadDim], a1 = a[(c + 1) * kHeadDim];
+      const float a2 = a[(c + 2) * kHeadDim], a3 = a[(c + 3) * kHeadDim];
+      o += a0 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 0));
+      o += a1 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 1));
+      o += a2 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 2));
+      o += a3 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 3));
+    }
+    for (; c < n; ++c)
+      o += a[c * kHeadDim] *
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c));
   }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) den += __shfl_xor(den, off);
+  den += fast_exp2((sink - M) * kLog2e);
   const size_t orow = (size_t)(row0 + t) * p.num_q_heads + head;
-  const float val = o / den;
-  const uint32_t pk = pack_bf16(val, 0.f);
+  const uint32_t pk = pack_bf16(o / den, 0.f);
   p.out[orow * kHeadDim + lane] = (uint16_t)(pk & 0xffffu);
   if (p.lse && lane == 0) p.lse[orow] = M + __log2f(den) * kLn2;
 }
@@ -520,20 +580,73 @@ __global__ __launch_bounds__(128) void kv_write_kernel(const uint16_t *__restric
 // ---------------------------------------------------------------------------------------
 // Host-side launchers (called from the C ABI after validation).
 // ---------------------------------------------------------------------------------------
+// Workgroups of kernel `fn` the whole device holds at once (cached per instantiation),
+// from the kernel's own register and LDS footprint: a gfx950 SIMD has 512 VGPRs per lane
+// (allocated in eights, at most 8 waves), a CU has 4 SIMDs and 160 KB of LDS.
+template <typename F>
+static int device_fill(F fn, int block) {
+  hipFuncAttributes attr;
+  hipDeviceProp_t prop;
+  int dev = 0;
+  if (hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(fn)) != hipSuccess ||
+      hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess)
+    return 512;
+  const int regs = max(8, (attr.numRegs + 7) / 8 * 8);
+  const int waves_per_simd = max(1, min(8, 512 / regs));
+  const int waves_per_wg = block / 64;
+  int per_cu = max(1, 4 * waves_per_simd / waves_per_wg);
+  if (attr.sharedSizeBytes > 0)
+    per_cu = min(per_cu, max(1, (int)(prop.maxSharedMemoryPerMultiProcessor / attr.sharedSizeBytes)));
+  if (getenv("EID_DEBUG"))
+    fprintf(stderr, "[eid] kernel regs=%d lds=%zu block=%d -> %d workgroups/CU x %d CUs\n",
+            attr.numRegs, attr.sharedSizeBytes, block, per_cu, prop.multiProcessorCount);
+  return per_cu * max(1, prop.multiProcessorCount);
+}
+
+template <int NT, bool FP8, int WAVES>
+static int fill_of() {
+  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES>, WAVES * 64);
+  return fill;
+}
+
 template <int NT, bool FP8>
-static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
-  const int Hkv = p.num_kv_heads;
-  const int waves = Hkv >= 8 ? 8 : Hkv;
-  dim3 grid(p.num_seqs * p.nparts_max, Hkv / waves);
+static int fill_t(int waves) {
   switch (waves) {
-    case 8: splitkv_kernel<NT, FP8, 8><<<grid, 512, 0, st>>>(p); break;
-    case 4: splitkv_kernel<NT, FP8, 4><<<grid, 256, 0, st>>>(p); break;
-    case 2: splitkv_kernel<NT, FP8, 2><<<grid, 128, 0, st>>>(p); break;
-    default: splitkv_kernel<NT, FP8, 1><<<grid, 64, 0, st>>>(p); break;
+    case 8: return fill_of<NT, FP8, 8>();
+    case 4: return fill_of<NT, FP8, 4>();
+    case 2: return fill_of<NT, FP8, 2>();
+    default: return fill_of<NT, FP8, 1>();
   }
+}
+
+static int waves_for(int Hkv) { return Hkv >= 8 ? 8 : Hkv; }
+
+// Workgroups of the split-KV instantiation (ntiles, fp8, Hkv) the device holds at once.
+int splitkv_fill(int ntiles, bool fp8, int Hkv) {
+  const int waves = waves_for(Hkv);
+  if (fp8) return ntiles == 1 ? fill_t<1, true>(waves) : fill_t<3, true>(waves);
+  return ntiles == 1 ? fill_t<1, false>(waves) : fill_t<3, false>(waves);
+}
+
+template <int NT, bool FP8, int WAVES>
+static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
+  dim3 grid(p.num_seqs * p.nparts_max, p.num_kv_heads / WAVES);
+  splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
   return hipGetLastError();
 }
 
+template <int NT, bool FP8>
+static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
+  switch (waves_for(p.num_kv_heads)) {
+    case 8: return launch_splitkv_w<NT, FP8, 8>(p, st);
+    case 4: return launch_splitkv_w<NT, FP8, 4>(p, st);
+    case 2: return launch_splitkv_w<NT, FP8, 2>(p, st);
+    default: return launch_splitkv_w<NT, FP8, 1>(p, st);
+  }
+}
+
+// p.target_items must hold splitkv_fill(ntiles, fp8, Hkv); the merge launch that follows is
+// given the same params so that it derives the same dynamic partition.
 hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
   if (fp8) {
     if (ntiles == 1) return launch_splitkv_t<1, true>(p, st);

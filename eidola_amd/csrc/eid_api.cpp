@@ -11,6 +11,7 @@
 
 namespace eid {
 hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
+int splitkv_fill(int ntiles, bool fp8, int Hkv);
 hipError_t launch_tile(const AttnParams &p, int max_q_len, bool fp8, hipStream_t st);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
 hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
@@ -84,6 +85,7 @@ int32_t check_attn_desc(const eid_attn_desc *d) {
 
 struct Plan {
   int32_t partition, nparts_max, ws_rows;
+  bool dynamic;
   size_t ml_bytes, acc_bytes;
 };
 
@@ -99,17 +101,11 @@ int32_t max_span(const eid_attn_desc *d) {
 Plan make_plan(const eid_attn_desc *d) {
   Plan pl;
   const int32_t span = max_span(d);
-  int32_t P = d->partition_size;
-  if (P == 0) {
-    // Aim at ~8 workgroups per CU if every sequence were max length.
-    const int64_t target_wgs = 2048;
-    int64_t want = ((int64_t)span * d->num_seqs + target_wgs - 1) / target_wgs;
-    want = (want + 63) / 64 * 64;
-    if (want < 128) want = 128;
-    if (want > 1024) want = 1024;
-    P = (int32_t)want;
-  }
+  // partition_size == 0: the kernels size the partition from the batch at run time, never
+  // below kDynPartitionMin, which therefore bounds the partition count for the workspace.
+  const int32_t P = d->partition_size ? d->partition_size : eid::kDynPartitionMin;
   pl.partition = P;
+  pl.dynamic = d->partition_size == 0;
   pl.nparts_max = (span + P - 1) / P;
   pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
@@ -160,6 +156,8 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.max_blocks_per_seq = d->max_blocks_per_seq;
   p.window = d->window;
   p.partition = pl.partition;
+  p.dynamic_partition = pl.dynamic ? 1 : 0;
+  p.target_items = 512;
   p.nparts_max = pl.nparts_max;
   p.ws_rows = pl.ws_rows;
   p.softmax_scale = d->softmax_scale;
@@ -225,6 +223,7 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   p.qlen_hi = 1;
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
   hipError_t e = eid::launch_splitkv(p, 1, fp8, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (pl.nparts_max > 1) {
@@ -243,28 +242,33 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   hipError_t e;
-  // q_len 1..2: one 16-row tile per KV head
+  // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
+  // of its own class of sequences (they share the partition plan)
   p.qlen_lo = 1;
   p.qlen_hi = 2;
+  p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
   e = eid::launch_splitkv(p, 1, fp8, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  if (pl.nparts_max > 1) {
+    e = eid::launch_merge(p, st);
+    if (e != hipSuccess) return hip_fail(e, "merge launch");
+  }
   if (desc->max_q_len > 2) {  // q_len 3..6: three tiles
     p.qlen_lo = 3;
     p.qlen_hi = eid::kShortQMax;
+    p.target_items = eid::splitkv_fill(3, fp8, desc->num_kv_heads);
     e = eid::launch_splitkv(p, 3, fp8, st);
     if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
+    if (pl.nparts_max > 1) {
+      e = eid::launch_merge(p, st);
+      if (e != hipSuccess) return hip_fail(e, "merge launch");
+    }
   }
   if (desc->max_q_len > eid::kShortQMax) {  // long chunks: MFMA tile kernel
     p.qlen_lo = eid::kShortQMax + 1;
     p.qlen_hi = 0x7fffffff;
     e = eid::launch_tile(p, desc->max_q_len, fp8, st);
     if (e != hipSuccess) return hip_fail(e, "tile launch");
-  }
-  if (pl.nparts_max > 1) {
-    p.qlen_lo = 1;
-    p.qlen_hi = eid::kShortQMax;
-    e = eid::launch_merge(p, st);
-    if (e != hipSuccess) return hip_fail(e, "merge launch");
   }
   return EID_OK;
 }
@@ -275,8 +279,11 @@ int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args, void
   if (int32_t rc = check_attn_args(desc, args, false, false)) return rc;
   const Plan pl = make_plan(desc);
   eid::AttnParams p = make_params(desc, args, pl);
-  p.qlen_lo = 1;
-  p.qlen_hi = eid::kShortQMax;
+  // One class of sequences per call, as the split-KV launches are: q_len <= 2, else 3..6.
+  const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  p.qlen_lo = desc->max_q_len <= 2 ? 1 : 3;
+  p.qlen_hi = desc->max_q_len <= 2 ? 2 : eid::kShortQMax;
+  p.target_items = eid::splitkv_fill(desc->max_q_len <= 2 ? 1 : 3, fp8, desc->num_kv_heads);
   hipError_t e = eid::launch_merge(p, static_cast<hipStream_t>(hip_stream));
   if (e != hipSuccess) return hip_fail(e, "merge launch");
   return EID_OK;

@@ -11,6 +11,8 @@ constexpr int kBlock = 16;        // tokens per KV page
 constexpr int kGroup = 8;         // query heads per KV head
 constexpr int kShortQMax = 6;     // q_len handled by the split-KV kernel (6*8 = 48 rows = 3 tiles)
 constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the split-KV loop
+constexpr int kDynPartitionMin = 256;   // lower bound (and workspace sizing) of the dynamic partition
+constexpr int kDynPartitionCap = 1024;  // a workgroup streams serially: keep its share bounded
 
 struct AttnParams {
   const uint16_t *q;
@@ -29,6 +31,8 @@ struct AttnParams {
   int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;
   int32_t window, partition, nparts_max, ws_rows;
   int32_t qlen_lo, qlen_hi;  // this launch serves sequences with qlen_lo <= q_len <= qlen_hi
+  int32_t dynamic_partition; // 1: kernels derive the partition from the batch (>= partition)
+  int32_t target_items;      // workgroups the device holds at once (dynamic partition only)
   float softmax_scale;
 };
 

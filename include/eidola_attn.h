@@ -74,8 +74,9 @@ typedef struct eid_attn_desc {
   float softmax_scale;        /* 1/sqrt(head_dim) normally                               */
   int32_t window;             /* 0 = full causal; W>0: row at position p sees p-W+1..p   */
   int32_t kv_dtype;           /* eid_kv_dtype                                            */
-  int32_t partition_size;     /* split-KV partition in tokens; 0 = library picks; else a
-                                 multiple of 64 in [64, 4096]                            */
+  int32_t partition_size;     /* split-KV partition in tokens: a multiple of 64 in
+                                 [64, 4096], or 0 = the kernels size it from the batch at
+                                 run time (>= 256) so the work fills the device evenly   */
 } eid_attn_desc;
 
 /* Device pointers, all caller-owned. */
@@ -130,6 +131,12 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
 /*
  * Stage K4 alone — merge the split-KV partials found in args->workspace (as laid out by
  * the split-KV kernel for this desc) into args->out / args->lse.  Exposed for tests.
+ * Serves one class of sequences per call, as the split-KV launches do: q_len <= 2 when
+ * desc->max_q_len <= 2, otherwise q_len 3..6.  Sequences with a single partition are left
+ * alone (the split-KV kernel writes their output itself).
+ * Workspace layout, with R = min(max_q_len, 6) and N = partitions per sequence (max):
+ *   float ml [num_seqs*R][Hq][N][2]   m (natural-log units, -inf if empty) and l
+ *   float acc[num_seqs*R][Hq][N][64]  sum of e^(s-m) * v, at the next 256-byte boundary
  */
 int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
                       void *hip_stream);
@@ -138,7 +145,8 @@ int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
  * Returns 0 for an invalid desc. */
 size_t eid_workspace_bytes(const eid_attn_desc *desc);
 
-/* The partition size (tokens) the library will use for desc (resolves the 0 default). */
+/* The partition size (tokens) the workspace is planned with: desc->partition_size, or the
+ * lower bound 256 of the run-time choice when that is 0. */
 int32_t eid_partition_size(const eid_attn_desc *desc);
 
 /* Thread-local description of the last error on this thread; "" if none. */
