@@ -316,44 +316,64 @@ __device__ __forceinline__ SeqView view_seq(const AttnParams &p, const int s) {
   return v;
 }
 
-// Partition size of this launch.  Fixed when the caller gave one.  Otherwise every wave
-// derives the same value from the batch itself: the smallest multiple of 64 (>= the
-// planning minimum that sized the workspace) for which the item list fits in a whole
-// number R of device fills, R being the fewest fills that keep a partition <= the cap:
-//   items <= total/P + active <= target_items * R.
-__device__ __forceinline__ int effective_partition(const AttnParams &p) {
-  if (!p.dynamic_partition) return p.partition;
-  const int lane = threadIdx.x & 63;
-  long long total = 0;
-  int active = 0;
-  for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
-    const SeqView v = view_seq(p, s0 + lane);
-    total += v.span;
-    active += v.span > 0;
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    total += __shfl_xor(total, off);
-    active += __shfl_xor(active, off);
-  }
-  const long long T = max(p.target_items, 1);
-  const long long R = max(1LL, (total / kDynPartitionCap + active + T - 1) / T);
-  const long long denom = max(1LL, T * R - active);
-  long long P = ((total + denom - 1) / denom + 63) / 64 * 64;
-  P = max(P, (long long)p.partition);
-  return (int)min(P, 1LL << 20);
-}
-
 __device__ __forceinline__ int num_partitions(const AttnParams &p, const int span, const int P) {
   return min((span + P - 1) / P, p.nparts_max);
 }
 
-__device__ __forceinline__ bool find_work_item(const AttnParams &p, const int P, const int w,
+__device__ __forceinline__ long long wave_sum(long long v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+  return v;
+}
+
+// Partition size of this launch.  Fixed when the caller gave one.  Otherwise every wave
+// derives the same value from the batch itself.  With T = workgroups the device holds at
+// once: if the whole batch fits one device fill with partitions no longer than the cap,
+// take the smallest multiple of 64 (>= the planning minimum that sized the workspace)
+// whose exact item count is <= T, so every workgroup is resident from the start and no
+// second, partly filled round follows; otherwise take the cap, which leaves several
+// fills of equal items.  `first` is the view of sequences 0..63 (one per lane), which the
+// caller has loaded already.
+__device__ __forceinline__ int effective_partition(const AttnParams &p, const SeqView &first) {
+  if (!p.dynamic_partition) return p.partition;
+  const int lane = threadIdx.x & 63;
+  long long total = first.span;
+  int active = first.span > 0;
+  for (int s0 = 64; s0 < p.num_seqs; s0 += 64) {
+    const SeqView v = view_seq(p, s0 + lane);
+    total += v.span;
+    active += v.span > 0;
+  }
+  total = wave_sum(total);
+  active = (int)wave_sum(active);
+  const long long T = max(p.target_items, 1);
+  if (active >= T) return kDynPartitionCap;
+  long long P = ((total + (T - active) - 1) / (T - active) + 63) / 64 * 64;  // items <= total/P + active <= T
+  P = max(P, (long long)p.partition);
+  if (P >= kDynPartitionCap) return kDynPartitionCap;
+  // The bound is pessimistic by up to one item per sequence: walk down while the exact
+  // count still fits.
+  for (int step = 0; step < 4 && P - 64 >= p.partition; ++step) {
+    const int Pc = (int)P - 64;
+    long long items = num_partitions(p, first.span, Pc);
+    for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
+      items += num_partitions(p, view_seq(p, s0 + lane).span, Pc);
+    items = wave_sum(items);
+    if (items > T) break;
+    P = Pc;
+  }
+  return (int)P;
+}
+
+// Finds item `w` of the compacted list and the partition size it was built with.
+__device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w, int &P,
                                                WorkItem &it) {
   const int lane = threadIdx.x & 63;
+  const SeqView first = view_seq(p, lane);
+  P = effective_partition(p, first);
   int base = 0;
   for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
-    const SeqView v = view_seq(p, s0 + lane);
+    const SeqView v = s0 == 0 ? first : view_seq(p, s0 + lane);
     const int n = num_partitions(p, v.span, P);
     const int incl = wave_inclusive_scan(n, lane);
     const int total = __builtin_amdgcn_readlane(incl, 63);
@@ -384,9 +404,9 @@ __global__ __launch_bounds__(WAVES * 64) void splitkv_kernel(const AttnParams p)
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.y * WAVES + wave;
-  const int P = effective_partition(p);
+  int P;
   WorkItem it;
-  if (!find_work_item(p, P, blockIdx.x, it)) return;
+  if (!find_work_item(p, blockIdx.x, P, it)) return;
   const int s = it.seq, part = it.part, nparts = it.nparts;
   const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
   const int kb = kv_begin(L, qlen, p.window);
@@ -471,7 +491,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
   const int L = p.seq_lens[s];
   if (L < qlen) return;
-  const int P = effective_partition(p);
+  const int P = effective_partition(p, view_seq(p, lane));
   const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
   if (nparts <= 1) return;
 
@@ -630,7 +650,16 @@ int splitkv_fill(int ntiles, bool fp8, int Hkv) {
 
 template <int NT, bool FP8, int WAVES>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
-  dim3 grid(p.num_seqs * p.nparts_max, p.num_kv_heads / WAVES);
+  // Items never exceed num_seqs * nparts_max; with the run-time partition they also never
+  // exceed max(one device fill, the count at the cap), which keeps idle workgroups few.
+  long long items = (long long)p.num_seqs * p.nparts_max;
+  if (p.dynamic_partition) {
+    const long long at_cap =
+        (long long)p.num_seqs * (((long long)p.nparts_max * p.partition + kDynPartitionCap - 1) /
+                                     kDynPartitionCap + 1);
+    items = min(items, max((long long)p.target_items, at_cap));
+  }
+  dim3 grid((unsigned)items, p.num_kv_heads / WAVES);
   splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
   return hipGetLastError();
 }

@@ -58,21 +58,13 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, b);
 }
 
-// fp32 values that are exactly representable in bf16 (fp8 widened): truncate and pack.
-__device__ __forceinline__ uint32_t pack_bf16_exact(float lo, float hi) {
-  return (__float_as_uint(hi) & 0xffff0000u) | (__float_as_uint(lo) >> 16);
-}
-
-// 8 fp8-e4m3fn bytes (two dwords) -> 8 bf16 (exact widening)
+// 8 fp8-e4m3fn bytes (two dwords) -> 8 bf16, exact widening, two elements per instruction
+// (v_cvt_scalef32_pk_bf16_fp8 with a unit scale; op_sel picks the low or high byte pair).
 __device__ __forceinline__ void fp8x8_to_bf16x8(uint32_t d0, uint32_t d1, uint32_t out[4]) {
-  auto a = __builtin_amdgcn_cvt_pk_f32_fp8(d0, false);
-  auto b = __builtin_amdgcn_cvt_pk_f32_fp8(d0, true);
-  auto c = __builtin_amdgcn_cvt_pk_f32_fp8(d1, false);
-  auto d = __builtin_amdgcn_cvt_pk_f32_fp8(d1, true);
-  out[0] = pack_bf16_exact(a[0], a[1]);
-  out[1] = pack_bf16_exact(b[0], b[1]);
-  out[2] = pack_bf16_exact(c[0], c[1]);
-  out[3] = pack_bf16_exact(d[0], d[1]);
+  out[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d0, 1.0f, false));
+  out[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d0, 1.0f, true));
+  out[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d1, 1.0f, false));
+  out[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d1, 1.0f, true));
 }
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }

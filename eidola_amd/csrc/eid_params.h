@@ -12,7 +12,7 @@ constexpr int kGroup = 8;         // query heads per KV head
 constexpr int kShortQMax = 6;     // q_len handled by the split-KV kernel (6*8 = 48 rows = 3 tiles)
 constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the split-KV loop
 constexpr int kDynPartitionMin = 256;   // lower bound (and workspace sizing) of the dynamic partition
-constexpr int kDynPartitionCap = 1024;  // a workgroup streams serially: keep its share bounded
+constexpr int kDynPartitionCap = 2048;  // a workgroup streams serially: keep its share bounded
 
 struct AttnParams {
   const uint16_t *q;
