@@ -39,7 +39,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
                                        const int t_begin, const int t_end, const int seq_len,
                                        const int pos_first, const int lo_last,
                                        const Frag8 (&qf)[NT][2], const RowInfo (&ri)[NT],
-                                       uint8_t *wave_lds, float (&m)[NT], float (&lsum)[NT],
+                                       uint8_t *wave_lds, float (&m)[NT], f32x4 (&lacc)[NT],
                                        f32x4 (&acc)[NT][4]) {
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
@@ -51,31 +51,39 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
                             (uint32_t)g * (16 * kElt);
   const int32_t *bt = p.block_table + (size_t)s * p.max_blocks_per_seq;
   const int nblk_total = (t_end + kBlock - 1) / kBlock;
+  // scores enter the softmax as exp2(S * c2 - m): scale, log2(e) and the fp8 K scale in one
+  // factor (> 0: softmax_scale is validated, quantisation scales are magnitudes)
   const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
+  Frag8 ones;  // bf16 1.0 in every slot: a row of ones in place of V^T yields row sums of P
+  ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
 
   uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
   const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
 
   // Page ids travel through scalar registers: the table row and the index are wave-uniform,
   // so these are scalar loads that never share a wait counter with the K/V vector loads.
-  // The ids of chunk i+1 are fetched while chunk i is in flight.
-  int blk[4];
+  // The ids of iteration i+1 are fetched while iteration i is in flight.
+  // One iteration = 64 tokens: 16 KiB (bf16) or 8 KiB (fp8) per wave in flight.
+  constexpr int kSub = 1;                // 64-token chunks per iteration
+  constexpr int kPages = 4 * kSub;       // pages per iteration
+  constexpr int kIter = kChunk * kSub;   // tokens per iteration
+  int blk[kPages];
 #pragma unroll
-  for (int b = 0; b < 4; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
+  for (int b = 0; b < kPages; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
 
-  for (int tc = t_begin; tc < t_end; tc += kChunk) {
-    const int nb = min(4, (t_end - tc + kBlock - 1) / kBlock);
+  for (int ti = t_begin; ti < t_end; ti += kIter) {
+    const int nbi = min(kPages, (t_end - ti + kBlock - 1) / kBlock);
 
     // ---- global loads: each lane takes 32 B (bf16) / 16 B (fp8) of one token row ----
-    u32x4 kraw[4][kElt], vraw[4][kElt];
+    u32x4 kraw[kPages][kElt], vraw[kPages][kElt];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
+    for (int b = 0; b < kPages; ++b) {
 #pragma unroll
       for (int e = 0; e < kElt; ++e) {
         kraw[b][e] = u32x4{0, 0, 0, 0};
         vraw[b][e] = u32x4{0, 0, 0, 0};
       }
-      if (b < nb) {
+      if (b < nbi) {
         const uint8_t *kp = p.k_cache + (size_t)blk[b] * page_bytes + lane_off;
         const uint8_t *vp = p.v_cache + (size_t)blk[b] * page_bytes + lane_off;
 #pragma unroll
@@ -85,10 +93,15 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         }
       }
     }
-    if (tc + kChunk < t_end) {
+    if (ti + kIter < t_end) {
 #pragma unroll
-      for (int b = 0; b < 4; ++b) blk[b] = bt[min((tc + kChunk) / kBlock + b, nblk_total - 1)];
+      for (int b = 0; b < kPages; ++b) blk[b] = bt[min((ti + kIter) / kBlock + b, nblk_total - 1)];
     }
+
+#pragma unroll
+    for (int sub = 0; sub < kSub; ++sub) {
+    const int tc = ti + sub * kChunk;
+    if (tc >= t_end) break;
 
     // ---- V: zero rows past the sequence end, widen fp8, stage in LDS ----
     const bool tail = tc + kChunk > seq_len;
@@ -97,17 +110,20 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
       u32x4 v0, v1;
       if constexpr (FP8) {
         uint32_t lo4[4], hi4[4];
-        fp8x8_to_bf16x8(vraw[b][0][0], vraw[b][0][1], lo4);
-        fp8x8_to_bf16x8(vraw[b][0][2], vraw[b][0][3], hi4);
+        fp8x8_to_bf16x8(vraw[4 * sub + b][0][0], vraw[4 * sub + b][0][1], lo4);
+        fp8x8_to_bf16x8(vraw[4 * sub + b][0][2], vraw[4 * sub + b][0][3], hi4);
         v0 = u32x4{lo4[0], lo4[1], lo4[2], lo4[3]};
         v1 = u32x4{hi4[0], hi4[1], hi4[2], hi4[3]};
       } else {
-        v0 = vraw[b][0];
-        v1 = vraw[b][kElt - 1];
+        v0 = vraw[4 * sub + b][0];
+        v1 = vraw[4 * sub + b][kElt - 1];
       }
-      if (tail && tc + b * kBlock + i16 >= seq_len) {
-        v0 = u32x4{0, 0, 0, 0};
-        v1 = u32x4{0, 0, 0, 0};
+      if (tail) {  // last chunk of the sequence only (kept a real branch, not 8 selects)
+        asm volatile("" ::: "memory");
+        if (tc + b * kBlock + i16 >= seq_len) {
+          v0 = u32x4{0, 0, 0, 0};
+          v1 = u32x4{0, 0, 0, 0};
+        }
       }
       *(u32x4 *)(lds_wr + b * kVPageBytes) = v0;
       *(u32x4 *)(lds_wr + b * kVPageBytes + 16) = v1;
@@ -118,27 +134,24 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       if constexpr (FP8) {
-        fp8x8_to_bf16x8(kraw[b][0][0], kraw[b][0][1], kf[b][0].w);
-        fp8x8_to_bf16x8(kraw[b][0][2], kraw[b][0][3], kf[b][1].w);
+        fp8x8_to_bf16x8(kraw[4 * sub + b][0][0], kraw[4 * sub + b][0][1], kf[b][0].w);
+        fp8x8_to_bf16x8(kraw[4 * sub + b][0][2], kraw[4 * sub + b][0][3], kf[b][1].w);
       } else {
-        kf[b][0].u = kraw[b][0];
-        kf[b][1].u = kraw[b][kElt - 1];
+        kf[b][0].u = kraw[4 * sub + b][0];
+        kf[b][1].u = kraw[4 * sub + b][kElt - 1];
       }
     }
-
     const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
 
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-      // S^T = K Q^T, then scale into the base-2 domain
+      // S^T = K Q^T (raw scores, fp32)
       f32x4 S[4];
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         f32x4 z = {0.f, 0.f, 0.f, 0.f};
         z = mfma16x32(kf[b][0], qf[nt][0], z);
         S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
-#pragma unroll
-        for (int r = 0; r < 4; ++r) S[b][r] *= c2;
       }
       if (need_mask) {
 #pragma unroll
@@ -155,24 +168,19 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
 #pragma unroll
         for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, S[b][r]);
       mloc = rowgroup_max(mloc);
-      const float m_new = fmaxf(m[nt], mloc);
+      const float m_new = fmaxf(m[nt], mloc * c2);
       const float alpha = fast_exp2(m[nt] - m_new);
       m[nt] = m_new;
-      float psum = 0.f;
 #pragma unroll
       for (int b = 0; b < 4; ++b)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          S[b][r] = fast_exp2(S[b][r] - m_new);
-          psum += S[b][r];
-        }
-      lsum[nt] = lsum[nt] * alpha + psum;
-      if (__any(alpha != 1.0f)) {
+        for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_new));
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+      for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
-      }
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
       // P^T as B operands: pair 0 = pages 0,1; pair 1 = pages 2,3
       Frag8 pf[2];
 #pragma unroll
@@ -182,6 +190,9 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         pf[pr].w[2] = pack_bf16(S[2 * pr + 1][0], S[2 * pr + 1][1]);
         pf[pr].w[3] = pack_bf16(S[2 * pr + 1][2], S[2 * pr + 1][3]);
       }
+      // row sums of the bf16-rounded P (the same values the numerator uses), on the MFMA pipe
+      lacc[nt] = mfma16x32(ones, pf[0], lacc[nt]);
+      lacc[nt] = mfma16x32(ones, pf[1], lacc[nt]);
       // O^T += V^T P^T
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt)
@@ -197,6 +208,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
           acc[nt][mt] = mfma16x32(vf, pf[pr], acc[nt][mt]);
         }
     }
+    }  // sub
   }
 }
 
@@ -206,14 +218,14 @@ template <int NT, bool FP8>
 __device__ __forceinline__ void finish(const AttnParams &p, const int s, const int kvh,
                                        const int row0, const int qlen, const int tq0,
                                        const bool direct, const int part, float (&m)[NT],
-                                       float (&lsum)[NT], f32x4 (&acc)[NT][4]) {
+                                       f32x4 (&lacc)[NT], f32x4 (&acc)[NT][4]) {
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
   const int Hq = p.num_q_heads;
   const float vs = FP8 ? p.v_scale[kvh] : 1.0f;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const float l = rowgroup_sum(lsum[nt]);
+    const float l = lacc[nt][0];  // every lane of the row holds the full sum
     const int r = nt * 16 + i16;
     const int t = tq0 + (r >> 3);
     const int head = kvh * kGroup + (r & 7);
@@ -345,8 +357,12 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
     active += v.span > 0;
   }
   total = wave_sum(total);
-  active = (int)wave_sum(active);
+  total = ((long long)__builtin_amdgcn_readfirstlane((int)(total >> 32)) << 32) |
+          (unsigned)__builtin_amdgcn_readfirstlane((int)total);
+  active = __builtin_amdgcn_readfirstlane((int)wave_sum(active));
   const long long T = max(p.target_items, 1);
+  // (every value below is the same in all lanes; readfirstlane tells the compiler so, which
+  // keeps the partition and everything derived from it in scalar registers)
   if (active >= T) return kDynPartitionCap;
   long long P = ((total + (T - active) - 1) / (T - active) + 63) / 64 * 64;  // items <= total/P + active <= T
   P = max(P, (long long)p.partition);
@@ -359,10 +375,10 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
     for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
       items += num_partitions(p, view_seq(p, s0 + lane).span, Pc);
     items = wave_sum(items);
-    if (items > T) break;
+    if (__builtin_amdgcn_readfirstlane((int)(items > T))) break;
     P = Pc;
   }
-  return (int)P;
+  return __builtin_amdgcn_readfirstlane((int)P);
 }
 
 // Finds item `w` of the compacted list and the partition size it was built with.
@@ -400,7 +416,7 @@ __device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w,
 // heads) of its partition.
 // ---------------------------------------------------------------------------------------
 template <int NT, bool FP8, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void splitkv_kernel(const AttnParams p) {
+__global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(const AttnParams p) {
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.y * WAVES + wave;
@@ -418,18 +434,18 @@ __global__ __launch_bounds__(WAVES * 64) void splitkv_kernel(const AttnParams p)
   Frag8 qf[NT][2];
   RowInfo ri[NT];
   load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
-  float m[NT], lsum[NT];
-  f32x4 acc[NT][4];
+  float m[NT];
+  f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     m[nt] = kNegBig;
-    lsum[nt] = 0.f;
+    lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
-                  lsum, acc);
-  finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lsum, acc);
+                  lacc, acc);
+  finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lacc, acc);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -457,18 +473,18 @@ __global__ __launch_bounds__(WAVES * 64) void tile_kernel(const AttnParams p) {
   Frag8 qf[NT][2];
   RowInfo ri[NT];
   load_q<NT>(p, row0, qlen, tq0, kvh, pos0, qf, ri);
-  float m[NT], lsum[NT];
-  f32x4 acc[NT][4];
+  float m[NT];
+  f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     m[nt] = kNegBig;
-    lsum[nt] = 0.f;
+    lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   attend<NT, FP8>(p, s, kvh, lo_first & ~(kBlock - 1), pos_last + 1, L, pos_first, lo_last, qf,
-                  ri, lds + wave * kWaveLdsBytes, m, lsum, acc);
-  finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lsum, acc);
+                  ri, lds + wave * kWaveLdsBytes, m, lacc, acc);
+  finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc);
 }
 
 // ---------------------------------------------------------------------------------------
