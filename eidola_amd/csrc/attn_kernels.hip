@@ -1,6 +1,6 @@
 // Paged sink-attention kernels for gfx950 (MI355X): one wavefront-level engine shared by
 //   * the bandwidth-bound split-KV kernel (decode and short-q verify rows), and
-//   * the tile kernel for long query chunks (chunked prefill),
+//   * the prefill kernel for long query chunks (K/V tiles shared through LDS),
 // plus the cross-partition log-sum-exp merge.
 //
 // Engine, per wavefront, per chunk of 64 context tokens (four 16-token pages):
@@ -32,6 +32,89 @@ struct RowInfo {
   int lo;   // first key the row may see
 };
 
+// Scores, online softmax and PV for one 64-token chunk whose K operands are in registers
+// and whose V tile sits in LDS (four 16-token pages of kVRowBytes-padded rows; `v_rd` is
+// the lane's transpose-read base).  The V^T operands are fetched once and reused by all NT
+// row tiles.
+template <int NT>
+__device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
+                                           const Frag8 (&qf)[NT][2], const RowInfo (&ri)[NT],
+                                           const int tc, const bool need_mask, const float c2,
+                                           float (&m)[NT], f32x4 (&lacc)[NT],
+                                           f32x4 (&acc)[NT][4]) {
+  const int g = (threadIdx.x & 63) >> 4;
+  Frag8 ones;  // bf16 1.0 in every slot: a row of ones in place of V^T yields row sums of P
+  ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+  Frag8 vf[4][2];  // [dim tile][page pair]
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      const u32x2 a = lds_read_tr16(v_rd + (2 * pr) * kVPageBytes + 32 * mt);
+      const u32x2 b2 = lds_read_tr16(v_rd + (2 * pr + 1) * kVPageBytes + 32 * mt);
+      vf[mt][pr].w[0] = a[0];
+      vf[mt][pr].w[1] = a[1];
+      vf[mt][pr].w[2] = b2[0];
+      vf[mt][pr].w[3] = b2[1];
+    }
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    // S^T = K Q^T (raw scores, fp32)
+    f32x4 S[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      z = mfma16x32(kf[b][0], qf[nt][0], z);
+      S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int j = tc + b * kBlock + 4 * g + r;
+          if (j < ri[nt].lo || j > ri[nt].pos) S[b][r] = -INFINITY;
+        }
+    }
+    float mloc = S[0][0];
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, S[b][r]);
+    mloc = rowgroup_max(mloc);
+    const float m_new = fmaxf(m[nt], mloc * c2);
+    const float alpha = fast_exp2(m[nt] - m_new);
+    m[nt] = m_new;
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_new));
+#pragma unroll
+    for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+    // P^T as B operands: pair 0 = pages 0,1; pair 1 = pages 2,3
+    Frag8 pf[2];
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      pf[pr].w[0] = pack_bf16(S[2 * pr][0], S[2 * pr][1]);
+      pf[pr].w[1] = pack_bf16(S[2 * pr][2], S[2 * pr][3]);
+      pf[pr].w[2] = pack_bf16(S[2 * pr + 1][0], S[2 * pr + 1][1]);
+      pf[pr].w[3] = pack_bf16(S[2 * pr + 1][2], S[2 * pr + 1][3]);
+    }
+    // row sums of the bf16-rounded P (the same values the numerator uses), on the MFMA pipe
+    lacc[nt] = mfma16x32(ones, pf[0], lacc[nt]);
+    lacc[nt] = mfma16x32(ones, pf[1], lacc[nt]);
+    // O^T += V^T P^T
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) acc[nt][mt] = mfma16x32(vf[mt][pr], pf[pr], acc[nt][mt]);
+  }
+}
+
 // One wavefront attends rows [16*NT) over keys [t_begin, t_end) of sequence `s`.
 // t_begin is a multiple of 16.  Tokens >= seq_len are never used (K masked, V zeroed).
 template <int NT, bool FP8>
@@ -54,8 +137,6 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   // scores enter the softmax as exp2(S * c2 - m): scale, log2(e) and the fp8 K scale in one
   // factor (> 0: softmax_scale is validated, quantisation scales are magnitudes)
   const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
-  Frag8 ones;  // bf16 1.0 in every slot: a row of ones in place of V^T yields row sums of P
-  ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
 
   uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
   const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
@@ -63,10 +144,8 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   // Page ids travel through scalar registers: the table row and the index are wave-uniform,
   // so these are scalar loads that never share a wait counter with the K/V vector loads.
   // The ids of iteration i+1 are fetched while iteration i is in flight.
-  // One iteration = 64 tokens: 16 KiB (bf16) or 8 KiB (fp8) per wave in flight.
-  constexpr int kSub = 1;                // 64-token chunks per iteration
-  constexpr int kPages = 4 * kSub;       // pages per iteration
-  constexpr int kIter = kChunk * kSub;   // tokens per iteration
+  constexpr int kPages = 4;
+  constexpr int kIter = kChunk;
   int blk[kPages];
 #pragma unroll
   for (int b = 0; b < kPages; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
@@ -98,10 +177,9 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
       for (int b = 0; b < kPages; ++b) blk[b] = bt[min((ti + kIter) / kBlock + b, nblk_total - 1)];
     }
 
-#pragma unroll
-    for (int sub = 0; sub < kSub; ++sub) {
-    const int tc = ti + sub * kChunk;
-    if (tc >= t_end) break;
+    {
+    const int tc = ti;
+    constexpr int sub = 0;
 
     // ---- V: zero rows past the sequence end, widen fp8, stage in LDS ----
     const bool tail = tc + kChunk > seq_len;
@@ -142,72 +220,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
       }
     }
     const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
-
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      // S^T = K Q^T (raw scores, fp32)
-      f32x4 S[4];
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        z = mfma16x32(kf[b][0], qf[nt][0], z);
-        S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
-      }
-      if (need_mask) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int j = tc + b * kBlock + 4 * g + r;
-            if (j < ri[nt].lo || j > ri[nt].pos) S[b][r] = -INFINITY;
-          }
-      }
-      float mloc = S[0][0];
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, S[b][r]);
-      mloc = rowgroup_max(mloc);
-      const float m_new = fmaxf(m[nt], mloc * c2);
-      const float alpha = fast_exp2(m[nt] - m_new);
-      m[nt] = m_new;
-#pragma unroll
-      for (int b = 0; b < 4; ++b)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_new));
-#pragma unroll
-      for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
-      // P^T as B operands: pair 0 = pages 0,1; pair 1 = pages 2,3
-      Frag8 pf[2];
-#pragma unroll
-      for (int pr = 0; pr < 2; ++pr) {
-        pf[pr].w[0] = pack_bf16(S[2 * pr][0], S[2 * pr][1]);
-        pf[pr].w[1] = pack_bf16(S[2 * pr][2], S[2 * pr][3]);
-        pf[pr].w[2] = pack_bf16(S[2 * pr + 1][0], S[2 * pr + 1][1]);
-        pf[pr].w[3] = pack_bf16(S[2 * pr + 1][2], S[2 * pr + 1][3]);
-      }
-      // row sums of the bf16-rounded P (the same values the numerator uses), on the MFMA pipe
-      lacc[nt] = mfma16x32(ones, pf[0], lacc[nt]);
-      lacc[nt] = mfma16x32(ones, pf[1], lacc[nt]);
-      // O^T += V^T P^T
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int pr = 0; pr < 2; ++pr) {
-          const u32x2 a = lds_read_tr16(lds_rd + (2 * pr) * kVPageBytes + 32 * mt);
-          const u32x2 b2 = lds_read_tr16(lds_rd + (2 * pr + 1) * kVPageBytes + 32 * mt);
-          Frag8 vf;
-          vf.w[0] = a[0];
-          vf.w[1] = a[1];
-          vf.w[2] = b2[0];
-          vf.w[3] = b2[1];
-          acc[nt][mt] = mfma16x32(vf, pf[pr], acc[nt][mt]);
-        }
-    }
+    chunk_step<NT>(kf, lds_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
     }  // sub
   }
 }
@@ -449,30 +462,88 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// Tile kernel for long query chunks.  grid = (ceil(max_q_len / (WAVES*2*NT)), Hkv, num_seqs);
-// each wave owns 2*NT consecutive query tokens x 8 heads and walks its whole causal range.
+// Prefill kernel for long query chunks (q_len > 6): the MFMA-bound path.
+//
+// A workgroup of 4 waves owns 32 consecutive query tokens of one sequence for one KV head:
+// 256 (token, head) rows, 64 per wave (four 16-row tiles).  It walks the keys its rows can
+// see in 64-token chunks; each chunk's K and V (one KV head: 8 KiB each) are fetched from
+// the paged cache ONCE per workgroup into a double-buffered LDS tile (rows padded to 144 B,
+// fp8 widened on the way in) while the previous chunk is being consumed, and every wave
+// reads its K operands (ds_read_b128) and V^T operands (ds_read_b64_tr_b16) from there.
+//
+// grid.x = Hkv * items with the KV head as the fastest index: workgroup ids are dealt
+// round-robin to the 8 XCDs, so with 8 KV heads every XCD serves a single KV head and the
+// K/V stream of a sequence is fetched into that XCD's L2 once for all its query tiles.
+// Items = 32-token tiles of the sequences of this class, compacted by a prefix scan and
+// visited heaviest (latest tile) first within a sequence.
 // ---------------------------------------------------------------------------------------
-template <int NT, bool FP8, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void tile_kernel(const AttnParams p) {
-  __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int s = blockIdx.z, kvh = blockIdx.y;
-  const int row0 = p.cu_seqlens_q[s];
-  const int qlen = p.cu_seqlens_q[s + 1] - row0;
-  if (qlen < p.qlen_lo || qlen > p.qlen_hi) return;
-  const int tq0 = (blockIdx.x * WAVES + wave) * (2 * NT);
-  if (tq0 >= qlen) return;
-  const int L = p.seq_lens[s];
-  if (L < qlen) return;
+constexpr int kPfWaves = 4;
+constexpr int kPfWaveTok = 8;                     // query tokens per wave (x 8 heads = 64 rows)
+constexpr int kPfTok = kPfWaves * kPfWaveTok;     // query tokens per workgroup
+constexpr int kPfTileBytes = kChunk * kVRowBytes; // one 64-token K or V tile of one KV head
+
+__device__ __forceinline__ bool find_prefill_item(const AttnParams &p, const int w, int &seq,
+                                                  int &tile, int &row0, int &qlen, int &seq_len) {
+  const int lane = threadIdx.x & 63;
+  int base = 0;
+  for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
+    const int s = s0 + lane;
+    int n = 0, r0 = 0, ql = 0, L = 0;
+    if (s < p.num_seqs) {
+      L = p.seq_lens[s];
+      r0 = p.cu_seqlens_q[s];
+      ql = p.cu_seqlens_q[s + 1] - r0;
+      if (ql >= p.qlen_lo && ql <= p.qlen_hi && L >= ql) n = (ql + kPfTok - 1) / kPfTok;
+    }
+    const int incl = wave_inclusive_scan(n, lane);
+    const int total = __builtin_amdgcn_readlane(incl, 63);
+    if (w < base + total) {
+      const unsigned long long hit = __ballot(base + incl > w);
+      const int idx = __builtin_ctzll(hit);
+      const int nt = __builtin_amdgcn_readlane(n, idx);
+      seq = s0 + idx;
+      tile = nt - 1 - (w - (base + __builtin_amdgcn_readlane(incl, idx) - nt));
+      row0 = __builtin_amdgcn_readlane(r0, idx);
+      qlen = __builtin_amdgcn_readlane(ql, idx);
+      seq_len = __builtin_amdgcn_readlane(L, idx);
+      return true;
+    }
+    base += total;
+  }
+  return false;
+}
+
+template <bool FP8>
+__global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnParams p) {
+  constexpr int NT = 4;
+  constexpr int kElt = FP8 ? 1 : 2;
+  __shared__ __align__(16) uint8_t lds[2][2][kPfTileBytes];  // [buffer][K, V]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i16 = lane & 15, g = lane >> 4;
+  const int Hkv = p.num_kv_heads;
+  const int kvh = blockIdx.x % Hkv;
+  int s, tile, row0, qlen, L;
+  if (!find_prefill_item(p, blockIdx.x / Hkv, s, tile, row0, qlen, L)) return;
+
+  const int W = p.window;
   const int pos0 = L - qlen;
-  const int tq_last = min(tq0 + 2 * NT, qlen) - 1;
-  const int pos_first = pos0 + tq0, pos_last = pos0 + tq_last;
-  const int lo_first = p.window > 0 ? max(0, pos_first - p.window + 1) : 0;
-  const int lo_last = p.window > 0 ? max(0, pos_last - p.window + 1) : 0;
+  const int tq_wg = tile * kPfTok;
+  const int pos_first_wg = pos0 + tq_wg;
+  const int pos_last_wg = pos0 + min(tq_wg + kPfTok, qlen) - 1;
+  const int t_begin = (W > 0 ? max(0, pos_first_wg - W + 1) : 0) & ~(kBlock - 1);
+  const int t_end = pos_last_wg + 1;
+  // this wave's rows
+  const int tq0 = tq_wg + wave * kPfWaveTok;
+  const bool wave_active = tq0 < qlen;
+  const int pos_first = pos0 + tq0;
+  const int pos_last = pos0 + min(tq0 + kPfWaveTok, qlen) - 1;
+  const int lo_first = W > 0 ? max(0, pos_first - W + 1) : 0;
+  const int lo_last = W > 0 ? max(0, pos_last - W + 1) : 0;
 
   Frag8 qf[NT][2];
   RowInfo ri[NT];
-  load_q<NT>(p, row0, qlen, tq0, kvh, pos0, qf, ri);
+  load_q<NT>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri);
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
@@ -482,9 +553,91 @@ __global__ __launch_bounds__(WAVES * 64) void tile_kernel(const AttnParams p) {
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  attend<NT, FP8>(p, s, kvh, lo_first & ~(kBlock - 1), pos_last + 1, L, pos_first, lo_last, qf,
-                  ri, lds + wave * kWaveLdsBytes, m, lacc, acc);
-  finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc);
+  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
+
+  // cooperative loader: thread -> (row of the 64-token chunk, 32-byte segment of the head row)
+  const int ld_row = tid >> 2, ld_seg = tid & 3;
+  const int ld_page = ld_row >> 4;
+  const uint32_t row_bytes = (uint32_t)Hkv * kHeadDim * kElt;
+  const size_t page_bytes = (size_t)kBlock * row_bytes;
+  const uint32_t gl_off = (uint32_t)(ld_row & 15) * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
+                          (uint32_t)ld_seg * (16 * kElt);
+  const uint32_t st_off = (uint32_t)ld_row * kVRowBytes + ld_seg * 32;
+  const int32_t *bt = p.block_table + (size_t)s * p.max_blocks_per_seq;
+  const int nblk_total = (t_end + kBlock - 1) / kBlock;
+
+  u32x4 kr[kElt], vr[kElt];
+  auto fetch = [&](const int tc) {  // global -> registers for chunk starting at token tc
+    int ids[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) ids[b] = bt[min(tc / kBlock + b, nblk_total - 1)];
+    const int blk = ld_page == 0 ? ids[0] : ld_page == 1 ? ids[1] : ld_page == 2 ? ids[2] : ids[3];
+#pragma unroll
+    for (int e = 0; e < kElt; ++e) {
+      kr[e] = u32x4{0, 0, 0, 0};
+      vr[e] = u32x4{0, 0, 0, 0};
+    }
+    if (tc + ld_page * kBlock < t_end) {
+      const uint8_t *kp = p.k_cache + (size_t)blk * page_bytes + gl_off;
+      const uint8_t *vp = p.v_cache + (size_t)blk * page_bytes + gl_off;
+#pragma unroll
+      for (int e = 0; e < kElt; ++e) {
+        kr[e] = ldg128(kp + 16 * e);
+        vr[e] = ldg128(vp + 16 * e);
+      }
+    }
+  };
+  auto stash = [&](const int tc, const int buf) {  // registers -> LDS tile (bf16)
+    u32x4 k0, k1, v0, v1;
+    if constexpr (FP8) {
+      uint32_t a4[4], b4[4];
+      fp8x8_to_bf16x8(kr[0][0], kr[0][1], a4);
+      fp8x8_to_bf16x8(kr[0][2], kr[0][3], b4);
+      k0 = u32x4{a4[0], a4[1], a4[2], a4[3]};
+      k1 = u32x4{b4[0], b4[1], b4[2], b4[3]};
+      fp8x8_to_bf16x8(vr[0][0], vr[0][1], a4);
+      fp8x8_to_bf16x8(vr[0][2], vr[0][3], b4);
+      v0 = u32x4{a4[0], a4[1], a4[2], a4[3]};
+      v1 = u32x4{b4[0], b4[1], b4[2], b4[3]};
+    } else {
+      k0 = kr[0];
+      k1 = kr[kElt - 1];
+      v0 = vr[0];
+      v1 = vr[kElt - 1];
+    }
+    if (tc + ld_row >= L) {  // rows past the sequence end may hold anything: V must be 0
+      v0 = u32x4{0, 0, 0, 0};
+      v1 = u32x4{0, 0, 0, 0};
+    }
+    *(u32x4 *)(&lds[buf][0][st_off]) = k0;
+    *(u32x4 *)(&lds[buf][0][st_off + 16]) = k1;
+    *(u32x4 *)(&lds[buf][1][st_off]) = v0;
+    *(u32x4 *)(&lds[buf][1][st_off + 16]) = v1;
+  };
+
+  fetch(t_begin);
+  stash(t_begin, 0);
+  __syncthreads();
+  int cur = 0;
+  for (int tc = t_begin; tc < t_end; tc += kChunk, cur ^= 1) {
+    const bool has_next = tc + kChunk < t_end;
+    if (has_next) fetch(tc + kChunk);
+    if (wave_active && tc <= pos_last && tc + kChunk > lo_first) {
+      const uint8_t *kt = &lds[cur][0][0] + i16 * kVRowBytes + g * 32;
+      const uint8_t *v_rd = &lds[cur][1][0] + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
+      Frag8 kf[4][2];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        kf[b][0].u = *(const u32x4 *)(kt + b * kVPageBytes);
+        kf[b][1].u = *(const u32x4 *)(kt + b * kVPageBytes + 16);
+      }
+      const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
+      chunk_step<NT>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
+    }
+    if (has_next) stash(tc + kChunk, cur ^ 1);
+    __syncthreads();
+  }
+  if (wave_active) finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -701,14 +854,14 @@ hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t
   return launch_splitkv_t<3, false>(p, st);
 }
 
-hipError_t launch_tile(const AttnParams &p, int max_q_len, bool fp8, hipStream_t st) {
-  constexpr int NT = 4, WAVES = 4;
-  const int tokens_per_wg = WAVES * 2 * NT;
-  dim3 grid((max_q_len + tokens_per_wg - 1) / tokens_per_wg, p.num_kv_heads, p.num_seqs);
+hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st) {
+  // upper bound on 32-token tiles: every sequence rounds up by at most one tile
+  const long long items = (long long)num_q_tokens / kPfTok + p.num_seqs;
+  dim3 grid((unsigned)(items * p.num_kv_heads));
   if (fp8)
-    tile_kernel<NT, true, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
+    prefill_kernel<true><<<grid, kPfWaves * 64, 0, st>>>(p);
   else
-    tile_kernel<NT, false, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
+    prefill_kernel<false><<<grid, kPfWaves * 64, 0, st>>>(p);
   return hipGetLastError();
 }
 

@@ -12,7 +12,7 @@
 namespace eid {
 hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
 int splitkv_fill(int ntiles, bool fp8, int Hkv);
-hipError_t launch_tile(const AttnParams &p, int max_q_len, bool fp8, hipStream_t st);
+hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
 hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
                            uint8_t *v_cache, const int64_t *slot_mapping, const float *k_scale,
@@ -264,11 +264,11 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
       if (e != hipSuccess) return hip_fail(e, "merge launch");
     }
   }
-  if (desc->max_q_len > eid::kShortQMax) {  // long chunks: MFMA tile kernel
+  if (desc->max_q_len > eid::kShortQMax) {  // long chunks: MFMA prefill kernel
     p.qlen_lo = eid::kShortQMax + 1;
     p.qlen_hi = 0x7fffffff;
-    e = eid::launch_tile(p, desc->max_q_len, fp8, st);
-    if (e != hipSuccess) return hip_fail(e, "tile launch");
+    e = eid::launch_prefill(p, desc->num_q_tokens, fp8, st);
+    if (e != hipSuccess) return hip_fail(e, "prefill launch");
   }
   return EID_OK;
 }
