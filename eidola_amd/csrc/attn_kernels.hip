@@ -20,11 +20,20 @@
 
 namespace eid {
 
+constexpr float kLazyLog2 = 8.0f;               // slack of the lazily updated softmax maximum
 constexpr int kVRowBytes = 144;                 // 128 B of bf16 + 16 B pad (bank spread)
 constexpr int kVPageBytes = kBlock * kVRowBytes;  // one 16-token page of V for one KV head
 constexpr int kWaveLdsBytes = 4 * kVPageBytes;  // 64 tokens
 
 __device__ __forceinline__ u32x4 ldg128(const uint8_t *p) { return *(const u32x4 *)p; }
+
+// Block tables are read-only for the lifetime of a launch.  Reading them through the
+// constant address space keeps wave-uniform page-id loads on the scalar unit whatever else
+// the kernel stores, so they never share a wait counter with the K/V vector loads.
+typedef const __attribute__((address_space(4))) int32_t *const_i32_ptr;
+__device__ __forceinline__ const_i32_ptr as_constant(const int32_t *p) {
+  return (const_i32_ptr)(uintptr_t)p;
+}
 
 // Row bookkeeping of one 16-row MFMA column tile.
 struct RowInfo {
@@ -76,25 +85,36 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
           if (j < ri[nt].lo || j > ri[nt].pos) S[b][r] = -INFINITY;
         }
     }
-    float mloc = S[0][0];
+    // row maximum: v_max3 tree over the lane's 16 scores, then across the four lane rows
+    float mloc = __builtin_fmaxf(__builtin_fmaxf(S[0][0], S[0][1]), S[0][2]);
+    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[0][3]), S[1][0]);
+    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[1][1]), S[1][2]);
+    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[1][3]), S[2][0]);
+    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[2][1]), S[2][2]);
+    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[2][3]), S[3][0]);
+    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[3][1]), S[3][2]);
+    mloc = __builtin_fmaxf(mloc, S[3][3]);
+    mloc = rowgroup_max(mloc) * c2;
+    // Lazy rescaling: the reference maximum m only moves when the running maximum has
+    // outgrown it by more than kLazyLog2 (in log2 units), so exp2(s - m) stays <= 2^kLazyLog2
+    // (exact in the end: numerator and denominator share m) and the accumulators are
+    // rescaled on few chunks only.
+    if (__any(mloc > m[nt] + kLazyLog2)) {
+      const float m_new = mloc > m[nt] + kLazyLog2 ? mloc : m[nt];
+      const float alpha = fast_exp2(m[nt] - m_new);
+      m[nt] = m_new;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+    }
+    const float m_ref = m[nt];
 #pragma unroll
     for (int b = 0; b < 4; ++b)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) mloc = fmaxf(mloc, S[b][r]);
-    mloc = rowgroup_max(mloc);
-    const float m_new = fmaxf(m[nt], mloc * c2);
-    const float alpha = fast_exp2(m[nt] - m_new);
-    m[nt] = m_new;
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_new));
-#pragma unroll
-    for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+      for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_ref));
     // P^T as B operands: pair 0 = pages 0,1; pair 1 = pages 2,3
     Frag8 pf[2];
 #pragma unroll
@@ -132,7 +152,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   const size_t page_bytes = (size_t)kBlock * row_bytes;
   const uint32_t lane_off = (uint32_t)i16 * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
                             (uint32_t)g * (16 * kElt);
-  const int32_t *bt = p.block_table + (size_t)s * p.max_blocks_per_seq;
+  const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
   const int nblk_total = (t_end + kBlock - 1) / kBlock;
   // scores enter the softmax as exp2(S * c2 - m): scale, log2(e) and the fp8 K scale in one
   // factor (> 0: softmax_scale is validated, quantisation scales are magnitudes)
@@ -563,7 +583,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const uint32_t gl_off = (uint32_t)(ld_row & 15) * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
                           (uint32_t)ld_seg * (16 * kElt);
   const uint32_t st_off = (uint32_t)ld_row * kVRowBytes + ld_seg * 32;
-  const int32_t *bt = p.block_table + (size_t)s * p.max_blocks_per_seq;
+  const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
   const int nblk_total = (t_end + kBlock - 1) / kBlock;
 
   u32x4 kr[kElt], vr[kElt];
