@@ -186,6 +186,9 @@ def main():
     ap.add_argument("--report", default=os.path.join(ROOT, "gpurun_out", "bench_all.jsonl"))
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--partition", type=int, default=0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run plain 1 GiB device copies (a kernel of known traffic, for "
+                         "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-shuffle", action="store_true",
                     help="experiment: physically contiguous pages instead of a shuffled pool")
     a = ap.parse_args()
@@ -226,6 +229,13 @@ def main():
                      "how": "HIP events: (eid_attn_decode call) minus (eid_lse_merge call)"},
     }
     extra = [r]
+    if a.calibrate_copy:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if a.all:
         w = None
         torch.cuda.empty_cache()

@@ -207,6 +207,69 @@ def test_varlen_at_qlen1_equals_decode_entry_point(G):
     assert np.array_equal(a, c)
 
 
+def test_many_sequences_cross_the_64_wide_scan(G):
+    """More than 64 sequences of mixed classes: the device-side work lists are built by
+    64-wide prefix scans that must chain across batches."""
+    rng = np.random.default_rng(3)
+    S = 150
+    q_lens = rng.choice([1, 1, 1, 2, 4, 5, 6, 9, 33, 70], size=S)
+    seq_lens = q_lens + rng.integers(0, 700, size=S)
+    for window in (0, 48):
+        b = make_batch(seq_lens, q_lens, window=window)
+        q, k, v, sinks = logical_tensors(b)
+        kc, vc = cpu_caches(b, k, v)
+        kc_d, vc_d = G.gpu_caches(b, k, v)
+        ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+        out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+        assert_close(out, ref, f"150 sequences w={window}")
+        assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+@pytest.mark.parametrize("hkv", [1, 4, 16])
+def test_other_kv_head_counts(G, hkv):
+    b = make_batch([300, 40, 1, 77], [1, 5, 1, 40], num_kv_heads=hkv, partition=128)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, f"Hkv={hkv}")
+
+
+def test_prefill_from_empty_context_and_exact_page_multiples(G):
+    """Chunks whose context is exactly the chunk (no prior), page- and tile-aligned or not."""
+    seq_lens = [32, 64, 96, 100, 512, 7]
+    b = make_batch(seq_lens, seq_lens)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "no-prior prefill")
+
+
+def test_partition_count_at_its_maximum(G):
+    """Smallest partition on a long sequence: 4096/64 = 64 partitions for one row."""
+    b = make_batch([4096, 4095, 65], [1, 1, 1], partition=64)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "64 partitions")
+
+
+def test_errors_surface_as_status_codes_on_the_gpu_box(G):
+    b = make_batch([100], [1])
+    q, k, v, sinks = logical_tensors(b)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    with pytest.raises(ea.EidError) as e:
+        ea.attn_decode(b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                       max_kv_len=100, workspace=torch.empty(256, dtype=torch.uint8, device=G.DEV))
+    assert e.value.name == "EID_ERR_WORKSPACE"
+    with pytest.raises(ea.EidError) as e:   # block table too narrow for max_kv_len
+        ea.attn_decode(b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                       max_kv_len=100000)
+    assert e.value.name == "EID_ERR_INVALID_ARG"
+
+
 # ---------------------------------------------------------------- fp8 KV
 @pytest.mark.parametrize("q_len", [1, 5, 48])
 def test_fp8_kv_attention(G, q_len):
