@@ -494,8 +494,9 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
 // grid.x = Hkv * items with the KV head as the fastest index: workgroup ids are dealt
 // round-robin to the 8 XCDs, so with 8 KV heads every XCD serves a single KV head and the
 // K/V stream of a sequence is fetched into that XCD's L2 once for all its query tiles.
-// Items = 32-token tiles of the sequences of this class, compacted by a prefix scan and
-// visited heaviest (latest tile) first within a sequence.
+// Items = 32-token tiles of the sequences of this class, compacted by a prefix scan; within
+// each batch of 64 sequences the longest come first, and within a sequence the latest
+// (heaviest) tile comes first, so the long-running workgroups start early.
 // ---------------------------------------------------------------------------------------
 constexpr int kPfWaves = 4;
 constexpr int kPfWaveTok = 8;                     // query tokens per wave (x 8 heads = 64 rows)
@@ -515,14 +516,26 @@ __device__ __forceinline__ bool find_prefill_item(const AttnParams &p, const int
       ql = p.cu_seqlens_q[s + 1] - r0;
       if (ql >= p.qlen_lo && ql <= p.qlen_hi && L >= ql) n = (ql + kPfTok - 1) / kPfTok;
     }
-    const int incl = wave_inclusive_scan(n, lane);
+    // Longest sequences first within the batch of 64 (their tiles walk the most keys):
+    // rank by key length, then let lane r speak for the sequence of rank r.
+    const int key = n > 0 ? L : -1;
+    int rank = 0;
+#pragma unroll
+    for (int j = 0; j < 64; ++j) {
+      const int kj = __builtin_amdgcn_readlane(key, j);
+      rank += (kj > key || (kj == key && j < lane)) ? 1 : 0;
+    }
+    const int n_sorted = __builtin_amdgcn_ds_permute(rank << 2, n);
+    const int lane_sorted = __builtin_amdgcn_ds_permute(rank << 2, lane);
+    const int incl = wave_inclusive_scan(n_sorted, lane);
     const int total = __builtin_amdgcn_readlane(incl, 63);
     if (w < base + total) {
       const unsigned long long hit = __ballot(base + incl > w);
-      const int idx = __builtin_ctzll(hit);
+      const int pos = __builtin_ctzll(hit);
+      const int idx = __builtin_amdgcn_readlane(lane_sorted, pos);
       const int nt = __builtin_amdgcn_readlane(n, idx);
       seq = s0 + idx;
-      tile = nt - 1 - (w - (base + __builtin_amdgcn_readlane(incl, idx) - nt));
+      tile = nt - 1 - (w - (base + __builtin_amdgcn_readlane(incl, pos) - nt));
       row0 = __builtin_amdgcn_readlane(r0, idx);
       qlen = __builtin_amdgcn_readlane(ql, idx);
       seq_len = __builtin_amdgcn_readlane(L, idx);
