@@ -19,6 +19,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+# HBM bytes per launch of the split-KV decode kernel on this exact seeded batch, from two
+# rocprofv3 --pmc passes over this script (FETCH_SIZE 242,823 KiB x 2.0, WRITE_SIZE 8,972 KiB
+# x 1.0; the factors are what the same counters read for a plain 1 GiB device copy run with
+# --calibrate-copy).  See profiles/splitkv_decode_config2.md.
+TRAFFIC_BYTES_PER_LAUNCH = int((242_823 * 2.0 + 8_972 * 1.0) * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "paged sink-attn decode HBM GB/s (% peak) + ragged-batch tokens/s, 1 GPU"
 
@@ -160,7 +165,7 @@ def cpu_baseline(w, torch, synth, threads):
     while True:
         out, _ = oracle.attn_bf16(*args, num_threads=threads)
         reps += 1
-        if time.time() - t0 > 8.0 or reps >= 20:
+        if time.time() - t0 > 10.0 or reps >= 1000:
             break
     dt = (time.time() - t0) / reps
     # cross-check while we are here: GPU result of set 0 against the CPU path
@@ -170,7 +175,7 @@ def cpu_baseline(w, torch, synth, threads):
     work = synth.algorithmic_work(b)
     return {"value": work["bytes"] / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": f"{reps} full passes of the same 64-sequence decode batch "
-                      f"({work['ctx_tokens']} context tokens), {dt:.2f} s each; "
+                      f"({work['ctx_tokens']} context tokens), {dt:.3f} s each, {reps*dt:.1f} s in all; "
                       "CPU restatement of this repo (no reference CPU path exists)",
             "tokens_per_s": work["q_tokens"] / dt,
             "gpu_vs_cpu_max_abs_diff": float(err.max())}
@@ -216,7 +221,8 @@ def main():
         "config": {"workload": "configs[1] decode continuous batch, full attention: 64 seqs, "
                                "ctx U[1,8192], Hq64/Hkv8/D64, block 16, 300k-block pool; "
                                "step = kv_write(64 tokens) + split-KV decode + LSE merge",
-                   "partition_size": ea.partition_size(w.attn[0].desc),
+                   "partition_size": a.partition if a.partition else "run-time (workspace planned for >= %d)"
+                   % ea.partition_size(w.attn[0].desc),
                    "page_sets_rotated": a.sets},
         "pct_hbm_peak": 100 * r["step_GBps"] / HBM_PEAK_GBS,
         "tokens_per_s": r["q_tokens_per_s"], "ctx_tokens_per_s": r["ctx_tokens_per_s"],
@@ -224,7 +230,8 @@ def main():
                          "merge": r["ms_merge"] * 1e3},
         "roofline": {"bound": "hbm", "kernel": "splitkv_kernel<1,bf16,8 waves>",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": TRAFFIC_BYTES_PER_LAUNCH if a.partition == 0 and not a.no_shuffle else None,
                      "alg_bytes_per_launch": r["alg_bytes"], "launch_us": split_ms * 1e3,
                      "how": "HIP events: (eid_attn_decode call) minus (eid_lse_merge call)"},
     }

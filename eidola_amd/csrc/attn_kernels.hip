@@ -376,8 +376,9 @@ __device__ __forceinline__ long long wave_sum(long long v) {
 // once: if the whole batch fits one device fill with partitions no longer than the cap,
 // take the smallest multiple of 64 (>= the planning minimum that sized the workspace)
 // whose exact item count is <= T, so every workgroup is resident from the start and no
-// second, partly filled round follows; otherwise take the cap, which leaves several
-// fills of equal items.  `first` is the view of sequences 0..63 (one per lane), which the
+// second, partly filled round follows; otherwise size the partition for about three fills
+// of equal items (two fills balance ragged batches badly, many small items pay the
+// per-item prologue too often), between a floor and the cap.  `first` is the view of sequences 0..63 (one per lane), which the
 // caller has loaded already.
 __device__ __forceinline__ int effective_partition(const AttnParams &p, const SeqView &first) {
   if (!p.dynamic_partition) return p.partition;
@@ -396,10 +397,13 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
   const long long T = max(p.target_items, 1);
   // (every value below is the same in all lanes; readfirstlane tells the compiler so, which
   // keeps the partition and everything derived from it in scalar registers)
-  if (active >= T) return kDynPartitionCap;
+  // more than one fill: aim at about three fills of equal items, within [floor, cap]
+  const int P3 = (int)min((long long)kDynPartitionCap,
+                          max((long long)kDynPartitionFloor, (total / (3 * T) + 63) / 64 * 64));
+  if (active >= T) return P3;
   long long P = ((total + (T - active) - 1) / (T - active) + 63) / 64 * 64;  // items <= total/P + active <= T
   P = max(P, (long long)p.partition);
-  if (P >= kDynPartitionCap) return kDynPartitionCap;
+  if (P >= kDynPartitionCap) return P3;
   // The bound is pessimistic by up to one item per sequence: walk down while the exact
   // count still fits.
   for (int step = 0; step < 4 && P - 64 >= p.partition; ++step) {
@@ -414,12 +418,18 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
   return __builtin_amdgcn_readfirstlane((int)P);
 }
 
+// Partition size of this launch: from the plan header when a plan kernel ran, else derived
+// here.  With a plan, `w` past the end of the item list is known at once.
+__device__ __forceinline__ bool planned_out(const AttnParams &p, const int w) {
+  return p.plan && w >= p.plan[1];
+}
+
 // Finds item `w` of the compacted list and the partition size it was built with.
 __device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w, int &P,
                                                WorkItem &it) {
   const int lane = threadIdx.x & 63;
   const SeqView first = view_seq(p, lane);
-  P = effective_partition(p, first);
+  P = p.plan ? p.plan[0] : effective_partition(p, first);
   int base = 0;
   for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
     const SeqView v = s0 == 0 ? first : view_seq(p, s0 + lane);
@@ -443,6 +453,27 @@ __device__ __forceinline__ bool find_work_item(const AttnParams &p, const int w,
 }
 
 // ---------------------------------------------------------------------------------------
+// Plan kernel (one wave).  The host sizes the split-KV grid from max_kv_len alone, so on
+// ragged batches most of that grid has nothing to do, and a workgroup that has to scan
+// seq_lens to find that out still costs a dispatch, a slot and ~2 us.  When the bound is
+// large the library runs this kernel first: it writes {partition, number of items} to the
+// head of the workspace, and every surplus workgroup then leaves after one scalar load.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *plan_out) {
+  const int lane = threadIdx.x & 63;
+  const SeqView first = view_seq(p, lane);
+  const int P = effective_partition(p, first);
+  long long items = num_partitions(p, first.span, P);
+  for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
+    items += num_partitions(p, view_seq(p, s0 + lane).span, P);
+  items = wave_sum(items);
+  if (lane == 0) {
+    plan_out[0] = P;
+    plan_out[1] = (int32_t)items;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Split-KV kernel.  grid = (num_seqs * nparts_max, Hkv / WAVES); workgroup blockIdx.x takes
 // work item blockIdx.x (see find_work_item) and wave w of it owns KV head
 // blockIdx.y*WAVES + w, so the workgroup as a whole streams whole 16-token pages (all KV
@@ -453,6 +484,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.y * WAVES + wave;
+  if (planned_out(p, blockIdx.x)) return;
   int P;
   WorkItem it;
   if (!find_work_item(p, blockIdx.x, P, it)) return;
@@ -693,7 +725,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
   const int L = p.seq_lens[s];
   if (L < qlen) return;
-  const int P = effective_partition(p, view_seq(p, lane));
+  const int P = p.plan ? p.plan[0] : effective_partition(p, view_seq(p, lane));
   const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
   if (nparts <= 1) return;
 
@@ -853,13 +885,13 @@ int splitkv_fill(int ntiles, bool fp8, int Hkv) {
 template <int NT, bool FP8, int WAVES>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
   // Items never exceed num_seqs * nparts_max; with the run-time partition they also never
-  // exceed max(one device fill, the count at the cap), which keeps idle workgroups few.
+  // exceed max(one device fill, the count at the multi-fill floor).
   long long items = (long long)p.num_seqs * p.nparts_max;
   if (p.dynamic_partition) {
-    const long long at_cap =
-        (long long)p.num_seqs * (((long long)p.nparts_max * p.partition + kDynPartitionCap - 1) /
-                                     kDynPartitionCap + 1);
-    items = min(items, max((long long)p.target_items, at_cap));
+    const long long at_floor =
+        (long long)p.num_seqs * (((long long)p.nparts_max * p.partition + kDynPartitionFloor - 1) /
+                                     kDynPartitionFloor + 1);
+    items = min(items, max((long long)p.target_items, at_floor));
   }
   dim3 grid((unsigned)items, p.num_kv_heads / WAVES);
   splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
@@ -876,9 +908,18 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
   }
 }
 
-// p.target_items must hold splitkv_fill(ntiles, fp8, Hkv); the merge launch that follows is
-// given the same params so that it derives the same dynamic partition.
-hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
+// p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
+// plan kernel was run for this launch; the merge launch that follows is given the same
+// params so that it uses the same partition.
+hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st) {
+  p.plan = nullptr;
+  if ((long long)p.num_seqs * p.nparts_max > 4LL * p.target_items) {
+    AttnParams q = p;
+    plan_kernel<<<1, 64, 0, st>>>(q, plan_slot);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    p.plan = plan_slot;
+  }
   if (fp8) {
     if (ntiles == 1) return launch_splitkv_t<1, true>(p, st);
     return launch_splitkv_t<3, true>(p, st);

@@ -10,7 +10,7 @@
 #include <cstring>
 
 namespace eid {
-hipError_t launch_splitkv(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
+hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st);
 int splitkv_fill(int ntiles, bool fp8, int Hkv);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
@@ -126,9 +126,10 @@ int32_t check_attn_args(const eid_attn_desc *d, const eid_attn_args *a, bool nee
   if (d->kv_dtype == EID_KV_FP8_E4M3 && need_q && (!a->k_scale || !a->v_scale))
     return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
   const Plan pl = make_plan(d);
-  if (!a->workspace || a->workspace_bytes < pl.ml_bytes + pl.acc_bytes)
+  if (!a->workspace || a->workspace_bytes < eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes)
     return fail(EID_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given",
-                pl.ml_bytes + pl.acc_bytes, a->workspace ? a->workspace_bytes : (size_t)0);
+                eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes,
+                a->workspace ? a->workspace_bytes : (size_t)0);
   if ((reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0)
     return fail(EID_ERR_WORKSPACE, "workspace must be 256-byte aligned");
   return EID_OK;
@@ -148,8 +149,10 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.sinks = a->sinks;
   p.k_scale = a->k_scale;
   p.v_scale = a->v_scale;
-  p.ws_ml = static_cast<float *>(a->workspace);
-  p.ws_acc = reinterpret_cast<float *>(static_cast<uint8_t *>(a->workspace) + pl.ml_bytes);
+  uint8_t *ws = static_cast<uint8_t *>(a->workspace);
+  p.plan = nullptr;
+  p.ws_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes);
+  p.ws_acc = reinterpret_cast<float *>(ws + eid::kPlanBytes + pl.ml_bytes);
   p.num_seqs = d->num_seqs;
   p.num_q_heads = d->num_q_heads;
   p.num_kv_heads = d->num_kv_heads;
@@ -184,7 +187,7 @@ int32_t eid_partition_size(const eid_attn_desc *desc) {
 size_t eid_workspace_bytes(const eid_attn_desc *desc) {
   if (check_attn_desc(desc)) return 0;
   const Plan pl = make_plan(desc);
-  return pl.ml_bytes + pl.acc_bytes;
+  return eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes;
 }
 
 int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v_new,
@@ -224,7 +227,8 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
-  hipError_t e = eid::launch_splitkv(p, 1, fp8, st);
+  int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
+  hipError_t e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (pl.nparts_max > 1) {
     e = eid::launch_merge(p, st);
@@ -247,7 +251,8 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   p.qlen_lo = 1;
   p.qlen_hi = 2;
   p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
-  e = eid::launch_splitkv(p, 1, fp8, st);
+  int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
+  e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (pl.nparts_max > 1) {
     e = eid::launch_merge(p, st);
@@ -257,7 +262,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     p.qlen_lo = 3;
     p.qlen_hi = eid::kShortQMax;
     p.target_items = eid::splitkv_fill(3, fp8, desc->num_kv_heads);
-    e = eid::launch_splitkv(p, 3, fp8, st);
+    e = eid::launch_splitkv(p, 3, fp8, plan_slots + 2, st);
     if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
     if (pl.nparts_max > 1) {
       e = eid::launch_merge(p, st);

@@ -13,6 +13,8 @@ constexpr int kShortQMax = 6;     // q_len handled by the split-KV kernel (6*8 =
 constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the split-KV loop
 constexpr int kDynPartitionMin = 256;   // lower bound (and workspace sizing) of the dynamic partition
 constexpr int kDynPartitionCap = 2048;  // a workgroup streams serially: keep its share bounded
+constexpr int kDynPartitionFloor = 512; // smallest partition when the batch needs several fills
+constexpr int kPlanBytes = 256;         // head of the workspace: two {partition, items} slots
 
 struct AttnParams {
   const uint16_t *q;
@@ -26,6 +28,7 @@ struct AttnParams {
   const float *sinks;    // may be null
   const float *k_scale;  // fp8 only
   const float *v_scale;  // fp8 only
+  const int32_t *plan;   // {partition, number of items} written by the plan kernel, or null
   float *ws_ml;          // [num_seqs*ws_rows][Hq][nparts_max][2]  (m natural-log units, l)
   float *ws_acc;         // [num_seqs*ws_rows][Hq][nparts_max][64] (sum e^(s-m) v, v_scale applied)
   int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;

@@ -265,10 +265,11 @@ def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_le
 
 
 def workspace_layout(desc):
-    """(partition, nparts_max, ws_rows, ml_bytes): the split-KV workspace holds
-    ml  float32 [num_seqs*ws_rows, Hq, nparts_max, 2]  (m in natural-log units, l), then at
-    byte offset ml_bytes
-    acc float32 [num_seqs*ws_rows, Hq, nparts_max, 64] (sum of e^(s-m) * v)."""
+    """(partition, nparts_max, ws_rows, ml_offset, acc_offset): after a 256-byte plan header
+    the split-KV workspace holds
+    ml  float32 [num_seqs*ws_rows, Hq, nparts_max, 2]  (m in natural-log units, l) and
+    acc float32 [num_seqs*ws_rows, Hq, nparts_max, 64] (sum of e^(s-m) * v) at the byte
+    offsets returned."""
     P = partition_size(desc)
     if desc.window > 0:
         span = min(desc.max_kv_len, desc.window + 6 + desc.block_size - 1)
@@ -278,4 +279,4 @@ def workspace_layout(desc):
     ws_rows = min(desc.max_q_len, 6)
     cells = desc.num_seqs * ws_rows * desc.num_q_heads * nparts
     ml_bytes = (cells * 8 + 255) // 256 * 256
-    return P, nparts, ws_rows, ml_bytes
+    return P, nparts, ws_rows, 256, 256 + ml_bytes

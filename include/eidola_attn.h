@@ -135,6 +135,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  * desc->max_q_len <= 2, otherwise q_len 3..6.  Sequences with a single partition are left
  * alone (the split-KV kernel writes their output itself).
  * Workspace layout, with R = min(max_q_len, 6) and N = partitions per sequence (max):
+ *   256 bytes                         launch plan (written by the library)
  *   float ml [num_seqs*R][Hq][N][2]   m (natural-log units, -inf if empty) and l
  *   float acc[num_seqs*R][Hq][N][64]  sum of e^(s-m) * v, at the next 256-byte boundary
  */

@@ -313,7 +313,7 @@ def test_lse_merge_entry_point_against_oracle_merge(G):
     q, k, v, sinks = logical_tensors(b)
     kc, vc = cpu_caches(b, k, v)
     d = desc_of(b)
-    P, nparts, ws_rows, ml_bytes = workspace_layout(d)
+    P, nparts, ws_rows, ml_off, acc_off = workspace_layout(d)
     assert P == 128 and ws_rows == 5
     ml, acc = oracle.splitkv_f64(d, P, nparts, q, kc, vc, b.block_table, b.seq_lens, b.cu_seqlens_q)
     ref, ref_lse = oracle.lse_merge_f64(ml, acc, sinks)
@@ -321,8 +321,8 @@ def test_lse_merge_entry_point_against_oracle_merge(G):
     assert np.allclose(ref, full, rtol=1e-10, atol=1e-13)
     # workspace rows are (sequence, row-in-sequence); here every sequence has ws_rows rows
     ws = np.zeros(ea.workspace_bytes(d), np.uint8)
-    ws[:ml.size * 4] = ml.astype(np.float32).reshape(-1).view(np.uint8)
-    ws[ml_bytes:ml_bytes + acc.size * 4] = acc.astype(np.float32).reshape(-1).view(np.uint8)
+    ws[ml_off:ml_off + ml.size * 4] = ml.astype(np.float32).reshape(-1).view(np.uint8)
+    ws[acc_off:acc_off + acc.size * 4] = acc.astype(np.float32).reshape(-1).view(np.uint8)
     ws_d = torch.from_numpy(ws).to(G.DEV)
     lse_d = torch.zeros((15, 64), dtype=torch.float32, device=G.DEV)
     out = ea.ops.lse_merge(b.geom, ws_d, G.dev(b.seq_lens), G.dev(b.cu_seqlens_q),
