@@ -286,13 +286,17 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
         ml.y = l;
         *(float2 *)(p.ws_ml + idx * 2) = ml;
       }
-      float *a = p.ws_acc + idx * kHeadDim + 4 * g;
+      // the partition's own normalised output, fp16: half the workspace traffic of fp32
+      // sums, and |o| <= max|v| whatever the softmax weights were
+      const float inv_l = l > 0.f ? vs / l : 0.f;
+      _Float16 *a = p.ws_acc + idx * kHeadDim + 4 * g;
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) {
-        f32x4 v = acc[nt][mt];
+        typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+        f16x4 h;
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) v[r4] *= vs;
-        *(f32x4 *)(a + 16 * mt) = v;
+        for (int r4 = 0; r4 < 4; ++r4) h[r4] = (_Float16)(acc[nt][mt][r4] * inv_l);
+        *(f16x4 *)(a + 16 * mt) = h;
       }
     }
   }
@@ -708,8 +712,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
 // ---------------------------------------------------------------------------------------
 // Cross-partition merge.  grid = (Hq / 4, num_seqs * ws_rows); one wave per (row, head),
 // lane = output dim.  The (m, l) pairs of up to 64 partitions are fetched one per lane, the
-// weights e^(m_c - M) are formed lane-parallel, and the accumulator rows are then streamed
-// with independent loads.  Sequences finished by the split-KV kernel itself (one
+// weights l_c e^(m_c - M) are formed lane-parallel, and the partitions' normalised outputs
+// (fp16) are then streamed with independent loads.  Sequences finished by the split-KV kernel itself (one
 // partition) and sequences outside [qlen_lo, qlen_hi] are skipped.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
@@ -752,19 +756,19 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
     }
     den += lw;
     const int n = min(64, nparts - c0);
-    const float *a = p.ws_acc + (base + c0) * kHeadDim + lane;
+    const _Float16 *a = p.ws_acc + (base + c0) * kHeadDim + lane;
     int c = 0;
     for (; c + 4 <= n; c += 4) {
-      const float a0 = a[(c + 0) * kHeadDim], a1 = a[(c + 1) * kHeadDim];
-      const float a2 = a[(c + 2) * kHeadDim], a3 = a[(c + 3) * kHeadDim];
-      o += a0 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 0));
-      o += a1 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 1));
-      o += a2 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 2));
-      o += a3 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c + 3));
+      const float a0 = (float)a[(c + 0) * kHeadDim], a1 = (float)a[(c + 1) * kHeadDim];
+      const float a2 = (float)a[(c + 2) * kHeadDim], a3 = (float)a[(c + 3) * kHeadDim];
+      o += a0 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 0));
+      o += a1 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 1));
+      o += a2 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 2));
+      o += a3 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 3));
     }
     for (; c < n; ++c)
-      o += a[c * kHeadDim] *
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, w), c));
+      o += (float)a[c * kHeadDim] *
+           __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c));
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) den += __shfl_xor(den, off);

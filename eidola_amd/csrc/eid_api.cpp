@@ -110,7 +110,7 @@ Plan make_plan(const eid_attn_desc *d) {
   pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
   pl.ml_bytes = (cells * 2 * sizeof(float) + 255) / 256 * 256;
-  pl.acc_bytes = cells * eid::kHeadDim * sizeof(float);
+  pl.acc_bytes = cells * eid::kHeadDim * sizeof(_Float16);
   return pl;
 }
 
@@ -152,7 +152,7 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   uint8_t *ws = static_cast<uint8_t *>(a->workspace);
   p.plan = nullptr;
   p.ws_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes);
-  p.ws_acc = reinterpret_cast<float *>(ws + eid::kPlanBytes + pl.ml_bytes);
+  p.ws_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes);
   p.num_seqs = d->num_seqs;
   p.num_q_heads = d->num_q_heads;
   p.num_kv_heads = d->num_kv_heads;

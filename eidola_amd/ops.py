@@ -268,8 +268,8 @@ def workspace_layout(desc):
     """(partition, nparts_max, ws_rows, ml_offset, acc_offset): after a 256-byte plan header
     the split-KV workspace holds
     ml  float32 [num_seqs*ws_rows, Hq, nparts_max, 2]  (m in natural-log units, l) and
-    acc float32 [num_seqs*ws_rows, Hq, nparts_max, 64] (sum of e^(s-m) * v) at the byte
-    offsets returned."""
+    o   float16 [num_seqs*ws_rows, Hq, nparts_max, 64] (partition output sum e^(s-m) v / l) at
+    the byte offsets returned."""
     P = partition_size(desc)
     if desc.window > 0:
         span = min(desc.max_kv_len, desc.window + 6 + desc.block_size - 1)

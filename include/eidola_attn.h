@@ -136,8 +136,10 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  * alone (the split-KV kernel writes their output itself).
  * Workspace layout, with R = min(max_q_len, 6) and N = partitions per sequence (max):
  *   256 bytes                         launch plan (written by the library)
- *   float ml [num_seqs*R][Hq][N][2]   m (natural-log units, -inf if empty) and l
- *   float acc[num_seqs*R][Hq][N][64]  sum of e^(s-m) * v, at the next 256-byte boundary
+ *   float ml [num_seqs*R][Hq][N][2]   m (natural-log units, -inf if empty) and
+ *                                     l = sum of e^(s-m) over the partition's keys
+ *   half  o  [num_seqs*R][Hq][N][64]  the partition's own output sum e^(s-m) v / l (fp16),
+ *                                     at the next 256-byte boundary
  */
 int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
                       void *hip_stream);

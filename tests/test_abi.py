@@ -43,11 +43,11 @@ def test_workspace_and_partition_planning():
     assert P % 64 == 0 and 64 <= P <= 4096
     nparts = (1000 + P - 1) // P
     cells = 4 * 1 * 64 * nparts
-    assert ea.workspace_bytes(d) == 256 + (cells * 8 + 255) // 256 * 256 + cells * 256
+    assert ea.workspace_bytes(d) == 256 + (cells * 8 + 255) // 256 * 256 + cells * 128
     d5 = ea.make_desc(ea.AttnGeometry(partition_size=512), num_seqs=128, num_q_tokens=640,
                       max_q_len=5, max_kv_len=65536, max_blocks_per_seq=4096, num_blocks=300000)
     assert ea.partition_size(d5) == 512
-    assert ea.workspace_bytes(d5) == 256 + 128 * 5 * 64 * 128 * (8 + 256)
+    assert ea.workspace_bytes(d5) == 256 + 128 * 5 * 64 * 128 * (8 + 128)
     dw = ea.make_desc(ea.AttnGeometry(window=128), num_seqs=64, num_q_tokens=64, max_q_len=1,
                       max_kv_len=8192, max_blocks_per_seq=512, num_blocks=300000)
     assert ea.workspace_bytes(dw) < ea.workspace_bytes(good_desc(num_seqs=64, num_q_tokens=64,

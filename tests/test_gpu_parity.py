@@ -322,7 +322,9 @@ def test_lse_merge_entry_point_against_oracle_merge(G):
     # workspace rows are (sequence, row-in-sequence); here every sequence has ws_rows rows
     ws = np.zeros(ea.workspace_bytes(d), np.uint8)
     ws[ml_off:ml_off + ml.size * 4] = ml.astype(np.float32).reshape(-1).view(np.uint8)
-    ws[acc_off:acc_off + acc.size * 4] = acc.astype(np.float32).reshape(-1).view(np.uint8)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        o_part = np.where(ml[..., 1:2] > 0, acc / ml[..., 1:2], 0.0).astype(np.float16)
+    ws[acc_off:acc_off + o_part.size * 2] = o_part.reshape(-1).view(np.uint8)
     ws_d = torch.from_numpy(ws).to(G.DEV)
     lse_d = torch.zeros((15, 64), dtype=torch.float32, device=G.DEV)
     out = ea.ops.lse_merge(b.geom, ws_d, G.dev(b.seq_lens), G.dev(b.cu_seqlens_q),
