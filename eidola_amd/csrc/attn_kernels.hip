@@ -492,6 +492,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   int P;
   WorkItem it;
   if (!find_work_item(p, blockIdx.x, P, it)) return;
+  // the merge launch that follows reads the partition from here instead of re-deriving it
+  if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
   const int s = it.seq, part = it.part, nparts = it.nparts;
   const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
   const int kb = kv_begin(L, qlen, p.window);
@@ -710,11 +712,13 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
 }
 
 // ---------------------------------------------------------------------------------------
-// Cross-partition merge.  grid = (Hq / 4, num_seqs * ws_rows); one wave per (row, head),
-// lane = output dim.  The (m, l) pairs of up to 64 partitions are fetched one per lane, the
-// weights l_c e^(m_c - M) are formed lane-parallel, and the partitions' normalised outputs
-// (fp16) are then streamed with independent loads.  Sequences finished by the split-KV kernel itself (one
-// partition) and sequences outside [qlen_lo, qlen_hi] are skipped.
+// Cross-partition merge.  grid = (Hq / 4, num_seqs * ws_rows); one wave per (row, head).
+// The (m, l) pairs of up to 64 partitions are fetched one per lane and the weights
+// l_c e^(m_c - M) formed lane-parallel.  The partitions' normalised outputs (fp16) are read
+// four partitions per load instruction: lane (g, q) = (lane / 16, lane % 16) takes dims
+// 4q..4q+3 of partitions g, g+4, g+8, ..., eight loads in flight, and the four lane groups
+// are summed at the end.  Sequences finished by the split-KV kernel itself (one partition)
+// and sequences outside [qlen_lo, qlen_hi] are skipped.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   const int lane = threadIdx.x & 63;
@@ -729,53 +733,74 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
   const int L = p.seq_lens[s];
   if (L < qlen) return;
-  const int P = p.plan ? p.plan[0] : effective_partition(p, view_seq(p, lane));
+  // recorded by the split-KV launch this merge follows; derived again when it stands alone
+  const int P = p.plan_slot ? p.plan_slot[0] : effective_partition(p, view_seq(p, lane));
   const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
   if (nparts <= 1) return;
 
+  const int g = lane >> 4, q = lane & 15;
   const size_t base = ((size_t)wsrow * p.num_q_heads + head) * p.nparts_max;
+  const _Float16 *acc_row = p.ws_acc + base * kHeadDim + q * 4;
   const float sink = p.sinks ? p.sinks[head] : -INFINITY;
+  // the first 64 partitions' (m, l), kept for both passes
+  float2 ml0 = make_float2(-INFINITY, 0.f);
+  if (lane < nparts) ml0 = *(const float2 *)(p.ws_ml + (base + lane) * 2);
   // pass 1: global maximum over non-empty partitions and the sink
   float M = sink;
-  for (int c = lane; c < nparts; c += 64) {
+  if (ml0.y > 0.f) M = fmaxf(M, ml0.x);
+  for (int c = 64 + lane; c < nparts; c += 64) {
     const float2 ml = *(const float2 *)(p.ws_ml + (base + c) * 2);
     if (ml.y > 0.f) M = fmaxf(M, ml.x);
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off));
-  // pass 2: weights per lane, accumulator rows with four loads in flight
-  float den = 0.f, o = 0.f;
+  // pass 2: weights per lane, then the weighted sum of the partitions' outputs
+  float den = 0.f;
+  float o[4] = {0.f, 0.f, 0.f, 0.f};
   for (int c0 = 0; c0 < nparts; c0 += 64) {
-    float w = 0.f, lw = 0.f;
-    if (c0 + lane < nparts) {
-      const float2 ml = *(const float2 *)(p.ws_ml + (base + c0 + lane) * 2);
-      if (ml.y > 0.f) {
-        w = fast_exp2((ml.x - M) * kLog2e);
-        lw = ml.y * w;
+    float2 ml = ml0;
+    if (c0 > 0) {
+      ml = make_float2(-INFINITY, 0.f);
+      if (c0 + lane < nparts) ml = *(const float2 *)(p.ws_ml + (base + c0 + lane) * 2);
+    }
+    const float lw = ml.y > 0.f ? ml.y * fast_exp2((ml.x - M) * kLog2e) : 0.f;
+    den += lw;
+#pragma unroll
+    for (int j0 = 0; j0 < 16; j0 += 8) {
+      if (c0 + 4 * j0 >= nparts) break;
+      uint2 v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int c = c0 + 4 * (j0 + j) + g;
+        v[j] = make_uint2(0u, 0u);  // never multiply an unwritten cell, it may hold a NaN
+        if (c < nparts) v[j] = *(const uint2 *)(acc_row + (size_t)c * kHeadDim);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float w = __shfl(lw, 4 * (j0 + j) + g);
+        typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+        const half2_t lo = __builtin_bit_cast(half2_t, v[j].x), hi = __builtin_bit_cast(half2_t, v[j].y);
+        o[0] += (float)lo[0] * w;
+        o[1] += (float)lo[1] * w;
+        o[2] += (float)hi[0] * w;
+        o[3] += (float)hi[1] * w;
       }
     }
-    den += lw;
-    const int n = min(64, nparts - c0);
-    const _Float16 *a = p.ws_acc + (base + c0) * kHeadDim + lane;
-    int c = 0;
-    for (; c + 4 <= n; c += 4) {
-      const float a0 = (float)a[(c + 0) * kHeadDim], a1 = (float)a[(c + 1) * kHeadDim];
-      const float a2 = (float)a[(c + 2) * kHeadDim], a3 = (float)a[(c + 3) * kHeadDim];
-      o += a0 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 0));
-      o += a1 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 1));
-      o += a2 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 2));
-      o += a3 * __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c + 3));
-    }
-    for (; c < n; ++c)
-      o += (float)a[c * kHeadDim] *
-           __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, lw), c));
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) den += __shfl_xor(den, off);
   den += fast_exp2((sink - M) * kLog2e);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    o[e] += __shfl_xor(o[e], 16);
+    o[e] += __shfl_xor(o[e], 32);
+  }
   const size_t orow = (size_t)(row0 + t) * p.num_q_heads + head;
-  const uint32_t pk = pack_bf16(o / den, 0.f);
-  p.out[orow * kHeadDim + lane] = (uint16_t)(pk & 0xffffu);
+  if (g == 0) {
+    const float inv = 1.f / den;
+    *(uint2 *)(p.out + orow * kHeadDim + q * 4) =
+        make_uint2(pack_bf16(o[0] * inv, o[1] * inv), pack_bf16(o[2] * inv, o[3] * inv));
+  }
   if (p.lse && lane == 0) p.lse[orow] = M + __log2f(den) * kLn2;
 }
 
@@ -917,6 +942,7 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
 // params so that it uses the same partition.
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st) {
   p.plan = nullptr;
+  p.plan_slot = plan_slot;
   if ((long long)p.num_seqs * p.nparts_max > 4LL * p.target_items) {
     AttnParams q = p;
     plan_kernel<<<1, 64, 0, st>>>(q, plan_slot);

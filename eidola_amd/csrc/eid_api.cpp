@@ -151,6 +151,7 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.v_scale = a->v_scale;
   uint8_t *ws = static_cast<uint8_t *>(a->workspace);
   p.plan = nullptr;
+  p.plan_slot = nullptr;
   p.ws_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes);
   p.ws_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes);
   p.num_seqs = d->num_seqs;

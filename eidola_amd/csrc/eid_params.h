@@ -29,6 +29,7 @@ struct AttnParams {
   const float *k_scale;  // fp8 only
   const float *v_scale;  // fp8 only
   const int32_t *plan;   // {partition, number of items} written by the plan kernel, or null
+  int32_t *plan_slot;    // where this launch's split-KV kernel records its partition for the merge
   float *ws_ml;          // [num_seqs*ws_rows][Hq][nparts_max][2]  (m natural-log units, l)
   _Float16 *ws_acc;      // [num_seqs*ws_rows][Hq][nparts_max][64] partition output, normalised
   int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;
