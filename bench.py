@@ -46,6 +46,9 @@ def event_ms(fn, iters, torch):
     return e0.elapsed_time(e1) / iters
 
 
+NO_HINT = False  # --no-hint: do not pass the host-side sum of seq_lens to the library
+
+
 class Workload:
     """One configuration materialised on the GPU with `nsets` disjoint page sets."""
 
@@ -84,8 +87,11 @@ class Workload:
         ws = None
         self.attn, self.merge = [], []
         for bt in self.tables:
+            # the scheduler's host-side copy of seq_lens gives the sum for free; the library
+            # sizes the split-KV launch with it
             kw = dict(max_q_len=b0.max_q_len, max_kv_len=b0.max_kv_len, sinks=self.sinks,
-                      k_scale=self.k_scale, v_scale=self.v_scale, workspace=ws)
+                      k_scale=self.k_scale, v_scale=self.v_scale, workspace=ws,
+                      sum_kv_len=0 if NO_HINT else int(b0.seq_lens.sum()))
             cu = self.cu if kind == "varlen" else None
             c = ea.prepare(fn, g, self.q, self.k_cache, self.v_cache, bt, self.seq_lens, cu, **kw)
             ws = c._keep[-1]
@@ -196,7 +202,11 @@ def main():
                          "scaling rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     ap.add_argument("--no-shuffle", action="store_true",
                     help="experiment: physically contiguous pages instead of a shuffled pool")
+    ap.add_argument("--no-hint", action="store_true",
+                    help="experiment: leave desc.sum_kv_len at 0 (grid sized from max_kv_len)")
     a = ap.parse_args()
+    global NO_HINT
+    NO_HINT = a.no_hint
     if a.gpus != 1:
         sys.exit("bench.py: this path runs on ONE MI355X (no sharding, no collectives); "
                  "--gpus must be 1")
@@ -223,6 +233,7 @@ def main():
                                "step = kv_write(64 tokens) + split-KV decode + LSE merge",
                    "partition_size": a.partition if a.partition else "run-time (workspace planned for >= %d)"
                    % ea.partition_size(w.attn[0].desc),
+                   "sum_kv_len_hint": not a.no_hint,
                    "page_sets_rotated": a.sets},
         "pct_hbm_peak": 100 * r["step_GBps"] / HBM_PEAK_GBS,
         "tokens_per_s": r["q_tokens_per_s"], "ctx_tokens_per_s": r["ctx_tokens_per_s"],

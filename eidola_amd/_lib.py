@@ -50,6 +50,7 @@ class AttnDesc(C.Structure):
         ("window", C.c_int32),
         ("kv_dtype", C.c_int32),
         ("partition_size", C.c_int32),
+        ("sum_kv_len", C.c_int64),
     ]
 
 

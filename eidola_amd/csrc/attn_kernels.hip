@@ -262,8 +262,9 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
     const int r = nt * 16 + i16;
     const int t = tq0 + (r >> 3);
     const int head = kvh * kGroup + (r & 7);
-    if (t >= qlen) continue;
+    const bool valid = t < qlen;
     if (direct) {
+      if (!valid) continue;
       const float sink2 = p.sinks ? p.sinks[head] * kLog2e : -INFINITY;
       const float M = fmaxf(m[nt], sink2);
       const float w = fast_exp2(m[nt] - M);
@@ -279,8 +280,10 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
       }
       if (p.lse && g == 0) p.lse[(size_t)(row0 + t) * Hq + head] = (M + __log2f(den)) * kLn2;
     } else {
-      const size_t idx = ((size_t)(s * p.ws_rows + t) * Hq + head) * p.nparts_max + part;
-      if (g == 0) {
+      // Partials are laid out [row][partition][head]: the 8 heads of this wave are
+      // neighbours, and the 64 heads of the workgroup form one contiguous 8 KiB block.
+      const size_t idx = ((size_t)(s * p.ws_rows + t) * p.nparts_max + part) * Hq + head;
+      if (valid && g == 0) {
         float2 ml;
         ml.x = l > 0.f ? m[nt] * kLn2 : -INFINITY;
         ml.y = l;
@@ -289,14 +292,32 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
       // the partition's own normalised output, fp16: half the workspace traffic of fp32
       // sums, and |o| <= max|v| whatever the softmax weights were
       const float inv_l = l > 0.f ? vs / l : 0.f;
-      _Float16 *a = p.ws_acc + idx * kHeadDim + 4 * g;
+      uint32_t w[4][2];
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) {
-        typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
-        f16x4 h;
+        typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+        const f16x2 h0 = {(_Float16)(acc[nt][mt][0] * inv_l), (_Float16)(acc[nt][mt][1] * inv_l)};
+        const f16x2 h1 = {(_Float16)(acc[nt][mt][2] * inv_l), (_Float16)(acc[nt][mt][3] * inv_l)};
+        w[mt][0] = __builtin_bit_cast(uint32_t, h0);
+        w[mt][1] = __builtin_bit_cast(uint32_t, h1);
+      }
+      // A lane holds dims 16 mt + 4 g .. +3 of its row.  Swapping the odd 16-lane rows of
+      // tile mt with the even rows of tile mt + 1 leaves every lane with 8 consecutive dims
+      // (16 bytes): at (g & 1) * 16 + (g >> 1) * 8, from tiles {0, 1} and again from {2, 3}.
+      // Executed by all lanes; only the stores are predicated.
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) h[r4] = (_Float16)(acc[nt][mt][r4] * inv_l);
-        *(f16x4 *)(a + 16 * mt) = h;
+      for (int mt = 0; mt < 4; mt += 2) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const auto r = __builtin_amdgcn_permlane16_swap(w[mt][k], w[mt + 1][k], false, false);
+          w[mt][k] = r[0];
+          w[mt + 1][k] = r[1];
+        }
+      }
+      if (valid) {
+        _Float16 *a = p.ws_acc + idx * kHeadDim + (g & 1) * 16 + (g >> 1) * 8;
+        *(u32x4 *)a = u32x4{w[0][0], w[0][1], w[1][0], w[1][1]};
+        *(u32x4 *)(a + 32) = u32x4{w[2][0], w[2][1], w[3][0], w[3][1]};
       }
     }
   }
@@ -489,9 +510,34 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.y * WAVES + wave;
   if (planned_out(p, blockIdx.x)) return;
-  int P;
+  // One wave looks the work item up and hands it to the others through LDS: the lookup is
+  // several hundred instructions, and eight waves doing it side by side on every CU at the
+  // start of the launch would spend microseconds of issue slots before the first K/V load.
+  __shared__ int item_lds[8];
+  if (wave == 0) {
+    int P0 = 0;
+    WorkItem w{};
+    const bool found = find_work_item(p, blockIdx.x, P0, w);
+    if ((threadIdx.x & 63) == 0) {
+      item_lds[0] = found ? P0 : 0;
+      item_lds[1] = w.seq;
+      item_lds[2] = w.part;
+      item_lds[3] = w.nparts;
+      item_lds[4] = w.row0;
+      item_lds[5] = w.qlen;
+      item_lds[6] = w.seq_len;
+    }
+  }
+  __syncthreads();
+  const int P = __builtin_amdgcn_readfirstlane(item_lds[0]);
+  if (P == 0) return;  // past the end of the item list
   WorkItem it;
-  if (!find_work_item(p, blockIdx.x, P, it)) return;
+  it.seq = __builtin_amdgcn_readfirstlane(item_lds[1]);
+  it.part = __builtin_amdgcn_readfirstlane(item_lds[2]);
+  it.nparts = __builtin_amdgcn_readfirstlane(item_lds[3]);
+  it.row0 = __builtin_amdgcn_readfirstlane(item_lds[4]);
+  it.qlen = __builtin_amdgcn_readfirstlane(item_lds[5]);
+  it.seq_len = __builtin_amdgcn_readfirstlane(item_lds[6]);
   // the merge launch that follows reads the partition from here instead of re-deriving it
   if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
   const int s = it.seq, part = it.part, nparts = it.nparts;
@@ -594,8 +640,27 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int i16 = lane & 15, g = lane >> 4;
   const int Hkv = p.num_kv_heads;
   const int kvh = blockIdx.x % Hkv;
-  int s, tile, row0, qlen, L;
-  if (!find_prefill_item(p, blockIdx.x / Hkv, s, tile, row0, qlen, L)) return;
+  // one wave looks the item up, the others receive it through LDS
+  __shared__ int item_lds[8];
+  if (wave == 0) {
+    int s0 = 0, tile0 = 0, row00 = 0, qlen0 = 0, L0 = 0;
+    const bool found = find_prefill_item(p, blockIdx.x / Hkv, s0, tile0, row00, qlen0, L0);
+    if (lane == 0) {
+      item_lds[0] = found;
+      item_lds[1] = s0;
+      item_lds[2] = tile0;
+      item_lds[3] = row00;
+      item_lds[4] = qlen0;
+      item_lds[5] = L0;
+    }
+  }
+  __syncthreads();
+  if (!__builtin_amdgcn_readfirstlane(item_lds[0])) return;
+  const int s = __builtin_amdgcn_readfirstlane(item_lds[1]);
+  const int tile = __builtin_amdgcn_readfirstlane(item_lds[2]);
+  const int row0 = __builtin_amdgcn_readfirstlane(item_lds[3]);
+  const int qlen = __builtin_amdgcn_readfirstlane(item_lds[4]);
+  const int L = __builtin_amdgcn_readfirstlane(item_lds[5]);
 
   const int W = p.window;
   const int pos0 = L - qlen;
@@ -739,17 +804,19 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (nparts <= 1) return;
 
   const int g = lane >> 4, q = lane & 15;
-  const size_t base = ((size_t)wsrow * p.num_q_heads + head) * p.nparts_max;
+  // cell (row, partition c, head) sits at ((row * nparts_max + c) * Hq + head)
+  const size_t base = (size_t)wsrow * p.nparts_max * p.num_q_heads + head;
+  const size_t cstride = p.num_q_heads;
   const _Float16 *acc_row = p.ws_acc + base * kHeadDim + q * 4;
   const float sink = p.sinks ? p.sinks[head] : -INFINITY;
   // the first 64 partitions' (m, l), kept for both passes
   float2 ml0 = make_float2(-INFINITY, 0.f);
-  if (lane < nparts) ml0 = *(const float2 *)(p.ws_ml + (base + lane) * 2);
+  if (lane < nparts) ml0 = *(const float2 *)(p.ws_ml + (base + lane * cstride) * 2);
   // pass 1: global maximum over non-empty partitions and the sink
   float M = sink;
   if (ml0.y > 0.f) M = fmaxf(M, ml0.x);
   for (int c = 64 + lane; c < nparts; c += 64) {
-    const float2 ml = *(const float2 *)(p.ws_ml + (base + c) * 2);
+    const float2 ml = *(const float2 *)(p.ws_ml + (base + c * cstride) * 2);
     if (ml.y > 0.f) M = fmaxf(M, ml.x);
   }
 #pragma unroll
@@ -761,7 +828,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
     float2 ml = ml0;
     if (c0 > 0) {
       ml = make_float2(-INFINITY, 0.f);
-      if (c0 + lane < nparts) ml = *(const float2 *)(p.ws_ml + (base + c0 + lane) * 2);
+      if (c0 + lane < nparts) ml = *(const float2 *)(p.ws_ml + (base + (c0 + lane) * cstride) * 2);
     }
     const float lw = ml.y > 0.f ? ml.y * fast_exp2((ml.x - M) * kLog2e) : 0.f;
     den += lw;
@@ -773,7 +840,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
       for (int j = 0; j < 8; ++j) {
         const int c = c0 + 4 * (j0 + j) + g;
         v[j] = make_uint2(0u, 0u);  // never multiply an unwritten cell, it may hold a NaN
-        if (c < nparts) v[j] = *(const uint2 *)(acc_row + (size_t)c * kHeadDim);
+        if (c < nparts) v[j] = *(const uint2 *)(acc_row + (size_t)c * cstride * kHeadDim);
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -911,18 +978,33 @@ int splitkv_fill(int ntiles, bool fp8, int Hkv) {
   return ntiles == 1 ? fill_t<1, false>(waves) : fill_t<3, false>(waves);
 }
 
-template <int NT, bool FP8, int WAVES>
-static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
-  // Items never exceed num_seqs * nparts_max; with the run-time partition they also never
-  // exceed max(one device fill, the count at the multi-fill floor).
-  long long items = (long long)p.num_seqs * p.nparts_max;
+// Upper bound on the number of work items of a launch, from what the host knows.  Items
+// never exceed num_seqs * nparts_max.  With the run-time partition they are at most one
+// device fill T in the single-fill regime, and sum/P3 + num_seqs in the multi-fill regime,
+// where P3 = min(cap, max(floor, ~sum/(3T))) makes sum/P3 <= min(sum/floor, max(sum/cap, 3T));
+// without the caller's sum_kv_len the sum is bounded by num_seqs * max_kv_len.
+static long long item_bound(const AttnParams &p) {
+  const long long S = p.num_seqs, T = p.target_items;
+  long long items = S * p.nparts_max;
   if (p.dynamic_partition) {
     const long long at_floor =
-        (long long)p.num_seqs * (((long long)p.nparts_max * p.partition + kDynPartitionFloor - 1) /
-                                     kDynPartitionFloor + 1);
-    items = min(items, max((long long)p.target_items, at_floor));
+        S * (((long long)p.nparts_max * p.partition + kDynPartitionFloor - 1) / kDynPartitionFloor + 1);
+    items = min(items, max(T, at_floor));
+    if (p.sum_kv_len > 0) {
+      const long long sum = p.sum_kv_len;
+      const long long multi =
+          min(sum / kDynPartitionFloor, max(sum / kDynPartitionCap, 3 * T)) + S + 16;
+      items = min(items, max(T, multi));
+    }
+  } else if (p.sum_kv_len > 0) {
+    items = min(items, p.sum_kv_len / p.partition + S);
   }
-  dim3 grid((unsigned)items, p.num_kv_heads / WAVES);
+  return items;
+}
+
+template <int NT, bool FP8, int WAVES>
+static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
+  dim3 grid((unsigned)item_bound(p), p.num_kv_heads / WAVES);
   splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
   return hipGetLastError();
 }
@@ -943,7 +1025,7 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st) {
   p.plan = nullptr;
   p.plan_slot = plan_slot;
-  if ((long long)p.num_seqs * p.nparts_max > 4LL * p.target_items) {
+  if (item_bound(p) > 4LL * p.target_items) {
     AttnParams q = p;
     plan_kernel<<<1, 64, 0, st>>>(q, plan_slot);
     const hipError_t e = hipGetLastError();

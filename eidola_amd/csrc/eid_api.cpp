@@ -70,6 +70,9 @@ int32_t check_attn_desc(const eid_attn_desc *d) {
     return fail(EID_ERR_INVALID_ARG, "num_q_tokens %d < num_seqs %d", d->num_q_tokens,
                 d->num_seqs);
   if (d->max_kv_len <= 0) return fail(EID_ERR_INVALID_ARG, "max_kv_len must be positive");
+  if (d->sum_kv_len != 0 && d->sum_kv_len < d->max_kv_len)
+    return fail(EID_ERR_INVALID_ARG, "sum_kv_len %lld is below max_kv_len %d (0 = not known)",
+                (long long)d->sum_kv_len, d->max_kv_len);
   if ((int64_t)d->max_blocks_per_seq * d->block_size < d->max_kv_len)
     return fail(EID_ERR_INVALID_ARG, "max_blocks_per_seq %d cannot hold max_kv_len %d",
                 d->max_blocks_per_seq, d->max_kv_len);
@@ -154,6 +157,7 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.plan_slot = nullptr;
   p.ws_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes);
   p.ws_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes);
+  p.sum_kv_len = d->sum_kv_len;
   p.num_seqs = d->num_seqs;
   p.num_q_heads = d->num_q_heads;
   p.num_kv_heads = d->num_kv_heads;

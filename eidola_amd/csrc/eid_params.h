@@ -30,8 +30,9 @@ struct AttnParams {
   const float *v_scale;  // fp8 only
   const int32_t *plan;   // {partition, number of items} written by the plan kernel, or null
   int32_t *plan_slot;    // where this launch's split-KV kernel records its partition for the merge
-  float *ws_ml;          // [num_seqs*ws_rows][Hq][nparts_max][2]  (m natural-log units, l)
-  _Float16 *ws_acc;      // [num_seqs*ws_rows][Hq][nparts_max][64] partition output, normalised
+  float *ws_ml;          // [num_seqs*ws_rows][nparts_max][Hq][2]  (m natural-log units, l)
+  _Float16 *ws_acc;      // [num_seqs*ws_rows][nparts_max][Hq][64] partition output, normalised
+  long long sum_kv_len;  // host's upper bound on the sum of seq_lens, 0 = unknown
   int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;
   int32_t window, partition, nparts_max, ws_rows;
   int32_t qlen_lo, qlen_hi;  // this launch serves sequences with qlen_lo <= q_len <= qlen_hi

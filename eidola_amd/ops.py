@@ -28,7 +28,7 @@ class AttnGeometry:
 
 
 def make_desc(geom, *, num_seqs, num_q_tokens, max_q_len, max_kv_len, max_blocks_per_seq,
-              num_blocks):
+              num_blocks, sum_kv_len=0):
     d = AttnDesc()
     d.struct_size = C.sizeof(AttnDesc)
     d.num_seqs = num_seqs
@@ -45,6 +45,7 @@ def make_desc(geom, *, num_seqs, num_q_tokens, max_q_len, max_kv_len, max_blocks
     d.window = geom.window
     d.kv_dtype = geom.kv_dtype
     d.partition_size = geom.partition_size
+    d.sum_kv_len = sum_kv_len  # host-side sum of seq_lens (or an upper bound), 0 = unknown
     return d
 
 
@@ -118,7 +119,7 @@ def kv_write(geom, k_new, v_new, k_cache, v_cache, slot_mapping, k_scale=None, v
 
 def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q,
                max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace,
-               return_lse):
+               return_lse, sum_kv_len=0):
     _require(q, "q", torch.bfloat16, 3)
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
@@ -141,7 +142,7 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
         _require(v_scale, "v_scale", torch.float32, 1)
     desc = make_desc(geom, num_seqs=S, num_q_tokens=T, max_q_len=max_q_len,
                      max_kv_len=max_kv_len, max_blocks_per_seq=block_table.shape[1],
-                     num_blocks=k_cache.shape[0])
+                     num_blocks=k_cache.shape[0], sum_kv_len=sum_kv_len)
     if out is None:
         out = torch.empty_like(q)
     else:
@@ -192,7 +193,7 @@ class PreparedCall:
 
 def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, *,
             max_q_len=1, max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
-            workspace=None):
+            workspace=None, sum_kv_len=0):
     """Build a PreparedCall for "eid_attn_decode" / "eid_attn_varlen" / "eid_lse_merge"."""
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
@@ -201,7 +202,8 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
     _require(seq_lens, "seq_lens", torch.int32, 1)
     desc = make_desc(geom, num_seqs=seq_lens.shape[0], num_q_tokens=q.shape[0],
                      max_q_len=max_q_len, max_kv_len=max_kv_len,
-                     max_blocks_per_seq=block_table.shape[1], num_blocks=k_cache.shape[0])
+                     max_blocks_per_seq=block_table.shape[1], num_blocks=k_cache.shape[0],
+                     sum_kv_len=sum_kv_len)
     need = load_library().eid_workspace_bytes(C.byref(desc))
     if need == 0:
         check(getattr(load_library(), fn_name)(C.byref(desc), C.byref(AttnArgs()), None))
@@ -227,19 +229,21 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
 
 def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, sinks=None,
                 k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
-                return_lse=False):
-    """Stages K2+K4: one query row per sequence (q is [num_seqs, Hq, D])."""
+                return_lse=False, sum_kv_len=0):
+    """Stages K2+K4: one query row per sequence (q is [num_seqs, Hq, D]).  `sum_kv_len` is the
+    optional host-side sum of seq_lens (any upper bound): it sizes the launch to the work."""
     return _attn_call("eid_attn_decode", geom, q, k_cache, v_cache, block_table, seq_lens, None,
-                      1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse)
+                      1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse,
+                      sum_kv_len)
 
 
 def attn_varlen(geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, *, max_q_len,
                 max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
-                workspace=None, return_lse=False):
+                workspace=None, return_lse=False, sum_kv_len=0):
     """Stages K2/K3+K4 on a ragged cu_seqlens batch (prefill chunks, verify rows, decodes)."""
     return _attn_call("eid_attn_varlen", geom, q, k_cache, v_cache, block_table, seq_lens,
                       cu_seqlens_q, max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse,
-                      workspace, return_lse)
+                      workspace, return_lse, sum_kv_len)
 
 
 def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_len, max_kv_len,
@@ -267,8 +271,8 @@ def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_le
 def workspace_layout(desc):
     """(partition, nparts_max, ws_rows, ml_offset, acc_offset): after a 256-byte plan header
     the split-KV workspace holds
-    ml  float32 [num_seqs*ws_rows, Hq, nparts_max, 2]  (m in natural-log units, l) and
-    o   float16 [num_seqs*ws_rows, Hq, nparts_max, 64] (partition output sum e^(s-m) v / l) at
+    ml  float32 [num_seqs*ws_rows, nparts_max, Hq, 2]  (m in natural-log units, l) and
+    o   float16 [num_seqs*ws_rows, nparts_max, Hq, 64] (partition output sum e^(s-m) v / l) at
     the byte offsets returned."""
     P = partition_size(desc)
     if desc.window > 0:

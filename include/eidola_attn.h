@@ -77,6 +77,12 @@ typedef struct eid_attn_desc {
   int32_t partition_size;     /* split-KV partition in tokens: a multiple of 64 in
                                  [64, 4096], or 0 = the kernels size it from the batch at
                                  run time (>= 256) so the work fills the device evenly   */
+  int64_t sum_kv_len;         /* optional launch-sizing hint: any value >= the sum of
+                                 seq_lens[s] over the batch, or 0 = not known.  An engine's
+                                 scheduler holds seq_lens on the host, so the sum is free;
+                                 with it the split-KV grid is sized to the work instead of
+                                 to num_seqs * max_kv_len.  A value below the true sum is a
+                                 caller error the library cannot detect (work is dropped). */
 } eid_attn_desc;
 
 /* Device pointers, all caller-owned. */
@@ -136,10 +142,12 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  * alone (the split-KV kernel writes their output itself).
  * Workspace layout, with R = min(max_q_len, 6) and N = partitions per sequence (max):
  *   256 bytes                         launch plan (written by the library)
- *   float ml [num_seqs*R][Hq][N][2]   m (natural-log units, -inf if empty) and
+ *   float ml [num_seqs*R][N][Hq][2]   m (natural-log units, -inf if empty) and
  *                                     l = sum of e^(s-m) over the partition's keys
- *   half  o  [num_seqs*R][Hq][N][64]  the partition's own output sum e^(s-m) v / l (fp16),
+ *   half  o  [num_seqs*R][N][Hq][64]  the partition's own output sum e^(s-m) v / l (fp16),
  *                                     at the next 256-byte boundary
+ * (heads innermost: the 64 heads of one (row, partition) cell form one contiguous block,
+ * which a split-KV workgroup writes with full-width stores)
  */
 int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
                       void *hip_stream);

@@ -49,13 +49,15 @@ def gpu_caches(batch, k, v, k_scale=None, v_scale=None):
 
 
 def run_attn(batch, q, kc_d, vc_d, sinks, k_scale=None, v_scale=None, *, decode=None,
-             return_lse=False, geom=None):
-    """Calls eid_attn_decode (all q_len == 1) or eid_attn_varlen through the C ABI."""
+             return_lse=False, geom=None, hint=False):
+    """Calls eid_attn_decode (all q_len == 1) or eid_attn_varlen through the C ABI; with
+    `hint` the host-side sum of seq_lens is passed as desc.sum_kv_len."""
     geom = geom or batch.geom
     if decode is None:
         decode = batch.max_q_len == 1
     kw = dict(max_kv_len=batch.max_kv_len, sinks=dev(sinks), k_scale=dev(k_scale),
-              v_scale=dev(v_scale), return_lse=return_lse)
+              v_scale=dev(v_scale), return_lse=return_lse,
+              sum_kv_len=int(batch.seq_lens.sum()) if hint else 0)
     bt, sl = dev(batch.block_table), dev(batch.seq_lens)
     if decode:
         r = ea.attn_decode(geom, bf16_dev(q), kc_d, vc_d, bt, sl, **kw)

@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
 
 
 def test_struct_layout_matches_header():
-    assert C.sizeof(AttnDesc) == 64
+    assert C.sizeof(AttnDesc) == 72
     assert AttnDesc.num_blocks.offset == 40 and AttnDesc.softmax_scale.offset == 48
     assert C.sizeof(AttnArgs) == 13 * 8
 
@@ -68,6 +68,7 @@ def test_workspace_and_partition_planning():
     ("softmax_scale", 0.0, "EID_ERR_INVALID_ARG"),
     ("softmax_scale", float("nan"), "EID_ERR_INVALID_ARG"),
     ("window", -1, "EID_ERR_INVALID_ARG"),
+    ("sum_kv_len", 999, "EID_ERR_INVALID_ARG"),          # below max_kv_len
     ("partition_size", 100, "EID_ERR_INVALID_ARG"),
     ("partition_size", 8192, "EID_ERR_INVALID_ARG"),
     ("num_blocks", 0, "EID_ERR_INVALID_ARG"),

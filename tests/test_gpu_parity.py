@@ -223,6 +223,7 @@ def test_many_sequences_cross_the_64_wide_scan(G):
         out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
         assert_close(out, ref, f"150 sequences w={window}")
         assert np.allclose(lse, ref_lse, atol=2e-3)
+        assert np.array_equal(G.run_attn(b, q, kc_d, vc_d, sinks, hint=True), out)
 
 
 @pytest.mark.parametrize("hkv", [1, 4, 16])
@@ -321,10 +322,13 @@ def test_lse_merge_entry_point_against_oracle_merge(G):
     assert np.allclose(ref, full, rtol=1e-10, atol=1e-13)
     # workspace rows are (sequence, row-in-sequence); here every sequence has ws_rows rows
     ws = np.zeros(ea.workspace_bytes(d), np.uint8)
-    ws[ml_off:ml_off + ml.size * 4] = ml.astype(np.float32).reshape(-1).view(np.uint8)
+    # the oracle returns [row, head, partition, ...]; the workspace is [row, partition, head, ...]
+    ml_ws = np.ascontiguousarray(ml.astype(np.float32).transpose(0, 2, 1, 3))
+    ws[ml_off:ml_off + ml.size * 4] = ml_ws.reshape(-1).view(np.uint8)
     with np.errstate(invalid="ignore", divide="ignore"):
         o_part = np.where(ml[..., 1:2] > 0, acc / ml[..., 1:2], 0.0).astype(np.float16)
-    ws[acc_off:acc_off + o_part.size * 2] = o_part.reshape(-1).view(np.uint8)
+    o_ws = np.ascontiguousarray(o_part.transpose(0, 2, 1, 3))
+    ws[acc_off:acc_off + o_part.size * 2] = o_ws.reshape(-1).view(np.uint8)
     ws_d = torch.from_numpy(ws).to(G.DEV)
     lse_d = torch.zeros((15, 64), dtype=torch.float32, device=G.DEV)
     out = ea.ops.lse_merge(b.geom, ws_d, G.dev(b.seq_lens), G.dev(b.cu_seqlens_q),
@@ -378,6 +382,15 @@ def test_config2_full_size(G, window):
         o2 = ea.attn_decode(g2, *args[1:], max_kv_len=b.max_kv_len, sinks=G.dev(sinks))
         torch.cuda.synchronize()
         assert np.abs(synth.bf16_bits_to_f32(G.bits_host(o2)) - o).max() <= 4e-3
+        o3 = ea.attn_decode(g2, *args[1:], max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
+                            sum_kv_len=int(b.seq_lens.sum()))
+        torch.cuda.synchronize()
+        assert torch.equal(o2, o3)
+    # the launch-sizing hint (exact sum, or any upper bound) only trims the grid
+    for hint in (int(b.seq_lens.sum()), 2 * int(b.seq_lens.sum()), 64 * b.max_kv_len):
+        oh = ea.attn_decode(*args, max_kv_len=b.max_kv_len, sinks=G.dev(sinks), sum_kv_len=hint)
+        torch.cuda.synchronize()
+        assert torch.equal(oh, out), hint
 
 
 def test_config3_mixed_full_size(G):
@@ -396,6 +409,11 @@ def test_config3_mixed_full_size(G):
                          sinks=G.dev(sinks))
     torch.cuda.synchronize()
     assert np.isfinite(synth.bf16_bits_to_f32(G.bits_host(out))).all()
+    oh = ea.attn_varlen(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                        G.dev(b.cu_seqlens_q), max_q_len=512, max_kv_len=b.max_kv_len,
+                        sinks=G.dev(sinks), sum_kv_len=int(b.seq_lens.sum()))
+    torch.cuda.synchronize()
+    assert torch.equal(oh, out)
     pre = int(np.argmin(b.seq_lens[:8]))
     _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [pre, 8, 9, 60, 127], "config3")
 
@@ -407,6 +425,11 @@ def test_config4_fp8_full_size(G):
     out = ea.attn_decode(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
                          max_kv_len=b.max_kv_len, sinks=G.dev(sinks), k_scale=ks, v_scale=vs)
     torch.cuda.synchronize()
+    oh = ea.attn_decode(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                        max_kv_len=b.max_kv_len, sinks=G.dev(sinks), k_scale=ks, v_scale=vs,
+                        sum_kv_len=int(b.seq_lens.sum()))
+    torch.cuda.synchronize()
+    assert torch.equal(oh, out)
     order = np.argsort(b.seq_lens)
     seqs = [int(order[0]), int(order[128]), int(order[-1]), 0, 1]
     _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, seqs, "config4",
@@ -423,6 +446,11 @@ def test_config5_verify_full_size(G, layer):
                          sinks=G.dev(sinks))
     torch.cuda.synchronize()
     assert np.isfinite(synth.bf16_bits_to_f32(G.bits_host(out))).all()
+    oh = ea.attn_varlen(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                        G.dev(b.cu_seqlens_q), max_q_len=5, max_kv_len=b.max_kv_len,
+                        sinks=G.dev(sinks), sum_kv_len=int(b.seq_lens.sum()))
+    torch.cuda.synchronize()
+    assert torch.equal(oh, out)
     order = np.argsort(b.seq_lens)
     _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [int(order[0]), int(order[64]), int(order[-1])],
                   f"config5 layer {layer}")
