@@ -355,13 +355,39 @@ struct WorkItem {
   int seq, part, nparts, row0, qlen, seq_len;
 };
 
-__device__ __forceinline__ int wave_inclusive_scan(int v, const int lane) {
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    const int o = __shfl_up(v, off);
-    if (lane >= off) v += o;
-  }
+// Inclusive prefix sum over the 64 lanes with DPP adds (row shifts, then the row totals
+// carried over with row_bcast): six dependent VALU ops instead of six LDS-crossbar
+// permutes.  A lane whose DPP source is out of range, or whose row is masked off, adds
+// the `old` operand, 0.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_add(const int v) {
+  return v + __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false);
+}
+__device__ __forceinline__ int wave_inclusive_scan(int v, const int /*lane*/) {
+  v = dpp_add<0x111, 0xf>(v);  // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);  // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);  // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);  // row_shr:8
+  v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
   return v;
+}
+// Sum over the 64 lanes, returned as a wave-uniform (scalar) value.  v must be >= 0.
+__device__ __forceinline__ int wave_total(const int v) {
+  return __builtin_amdgcn_readlane(wave_inclusive_scan(v, 0), 63);
+}
+__device__ __forceinline__ long long wave_total64(const long long v) {
+  // three 22-bit limbs: each limb's 64-lane sum stays below 2^28
+  const long long a = wave_total((int)(v & 0x3fffff));
+  const long long b = wave_total((int)((v >> 22) & 0x3fffff));
+  const long long c = wave_total((int)(v >> 44));
+  return a + (b << 22) + (c << 44);
+}
+// a / b for wave-uniform a >= 0, b > 0: the 64-bit division expands to some hundred
+// instructions, the 32-bit one to a third of that, and batches rarely need the former.
+__device__ __forceinline__ long long uniform_div(const long long a, const long long b) {
+  if (a < 0x7fffffffLL && b < 0x7fffffffLL) return (long long)((unsigned)a / (unsigned)b);
+  return a / b;
 }
 
 // Per-lane view of one sequence for the planning passes: partitions are counted from the
@@ -390,12 +416,6 @@ __device__ __forceinline__ int num_partitions(const AttnParams &p, const int spa
   return min((span + P - 1) / P, p.nparts_max);
 }
 
-__device__ __forceinline__ long long wave_sum(long long v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
-  return v;
-}
-
 // Partition size of this launch.  Fixed when the caller gave one.  Otherwise every wave
 // derives the same value from the batch itself.  With T = workgroups the device holds at
 // once: if the whole batch fits one device fill with partitions no longer than the cap,
@@ -409,38 +429,36 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
   if (!p.dynamic_partition) return p.partition;
   const int lane = threadIdx.x & 63;
   long long total = first.span;
-  int active = first.span > 0;
+  int active = __popcll(__ballot(first.span > 0));
   for (int s0 = 64; s0 < p.num_seqs; s0 += 64) {
     const SeqView v = view_seq(p, s0 + lane);
     total += v.span;
-    active += v.span > 0;
+    active += __popcll(__ballot(v.span > 0));
   }
-  total = wave_sum(total);
-  total = ((long long)__builtin_amdgcn_readfirstlane((int)(total >> 32)) << 32) |
-          (unsigned)__builtin_amdgcn_readfirstlane((int)total);
-  active = __builtin_amdgcn_readfirstlane((int)wave_sum(active));
+  total = wave_total64(total);
   const long long T = max(p.target_items, 1);
-  // (every value below is the same in all lanes; readfirstlane tells the compiler so, which
-  // keeps the partition and everything derived from it in scalar registers)
+  // (every value below is the same in all lanes and lives in scalar registers, and so does
+  // everything derived from the partition)
   // more than one fill: aim at about three fills of equal items, within [floor, cap]
   const int P3 = (int)min((long long)kDynPartitionCap,
-                          max((long long)kDynPartitionFloor, (total / (3 * T) + 63) / 64 * 64));
+                          max((long long)kDynPartitionFloor,
+                              (uniform_div(total, 3 * T) + 63) / 64 * 64));
   if (active >= T) return P3;
-  long long P = ((total + (T - active) - 1) / (T - active) + 63) / 64 * 64;  // items <= total/P + active <= T
+  // items <= total/P + active <= T
+  long long P = (uniform_div(total + (T - active) - 1, T - active) + 63) / 64 * 64;
   P = max(P, (long long)p.partition);
   if (P >= kDynPartitionCap) return P3;
   // The bound is pessimistic by up to one item per sequence: walk down while the exact
   // count still fits.
   for (int step = 0; step < 4 && P - 64 >= p.partition; ++step) {
     const int Pc = (int)P - 64;
-    long long items = num_partitions(p, first.span, Pc);
+    int items = num_partitions(p, first.span, Pc);
     for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
       items += num_partitions(p, view_seq(p, s0 + lane).span, Pc);
-    items = wave_sum(items);
-    if (__builtin_amdgcn_readfirstlane((int)(items > T))) break;
+    if (wave_total64(items) > T) break;
     P = Pc;
   }
-  return __builtin_amdgcn_readfirstlane((int)P);
+  return (int)P;
 }
 
 // Partition size of this launch: from the plan header when a plan kernel ran, else derived
@@ -491,7 +509,7 @@ __global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *p
   long long items = num_partitions(p, first.span, P);
   for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
     items += num_partitions(p, view_seq(p, s0 + lane).span, P);
-  items = wave_sum(items);
+  items = wave_total64(items);
   if (lane == 0) {
     plan_out[0] = P;
     plan_out[1] = (int32_t)items;
