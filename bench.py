@@ -131,9 +131,14 @@ def measure(w, steps, warmup, torch, synth, label):
         "q_tokens_per_s": work["q_tokens"] / ms_step * 1e3,
         "ctx_tokens_per_s": work["ctx_tokens"] / ms_step * 1e3,
     }
+    # the split-KV launch records the partition it ran with at the head of the workspace
+    # (meaningless when no sequence of the first class ran: reported as None)
+    part = int(w.attn[0]._keep[-1][:4].view(torch.int32).item())
+    r["partition"] = part if 64 <= part <= 4096 and part % 64 == 0 else None
     log(f"[bench] {label}: step {ms_step*1e3:.1f} us (attn {ms_attn*1e3:.1f}, merge "
         f"{ms_merge*1e3:.1f}, kv_write {ms_write*1e3:.1f}); attn {r['attn_GBps']:.0f} GB/s = "
-        f"{100*r['attn_GBps']/HBM_PEAK_GBS:.1f}% HBM, {r['attn_TFLOPs']:.1f} TFLOP/s")
+        f"{100*r['attn_GBps']/HBM_PEAK_GBS:.1f}% HBM, {r['attn_TFLOPs']:.1f} TFLOP/s; "
+        f"partition {r['partition']}")
     return r
 
 

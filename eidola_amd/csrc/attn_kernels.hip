@@ -439,26 +439,35 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
   const long long T = max(p.target_items, 1);
   // (every value below is the same in all lanes and lives in scalar registers, and so does
   // everything derived from the partition)
-  // more than one fill: aim at about three fills of equal items, within [floor, cap]
-  const int P3 = (int)min((long long)kDynPartitionCap,
-                          max((long long)kDynPartitionFloor,
-                              (uniform_div(total, 3 * T) + 63) / 64 * 64));
-  if (active >= T) return P3;
-  // items <= total/P + active <= T
-  long long P = (uniform_div(total + (T - active) - 1, T - active) + 63) / 64 * 64;
-  P = max(P, (long long)p.partition);
-  if (P >= kDynPartitionCap) return P3;
-  // The bound is pessimistic by up to one item per sequence: walk down while the exact
-  // count still fits.
-  for (int step = 0; step < 4 && P - 64 >= p.partition; ++step) {
-    const int Pc = (int)P - 64;
-    int items = num_partitions(p, first.span, Pc);
-    for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
-      items += num_partitions(p, view_seq(p, s0 + lane).span, Pc);
-    if (wave_total64(items) > T) break;
-    P = Pc;
+  // Smallest multiple of 64 (>= the planning minimum, < the cap) whose exact item count
+  // is <= Tx, or 0 if there is none.
+  auto single_fill = [&](const long long Tx) -> int {
+    if (active >= Tx) return 0;
+    // items <= total/P + active <= Tx
+    long long P = (uniform_div(total + (Tx - active) - 1, Tx - active) + 63) / 64 * 64;
+    P = max(P, (long long)p.partition);
+    if (P >= kDynPartitionCap) return 0;
+    // The bound is pessimistic by up to one item per sequence: walk down while the exact
+    // count still fits.
+    for (int step = 0; step < 4 && P - 64 >= p.partition; ++step) {
+      const int Pc = (int)P - 64;
+      int items = num_partitions(p, first.span, Pc);
+      for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
+        items += num_partitions(p, view_seq(p, s0 + lane).span, Pc);
+      if (wave_total64(items) > Tx) break;
+      P = Pc;
+    }
+    return (int)P;
+  };
+  // one workgroup per CU if the batch is small enough for that, else one device fill
+  if (p.target_items_lo < T) {
+    const int P = single_fill(max(p.target_items_lo, 1));
+    if (P) return P;
   }
-  return (int)P;
+  if (const int P = single_fill(T)) return P;
+  // more than one fill: aim at about three fills of equal items, within [floor, cap]
+  return (int)min((long long)kDynPartitionCap,
+                  max((long long)kDynPartitionFloor, (uniform_div(total, 3 * T) + 63) / 64 * 64));
 }
 
 // Partition size of this launch: from the plan header when a plan kernel ran, else derived
@@ -971,6 +980,16 @@ static int device_fill(F fn, int block) {
   return per_cu * max(1, prop.multiProcessorCount);
 }
 
+int device_cus() {
+  static const int cus = [] {
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 256;
+    return max(1, prop.multiProcessorCount);
+  }();
+  return cus;
+}
+
 template <int NT, bool FP8, int WAVES>
 static int fill_of() {
   static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES>, WAVES * 64);
@@ -997,12 +1016,16 @@ int splitkv_fill(int ntiles, bool fp8, int Hkv) {
 }
 
 // Upper bound on the number of work items of a launch, from what the host knows.  Items
-// never exceed num_seqs * nparts_max.  With the run-time partition they are at most one
-// device fill T in the single-fill regime, and sum/P3 + num_seqs in the multi-fill regime,
-// where P3 = min(cap, max(floor, ~sum/(3T))) makes sum/P3 <= min(sum/floor, max(sum/cap, 3T));
-// without the caller's sum_kv_len the sum is bounded by num_seqs * max_kv_len.
+// never exceed num_seqs * nparts_max.  With the run-time partition they are at most Tlo
+// (one workgroup per CU) or T (one device fill) in the single-fill tiers, and
+// sum/P3 + num_seqs in the multi-fill regime, where P3 = min(cap, max(floor, ~sum/(3T)))
+// makes sum/P3 <= min(sum/floor, max(sum/cap, 3T)).  Without the caller's sum_kv_len the
+// sum is bounded by num_seqs * max_kv_len.  With it, the host can often tell which tier the
+// kernels will take: their first estimate ceil64(total / (Tx - active)) grows with total
+// and with active, so if it is below the cap for (sum_kv_len, num_seqs) it is below the cap
+// for the real batch, and the tier Tx is taken.
 static long long item_bound(const AttnParams &p) {
-  const long long S = p.num_seqs, T = p.target_items;
+  const long long S = p.num_seqs, T = p.target_items, Tlo = p.target_items_lo;
   long long items = S * p.nparts_max;
   if (p.dynamic_partition) {
     const long long at_floor =
@@ -1010,9 +1033,14 @@ static long long item_bound(const AttnParams &p) {
     items = min(items, max(T, at_floor));
     if (p.sum_kv_len > 0) {
       const long long sum = p.sum_kv_len;
+      auto takes_tier = [&](const long long Tx) {
+        return S < Tx && ((sum + (Tx - S) - 1) / (Tx - S) + 63) / 64 * 64 < kDynPartitionCap;
+      };
       const long long multi =
           min(sum / kDynPartitionFloor, max(sum / kDynPartitionCap, 3 * T)) + S + 16;
-      items = min(items, max(T, multi));
+      if (Tlo < T && takes_tier(Tlo)) items = min(items, Tlo);
+      else if (takes_tier(T)) items = min(items, T);
+      else items = min(items, max(T, multi));
     }
   } else if (p.sum_kv_len > 0) {
     items = min(items, p.sum_kv_len / p.partition + S);
@@ -1037,10 +1065,17 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
   }
 }
 
+// Item count of the one-workgroup-per-CU tier of the run-time partition rule.
+static int fill_lo(int target_items) {
+  static const bool off = getenv("EID_FILL_LO_OFF") != nullptr;  // experiment switch
+  return off ? target_items : min(target_items, device_cus());
+}
+
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same
 // params so that it uses the same partition.
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st) {
+  p.target_items_lo = fill_lo(p.target_items);
   p.plan = nullptr;
   p.plan_slot = plan_slot;
   if (item_bound(p) > 4LL * p.target_items) {
@@ -1069,7 +1104,9 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
   return hipGetLastError();
 }
 
-hipError_t launch_merge(const AttnParams &p, hipStream_t st) {
+hipError_t launch_merge(const AttnParams &p0, hipStream_t st) {
+  AttnParams p = p0;
+  p.target_items_lo = fill_lo(p.target_items);  // read when the merge derives the partition itself
   dim3 grid(p.num_q_heads / 4, p.num_seqs * p.ws_rows);
   lse_merge_kernel<<<grid, 256, 0, st>>>(p);
   return hipGetLastError();

@@ -32,6 +32,7 @@ struct AttnParams {
   int32_t *plan_slot;    // where this launch's split-KV kernel records its partition for the merge
   float *ws_ml;          // [num_seqs*ws_rows][nparts_max][Hq][2]  (m natural-log units, l)
   _Float16 *ws_acc;      // [num_seqs*ws_rows][nparts_max][Hq][64] partition output, normalised
+  int32_t target_items_lo; // workgroups at one per CU (<= target_items)
   long long sum_kv_len;  // host's upper bound on the sum of seq_lens, 0 = unknown
   int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;
   int32_t window, partition, nparts_max, ws_rows;
