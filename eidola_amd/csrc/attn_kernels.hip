@@ -35,10 +35,18 @@ __device__ __forceinline__ const_i32_ptr as_constant(const int32_t *p) {
   return (const_i32_ptr)(uintptr_t)p;
 }
 
-// Row bookkeeping of one 16-row MFMA column tile.
+// Row bookkeeping of a wave's NT 16-row tiles.  Row r = 16 nt + (lane % 16) belongs to query
+// token tq0 + r / 8, so one per-lane value and four wave-uniform ones describe every tile;
+// the bounds are only materialised on chunks that need masking.
 struct RowInfo {
-  int pos;  // absolute position of the row's query token
-  int lo;   // first key the row may see
+  int t_lane;                    // tq0 + (lane % 16) / 8: the row's token in tile 0
+  int tq0, qlen, pos0, window;   // wave-uniform
+  // absolute position of the row's query token and the first key it may see
+  __device__ __forceinline__ void bounds(const int nt, int &pos, int &lo) const {
+    const int t = t_lane + 2 * nt;
+    pos = pos0 + (t < qlen ? t : tq0);
+    lo = window > 0 ? max(0, pos - window + 1) : 0;
+  }
 };
 
 // Scores, online softmax and PV for one 64-token chunk whose K operands are in registers
@@ -47,7 +55,7 @@ struct RowInfo {
 // row tiles.
 template <int NT>
 __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
-                                           const Frag8 (&qf)[NT][2], const RowInfo (&ri)[NT],
+                                           const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                            const int tc, const bool need_mask, const float c2,
                                            float (&m)[NT], f32x4 (&lacc)[NT],
                                            f32x4 (&acc)[NT][4]) {
@@ -66,23 +74,41 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
       vf[mt][pr].w[2] = b2[0];
       vf[mt][pr].w[3] = b2[1];
     }
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    // S^T = K Q^T (raw scores, fp32)
-    f32x4 S[4];
+  // S^T = K Q^T (raw scores, fp32).  With four row tiles the scores of tile nt + 1 are
+  // issued before the softmax of tile nt, so that the matrix pipe has work while the
+  // vector ALU runs the softmax.
+  constexpr bool kPipe = false;  // (four-tile pipelining needs 16 more VGPRs than the prefill kernel has)
+  auto scores = [&](const int nt, f32x4 (&S)[4]) {
+    if (NT == 4) __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       f32x4 z = {0.f, 0.f, 0.f, 0.f};
       z = mfma16x32(kf[b][0], qf[nt][0], z);
       S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
     }
+    if (NT == 4) __builtin_amdgcn_s_setprio(0);
+  };
+  f32x4 Snext[4];
+  if (kPipe) scores(0, Snext);
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    f32x4 S[4];
+    if (kPipe) {
+#pragma unroll
+      for (int b = 0; b < 4; ++b) S[b] = Snext[b];
+      if (nt + 1 < NT) scores(nt + 1, Snext);
+    } else {
+      scores(nt, S);
+    }
     if (need_mask) {
+      int pos, lo;
+      ri.bounds(nt, pos, lo);
 #pragma unroll
       for (int b = 0; b < 4; ++b)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int j = tc + b * kBlock + 4 * g + r;
-          if (j < ri[nt].lo || j > ri[nt].pos) S[b][r] = -INFINITY;
+          if (j < lo || j > pos) S[b][r] = -INFINITY;
         }
     }
     // row maximum: v_max3 tree over the lane's 16 scores, then across the four lane rows
@@ -125,6 +151,7 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
       pf[pr].w[3] = pack_bf16(S[2 * pr + 1][2], S[2 * pr + 1][3]);
     }
     // row sums of the bf16-rounded P (the same values the numerator uses), on the MFMA pipe
+    if (NT == 4) __builtin_amdgcn_s_setprio(2);
     lacc[nt] = mfma16x32(ones, pf[0], lacc[nt]);
     lacc[nt] = mfma16x32(ones, pf[1], lacc[nt]);
     // O^T += V^T P^T
@@ -132,6 +159,7 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
       for (int pr = 0; pr < 2; ++pr) acc[nt][mt] = mfma16x32(vf[mt][pr], pf[pr], acc[nt][mt]);
+    if (NT == 4) __builtin_amdgcn_s_setprio(0);
   }
 }
 
@@ -141,7 +169,7 @@ template <int NT, bool FP8>
 __device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
                                        const int t_begin, const int t_end, const int seq_len,
                                        const int pos_first, const int lo_last,
-                                       const Frag8 (&qf)[NT][2], const RowInfo (&ri)[NT],
+                                       const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                        uint8_t *wave_lds, float (&m)[NT], f32x4 (&lacc)[NT],
                                        f32x4 (&acc)[NT][4]) {
   const int lane = threadIdx.x & 63;
@@ -326,7 +354,7 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
 template <int NT>
 __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, const int qlen,
                                        const int tq0, const int kvh, const int pos0,
-                                       Frag8 (&qf)[NT][2], RowInfo (&ri)[NT]) {
+                                       Frag8 (&qf)[NT][2], RowInfo &ri) {
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
 #pragma unroll
@@ -339,9 +367,12 @@ __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, cons
         p.q + ((size_t)(row0 + tt) * p.num_q_heads + kvh * kGroup + (r & 7)) * kHeadDim + g * 16;
     qf[nt][0].u = valid ? *(const u32x4 *)qp : u32x4{0, 0, 0, 0};
     qf[nt][1].u = valid ? *(const u32x4 *)(qp + 8) : u32x4{0, 0, 0, 0};
-    ri[nt].pos = pos0 + tt;
-    ri[nt].lo = p.window > 0 ? max(0, ri[nt].pos - p.window + 1) : 0;
   }
+  ri.t_lane = tq0 + (i16 >> 3);
+  ri.tq0 = tq0;
+  ri.qlen = qlen;
+  ri.pos0 = pos0;
+  ri.window = p.window;
 }
 
 // Work-item lookup shared by the split-KV kernel: the launch serves the compacted list of
@@ -576,7 +607,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
 
   Frag8 qf[NT][2];
-  RowInfo ri[NT];
+  RowInfo ri;
   load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
@@ -705,7 +736,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int lo_last = W > 0 ? max(0, pos_last - W + 1) : 0;
 
   Frag8 qf[NT][2];
-  RowInfo ri[NT];
+  RowInfo ri;
   load_q<NT>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri);
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
