@@ -53,7 +53,7 @@ struct RowInfo {
 // and whose V tile sits in LDS (four 16-token pages of kVRowBytes-padded rows; `v_rd` is
 // the lane's transpose-read base).  The V^T operands are fetched once and reused by all NT
 // row tiles.
-template <int NT>
+template <int NT, int VROW = kVRowBytes>
 __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
                                            const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                            const int tc, const bool need_mask, const float c2,
@@ -67,8 +67,8 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
   for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr) {
-      const u32x2 a = lds_read_tr16(v_rd + (2 * pr) * kVPageBytes + 32 * mt);
-      const u32x2 b2 = lds_read_tr16(v_rd + (2 * pr + 1) * kVPageBytes + 32 * mt);
+      const u32x2 a = lds_read_tr16(v_rd + (2 * pr) * (kBlock * VROW) + 32 * mt);
+      const u32x2 b2 = lds_read_tr16(v_rd + (2 * pr + 1) * (kBlock * VROW) + 32 * mt);
       vf[mt][pr].w[0] = a[0];
       vf[mt][pr].w[1] = a[1];
       vf[mt][pr].w[2] = b2[0];
@@ -643,7 +643,14 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
 constexpr int kPfWaves = 4;
 constexpr int kPfWaveTok = 8;                     // query tokens per wave (x 8 heads = 64 rows)
 constexpr int kPfTok = kPfWaves * kPfWaveTok;     // query tokens per workgroup
-constexpr int kPfTileBytes = kChunk * kVRowBytes; // one 64-token K or V tile of one KV head
+// Row strides of the LDS tiles.  K is read 16 bytes per lane by 16 lanes at a time, one row
+// each: 144 B (36 banks) sends them to 16 distinct 4-bank groups.  V^T is read 8 bytes per
+// lane by 32 lanes at a time, 8 rows x 32 B: that wants the rows 8 banks apart modulo 64,
+// i.e. a stride of 8 x odd banks: 160 B.  (With 144 B rows 0 and 7 share banks.)
+constexpr int kPfKRowBytes = 144;
+constexpr int kPfVRowBytes = 160;
+constexpr int kPfKTileBytes = kChunk * kPfKRowBytes;  // one 64-token K tile of one KV head
+constexpr int kPfVTileBytes = kChunk * kPfVRowBytes;  // one 64-token V tile
 
 __device__ __forceinline__ bool find_prefill_item(const AttnParams &p, const int w, int &seq,
                                                   int &tile, int &row0, int &qlen, int &seq_len) {
@@ -692,7 +699,8 @@ template <bool FP8>
 __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnParams p) {
   constexpr int NT = 4;
   constexpr int kElt = FP8 ? 1 : 2;
-  __shared__ __align__(16) uint8_t lds[2][2][kPfTileBytes];  // [buffer][K, V]
+  __shared__ __align__(16) uint8_t lds_k[2][kPfKTileBytes];  // double-buffered K tile
+  __shared__ __align__(16) uint8_t lds_v[2][kPfVTileBytes];  // double-buffered V tile
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
@@ -756,7 +764,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const size_t page_bytes = (size_t)kBlock * row_bytes;
   const uint32_t gl_off = (uint32_t)(ld_row & 15) * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
                           (uint32_t)ld_seg * (16 * kElt);
-  const uint32_t st_off = (uint32_t)ld_row * kVRowBytes + ld_seg * 32;
+  const uint32_t st_off_k = (uint32_t)ld_row * kPfKRowBytes + ld_seg * 32;
+  const uint32_t st_off_v = (uint32_t)ld_row * kPfVRowBytes + ld_seg * 32;
   const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
   const int nblk_total = (t_end + kBlock - 1) / kBlock;
 
@@ -803,10 +812,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
       v0 = u32x4{0, 0, 0, 0};
       v1 = u32x4{0, 0, 0, 0};
     }
-    *(u32x4 *)(&lds[buf][0][st_off]) = k0;
-    *(u32x4 *)(&lds[buf][0][st_off + 16]) = k1;
-    *(u32x4 *)(&lds[buf][1][st_off]) = v0;
-    *(u32x4 *)(&lds[buf][1][st_off + 16]) = v1;
+    *(u32x4 *)(&lds_k[buf][st_off_k]) = k0;
+    *(u32x4 *)(&lds_k[buf][st_off_k + 16]) = k1;
+    *(u32x4 *)(&lds_v[buf][st_off_v]) = v0;
+    *(u32x4 *)(&lds_v[buf][st_off_v + 16]) = v1;
   };
 
   fetch(t_begin);
@@ -817,16 +826,16 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     const bool has_next = tc + kChunk < t_end;
     if (has_next) fetch(tc + kChunk);
     if (wave_active && tc <= pos_last && tc + kChunk > lo_first) {
-      const uint8_t *kt = &lds[cur][0][0] + i16 * kVRowBytes + g * 32;
-      const uint8_t *v_rd = &lds[cur][1][0] + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
+      const uint8_t *kt = &lds_k[cur][0] + i16 * kPfKRowBytes + g * 32;
+      const uint8_t *v_rd = &lds_v[cur][0] + (4 * g + (i16 >> 2)) * kPfVRowBytes + 8 * (i16 & 3);
       Frag8 kf[4][2];
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        kf[b][0].u = *(const u32x4 *)(kt + b * kVPageBytes);
-        kf[b][1].u = *(const u32x4 *)(kt + b * kVPageBytes + 16);
+        kf[b][0].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes));
+        kf[b][1].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes) + 16);
       }
       const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
-      chunk_step<NT>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
+      chunk_step<NT, kPfVRowBytes>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
     }
     if (has_next) stash(tc + kChunk, cur ^ 1);
     __syncthreads();
