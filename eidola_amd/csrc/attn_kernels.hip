@@ -112,14 +112,14 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
         }
     }
     // row maximum: v_max3 tree over the lane's 16 scores, then across the four lane rows
-    float mloc = __builtin_fmaxf(__builtin_fmaxf(S[0][0], S[0][1]), S[0][2]);
-    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[0][3]), S[1][0]);
-    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[1][1]), S[1][2]);
-    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[1][3]), S[2][0]);
-    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[2][1]), S[2][2]);
-    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[2][3]), S[3][0]);
-    mloc = __builtin_fmaxf(__builtin_fmaxf(mloc, S[3][1]), S[3][2]);
-    mloc = __builtin_fmaxf(mloc, S[3][3]);
+    float mloc = max3(S[0][0], S[0][1], S[0][2]);
+    mloc = max3(mloc, S[0][3], S[1][0]);
+    mloc = max3(mloc, S[1][1], S[1][2]);
+    mloc = max3(mloc, S[1][3], S[2][0]);
+    mloc = max3(mloc, S[2][1], S[2][2]);
+    mloc = max3(mloc, S[2][3], S[3][0]);
+    mloc = max3(mloc, S[3][1], S[3][2]);
+    mloc = max2(mloc, S[3][3]);
     mloc = rowgroup_max(mloc) * c2;
     // Lazy rescaling: the reference maximum m only moves when the running maximum has
     // outgrown it by more than kLazyLog2 (in log2 units), so exp2(s - m) stays <= 2^kLazyLog2

@@ -28,15 +28,23 @@ __device__ __forceinline__ f32x4 mfma16x32(const Frag8 &a, const Frag8 &b, f32x4
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
 }
 
+// IEEE-754-2019 maximum (v_maximum3_f32 on gfx950).  fmaxf() in IEEE mode first quiets both
+// operands (v_max x, x), which doubles the length of a max tree; maximum() takes them as
+// they are and lets a NaN through, which is what a NaN score has to do anyway.
+__device__ __forceinline__ float max2(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  return __builtin_elementwise_maximum(__builtin_elementwise_maximum(a, b), c);
+}
+
 // max / sum over the four lanes {n, n+16, n+32, n+48} that share MFMA column n.
 // v_permlane16_swap / v_permlane32_swap exchange 16-lane rows (gfx950).
 __device__ __forceinline__ float rowgroup_max(float x) {
   uint32_t u = __float_as_uint(x);
   auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  x = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  x = max2(__uint_as_float(r[0]), __uint_as_float(r[1]));
   u = __float_as_uint(x);
   r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  return max2(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float rowgroup_sum(float x) {
   uint32_t u = __float_as_uint(x);
