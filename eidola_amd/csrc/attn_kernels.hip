@@ -865,8 +865,8 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
   const int L = p.seq_lens[s];
   if (L < qlen) return;
-  // recorded by the split-KV launch this merge follows; derived again when it stands alone
-  const int P = p.plan_slot ? p.plan_slot[0] : effective_partition(p, view_seq(p, lane));
+  // run-time partition: recorded by the split-KV launch of this class; else the caller's
+  const int P = p.plan_slot ? p.plan_slot[0] : p.partition;
   const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
   if (nparts <= 1) return;
 
@@ -1144,9 +1144,7 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
   return hipGetLastError();
 }
 
-hipError_t launch_merge(const AttnParams &p0, hipStream_t st) {
-  AttnParams p = p0;
-  p.target_items_lo = fill_lo(p.target_items);  // read when the merge derives the partition itself
+hipError_t launch_merge(const AttnParams &p, hipStream_t st) {
   dim3 grid(p.num_q_heads / 4, p.num_seqs * p.ws_rows);
   lse_merge_kernel<<<grid, 256, 0, st>>>(p);
   return hipGetLastError();

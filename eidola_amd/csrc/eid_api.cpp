@@ -294,6 +294,10 @@ int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args, void
   p.qlen_lo = desc->max_q_len <= 2 ? 1 : 3;
   p.qlen_hi = desc->max_q_len <= 2 ? 2 : eid::kShortQMax;
   p.target_items = eid::splitkv_fill(desc->max_q_len <= 2 ? 1 : 3, fp8, desc->num_kv_heads);
+  // With a run-time partition the merge takes the size the split-KV launch of this class
+  // recorded in the workspace header (the attention entry points do the same).
+  if (pl.dynamic)
+    p.plan_slot = static_cast<int32_t *>(args->workspace) + (desc->max_q_len <= 2 ? 0 : 2);
   hipError_t e = eid::launch_merge(p, static_cast<hipStream_t>(hip_stream));
   if (e != hipSuccess) return hip_fail(e, "merge launch");
   return EID_OK;

@@ -139,7 +139,9 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  * the split-KV kernel for this desc) into args->out / args->lse.  Exposed for tests.
  * Serves one class of sequences per call, as the split-KV launches do: q_len <= 2 when
  * desc->max_q_len <= 2, otherwise q_len 3..6.  Sequences with a single partition are left
- * alone (the split-KV kernel writes their output itself).
+ * alone (the split-KV kernel writes their output itself).  With desc->partition_size == 0
+ * the partition is the one the last eid_attn_decode / eid_attn_varlen call on this
+ * workspace recorded in its header, so such a call must have preceded.
  * Workspace layout, with R = min(max_q_len, 6) and N = partitions per sequence (max):
  *   256 bytes                         launch plan (written by the library)
  *   float ml [num_seqs*R][N][Hq][2]   m (natural-log units, -inf if empty) and
