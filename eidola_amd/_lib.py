@@ -69,6 +69,7 @@ class AttnArgs(C.Structure):
         ("v_scale", C.c_void_p),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
+        ("split_done_event", C.c_void_p),
     ]
 
 

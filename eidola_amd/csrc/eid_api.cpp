@@ -235,6 +235,10 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   hipError_t e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  if (args->split_done_event) {
+    e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
+    if (e != hipSuccess) return hip_fail(e, "split_done_event record");
+  }
   if (pl.nparts_max > 1) {
     e = eid::launch_merge(p, st);
     if (e != hipSuccess) return hip_fail(e, "merge launch");
@@ -259,6 +263,10 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  if (args->split_done_event) {
+    e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
+    if (e != hipSuccess) return hip_fail(e, "split_done_event record");
+  }
   if (pl.nparts_max > 1) {
     e = eid::launch_merge(p, st);
     if (e != hipSuccess) return hip_fail(e, "merge launch");

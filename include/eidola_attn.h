@@ -100,6 +100,10 @@ typedef struct eid_attn_args {
   const float *v_scale; /* fp8 only */
   void *workspace;      /* >= eid_workspace_bytes(desc), 256-byte aligned */
   size_t workspace_bytes;
+  void *split_done_event; /* optional hipEvent_t (NULL = none), for profiling: recorded on the
+                             stream right after the split-KV launch of the q_len <= 2 class,
+                             i.e. before its merge, so that a caller who records an event of
+                             his own before the call can time that kernel by itself */
 } eid_attn_args;
 
 /*

@@ -342,6 +342,31 @@ def test_lse_merge_entry_point_against_oracle_merge(G):
     assert (G.bits_host(out)[10:] == 0).all()
 
 
+def test_split_done_event_is_recorded_between_the_phases(G):
+    """args.split_done_event is a profiling hook: recorded after the split-KV launch, before
+    the merge; it must not change the result."""
+    b = make_batch([3000, 1500, 70], [1, 1, 1], partition=256)
+    q, k, v, sinks = logical_tensors(b)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    call = ea.prepare("eid_attn_decode", b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table),
+                      G.dev(b.seq_lens), max_kv_len=b.max_kv_len, sinks=G.dev(sinks))
+    ref = call().clone()
+    torch.cuda.synchronize()
+    e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    for e in (e0, e1, e2):
+        e.record()   # creates the hipEvent_t handles
+    torch.cuda.synchronize()
+    call.out.zero_()
+    e0.record()
+    call.args.split_done_event = e1.cuda_event
+    call()
+    e2.record()
+    torch.cuda.synchronize()
+    call.args.split_done_event = None
+    assert torch.equal(call.out, ref)
+    assert 0.0 < e0.elapsed_time(e1) <= e0.elapsed_time(e2)
+
+
 # ---------------------------------------------------------------- benchmark configurations
 def _sample_check(G, b, q_d, kc_d, vc_d, sinks, out_d, seqs, what, ks=None, vs=None):
     sub, kc, vc = G.compact_to_cpu(b, kc_d, vc_d, seqs)
