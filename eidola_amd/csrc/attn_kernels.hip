@@ -556,6 +556,36 @@ __global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *p
   }
 }
 
+// One work item: wave `wave` of the workgroup attends the rows of KV head `kvh` over
+// partition it.part (P tokens) of sequence it.seq and writes the output or the partial.
+template <int NT, bool FP8>
+__device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem &it, const int P,
+                                             const int kvh, const int wave, uint8_t *lds) {
+  const int s = it.seq, part = it.part, nparts = it.nparts;
+  const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
+  const int kb = kv_begin(L, qlen, p.window);
+  const int t0 = kb + part * P;
+  const int t1 = min(t0 + P, L);
+  const int pos0 = L - qlen;
+  const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
+
+  Frag8 qf[NT][2];
+  RowInfo ri;
+  load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
+  float m[NT];
+  f32x4 lacc[NT], acc[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    m[nt] = kNegBig;
+    lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
+                  lacc, acc);
+  finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lacc, acc);
+}
+
 // ---------------------------------------------------------------------------------------
 // Split-KV kernel.  grid = (num_seqs * nparts_max, Hkv / WAVES); workgroup blockIdx.x takes
 // work item blockIdx.x (see find_work_item) and wave w of it owns KV head
@@ -567,6 +597,22 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = blockIdx.y * WAVES + wave;
+  if (p.nparts_max == 1) {
+    // Every sequence is a single item (short spans: sliding-window layers, short contexts):
+    // workgroup w serves sequence w, found with scalar loads alone; sequences of another
+    // q_len class leave at once.
+    const SeqView v = view_seq(p, blockIdx.x);
+    if (v.span <= 0) return;
+    WorkItem it;
+    it.seq = blockIdx.x;
+    it.part = 0;
+    it.nparts = 1;
+    it.row0 = v.row0;
+    it.qlen = v.qlen;
+    it.seq_len = v.seq_len;
+    splitkv_item<NT, FP8>(p, it, 1 << 30, kvh, wave, lds);
+    return;
+  }
   if (planned_out(p, blockIdx.x)) return;
   // One wave looks the work item up and hands it to the others through LDS: the lookup is
   // several hundred instructions, and eight waves doing it side by side on every CU at the
@@ -598,29 +644,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   it.seq_len = __builtin_amdgcn_readfirstlane(item_lds[6]);
   // the merge launch that follows reads the partition from here instead of re-deriving it
   if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
-  const int s = it.seq, part = it.part, nparts = it.nparts;
-  const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
-  const int kb = kv_begin(L, qlen, p.window);
-  const int t0 = kb + part * P;
-  const int t1 = min(t0 + P, L);
-  const int pos0 = L - qlen;
-  const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
-
-  Frag8 qf[NT][2];
-  RowInfo ri;
-  load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
-  float m[NT];
-  f32x4 lacc[NT], acc[NT][4];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    m[nt] = kNegBig;
-    lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-  attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
-                  lacc, acc);
-  finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lacc, acc);
+  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1066,6 +1090,7 @@ int splitkv_fill(int ntiles, bool fp8, int Hkv) {
 // for the real batch, and the tier Tx is taken.
 static long long item_bound(const AttnParams &p) {
   const long long S = p.num_seqs, T = p.target_items, Tlo = p.target_items_lo;
+  if (p.nparts_max == 1) return S;  // workgroup w serves sequence w
   long long items = S * p.nparts_max;
   if (p.dynamic_partition) {
     const long long at_floor =
@@ -1118,7 +1143,7 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   p.target_items_lo = fill_lo(p.target_items);
   p.plan = nullptr;
   p.plan_slot = plan_slot;
-  if (item_bound(p) > 4LL * p.target_items) {
+  if (p.nparts_max > 1 && item_bound(p) > 4LL * p.target_items) {
     AttnParams q = p;
     plan_kernel<<<1, 64, 0, st>>>(q, plan_slot);
     const hipError_t e = hipGetLastError();

@@ -255,23 +255,31 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   hipError_t e;
+  // The kernels sort sequences into classes by q_len on the device.  When every sequence
+  // has max_q_len query rows (num_q_tokens says so) the host knows the one class that is
+  // populated and launches nothing for the others.
+  const bool uniform = (int64_t)desc->num_seqs * desc->max_q_len == desc->num_q_tokens;
+  const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= eid::kShortQMax;
+  const bool only_prefill = uniform && desc->max_q_len > eid::kShortQMax;
+  int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
-  p.qlen_lo = 1;
-  p.qlen_hi = 2;
-  p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
-  int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
-  if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  if (!only_verify && !only_prefill) {
+    p.qlen_lo = 1;
+    p.qlen_hi = 2;
+    p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
+    e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
+    if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  }
   if (args->split_done_event) {
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
     if (e != hipSuccess) return hip_fail(e, "split_done_event record");
   }
-  if (pl.nparts_max > 1) {
+  if (!only_verify && !only_prefill && pl.nparts_max > 1) {
     e = eid::launch_merge(p, st);
     if (e != hipSuccess) return hip_fail(e, "merge launch");
   }
-  if (desc->max_q_len > 2) {  // q_len 3..6: three tiles
+  if (desc->max_q_len > 2 && !only_prefill) {  // q_len 3..6: three tiles
     p.qlen_lo = 3;
     p.qlen_hi = eid::kShortQMax;
     p.target_items = eid::splitkv_fill(3, fp8, desc->num_kv_heads);
