@@ -20,10 +20,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # HBM bytes per launch of the split-KV decode kernel on this exact seeded batch, from two
-# rocprofv3 --pmc passes over this script (FETCH_SIZE 242,823 KiB x 2.0, WRITE_SIZE 8,972 KiB
+# rocprofv3 --pmc passes over this script (FETCH_SIZE 241,250 KiB x 2.0, WRITE_SIZE 2,080 KiB
 # x 1.0; the factors are what the same counters read for a plain 1 GiB device copy run with
 # --calibrate-copy).  See profiles/splitkv_decode_config2.md.
-TRAFFIC_BYTES_PER_LAUNCH = int((242_823 * 2.0 + 8_972 * 1.0) * 1024)
+TRAFFIC_BYTES_PER_LAUNCH = int((241_250 * 2.0 + 2_080 * 1.0) * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "paged sink-attn decode HBM GB/s (% peak) + ragged-batch tokens/s, 1 GPU"
 
