@@ -1131,10 +1131,7 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
 }
 
 // Item count of the one-workgroup-per-CU tier of the run-time partition rule.
-static int fill_lo(int target_items) {
-  static const bool off = getenv("EID_FILL_LO_OFF") != nullptr;  // experiment switch
-  return off ? target_items : min(target_items, device_cus());
-}
+static int fill_lo(int target_items) { return min(target_items, device_cus()); }
 
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same
