@@ -168,6 +168,47 @@ def measure(w, steps, warmup, torch, synth, label):
     return r
 
 
+def sched_bench(synth, ea, steps=200):
+    """Host cost of the batch-metadata builder on the decode configuration: 64 sequences
+    with config 2's context lengths are prefilled through the scheduler, then `steps`
+    decode steps (one new token per sequence) are built; microseconds per built step."""
+    import numpy as np
+    b = synth.config2()
+    mb = b.block_table.shape[1] + (steps + 15) // 16 + 1   # room for the decode steps
+    sched = ea.Scheduler(b.num_blocks, mb, prefix_reuse=True)
+    ids = np.arange(b.num_seqs, dtype=np.int64)
+    for i in ids:
+        sched.add_seq(int(i))
+    rng = np.random.default_rng(1)
+    first = np.maximum(b.seq_lens - 1, 1).astype(np.int32)
+    t0 = time.perf_counter()
+    sched.build_batch(ids, first, rng.integers(0, 50000, size=int(first.sum())))
+    t_prefill = time.perf_counter() - t0
+    ones = np.ones(b.num_seqs, dtype=np.int32)
+    # calling through the raw ABI with preallocated buffers, as an engine loop would
+    import ctypes as C
+    from eidola_amd._lib import BatchInfo
+    lib = ea.load_library()
+    bt = np.zeros((b.num_seqs, mb), np.int32)
+    slot, cu = np.empty(b.num_seqs, np.int64), np.empty(b.num_seqs + 1, np.int32)
+    sl, pos, tok = np.empty(b.num_seqs, np.int32), np.empty(b.num_seqs, np.int32), np.zeros(b.num_seqs, np.int32)
+    info = BatchInfo()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        rc = lib.eid_sched_build_batch(sched._h, ids.ctypes.data, ones.ctypes.data, b.num_seqs,
+                                       tok.ctypes.data, bt.ctypes.data, slot.ctypes.data,
+                                       cu.ctypes.data, sl.ctypes.data, pos.ctypes.data, C.byref(info))
+        assert rc == 0
+    us = (time.perf_counter() - t0) / steps * 1e6
+    r = {"config": "sched_build_batch_decode64", "host_us_per_step": us,
+         "prefill_build_ms": t_prefill * 1e3, "prefill_tokens": int(first.sum()),
+         "sum_kv_len": int(info.sum_kv_len)}
+    log(f"[bench] scheduler: {us:.1f} us of host time per 64-sequence decode step "
+        f"(prefix index on); building the {int(first.sum())}-token prefill batch took "
+        f"{t_prefill*1e3:.1f} ms")
+    return r
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -314,6 +355,7 @@ def main():
                                  f"config5_verify_layer{layer}"))
             w5 = None
             torch.cuda.empty_cache()
+        extra.append(sched_bench(synth, ea))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)

@@ -15,12 +15,14 @@ EID_ERR_INVALID_ARG = -1
 EID_ERR_UNSUPPORTED = -2
 EID_ERR_WORKSPACE = -3
 EID_ERR_HIP = -4
+EID_ERR_NO_BLOCKS = -5
 
 _STATUS_NAMES = {
     EID_ERR_INVALID_ARG: "EID_ERR_INVALID_ARG",
     EID_ERR_UNSUPPORTED: "EID_ERR_UNSUPPORTED",
     EID_ERR_WORKSPACE: "EID_ERR_WORKSPACE",
     EID_ERR_HIP: "EID_ERR_HIP",
+    EID_ERR_NO_BLOCKS: "EID_ERR_NO_BLOCKS",
 }
 
 
@@ -73,8 +75,31 @@ class AttnArgs(C.Structure):
     ]
 
 
+class SchedConfig(C.Structure):
+    _fields_ = [
+        ("struct_size", C.c_uint32),
+        ("block_size", C.c_int32),
+        ("num_blocks", C.c_int64),
+        ("max_blocks_per_seq", C.c_int32),
+        ("prefix_reuse", C.c_int32),
+    ]
+
+
+class BatchInfo(C.Structure):
+    _fields_ = [
+        ("num_seqs", C.c_int32),
+        ("num_q_tokens", C.c_int32),
+        ("max_q_len", C.c_int32),
+        ("max_kv_len", C.c_int32),
+        ("sum_kv_len", C.c_int64),
+    ]
+
+
 EXPORTS = ("eid_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
            "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
+SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
+                 "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
+                 "eid_sched_block_refs", "eid_sched_build_batch")
 
 _lib = None
 
@@ -112,6 +137,24 @@ def load_library():
     lib.eid_last_error.restype = C.c_char_p
     lib.eid_version.argtypes = []
     lib.eid_version.restype = C.c_uint32
+    # host-side scheduler (include/eidola_sched.h)
+    lib.eid_sched_create.argtypes = [C.POINTER(SchedConfig), C.POINTER(P)]
+    lib.eid_sched_create.restype = C.c_int32
+    lib.eid_sched_destroy.argtypes = [P]
+    lib.eid_sched_destroy.restype = None
+    lib.eid_sched_add_seq.argtypes = [P, C.c_int64, P, C.c_int32, C.POINTER(C.c_int32)]
+    lib.eid_sched_add_seq.restype = C.c_int32
+    lib.eid_sched_free_seq.argtypes = [P, C.c_int64]
+    lib.eid_sched_free_seq.restype = C.c_int32
+    lib.eid_sched_seq_len.argtypes = [P, C.c_int64]
+    lib.eid_sched_seq_len.restype = C.c_int32
+    lib.eid_sched_free_blocks.argtypes = [P]
+    lib.eid_sched_free_blocks.restype = C.c_int64
+    lib.eid_sched_block_refs.argtypes = [P, C.c_int64]
+    lib.eid_sched_block_refs.restype = C.c_int32
+    lib.eid_sched_build_batch.argtypes = [P, P, P, C.c_int32, P, P, P, P, P, P,
+                                          C.POINTER(BatchInfo)]
+    lib.eid_sched_build_batch.restype = C.c_int32
     _lib = lib
     return lib
 

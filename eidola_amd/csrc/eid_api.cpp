@@ -21,15 +21,26 @@ hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t
 }  // namespace eid
 
 namespace {
-
 thread_local char g_err[512] = "";
+}  // namespace
+
+namespace eid {
+// Records the thread-local error text of the library (shared with the scheduler's file).
+int32_t set_error(int32_t status, const char *fmt, va_list ap) {
+  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  return status;
+}
+void clear_error() { g_err[0] = 0; }
+}  // namespace eid
+
+namespace {
 
 int32_t fail(eid_status st, const char *fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
-  vsnprintf(g_err, sizeof g_err, fmt, ap);
+  const int32_t rc = eid::set_error((int32_t)st, fmt, ap);
   va_end(ap);
-  return (int32_t)st;
+  return rc;
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -53,7 +53,8 @@ typedef enum {
   EID_ERR_INVALID_ARG = -1, /* null pointer, bad shape, misalignment, bad struct_size */
   EID_ERR_UNSUPPORTED = -2, /* geometry or dtype outside what this version builds    */
   EID_ERR_WORKSPACE = -3,   /* workspace NULL or smaller than eid_workspace_bytes()  */
-  EID_ERR_HIP = -4          /* a HIP runtime call or kernel launch failed            */
+  EID_ERR_HIP = -4,         /* a HIP runtime call or kernel launch failed            */
+  EID_ERR_NO_BLOCKS = -5    /* eidola_sched.h: the KV pool cannot hold the request   */
 } eid_status;
 
 typedef enum { EID_KV_BF16 = 0, EID_KV_FP8_E4M3 = 1 } eid_kv_dtype;
