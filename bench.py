@@ -209,6 +209,35 @@ def sched_bench(synth, ea, steps=200):
     return r
 
 
+def rope_bench(torch, ea, synth, steps=50):
+    """eid_rope_kv_write on config 3's new tokens (4,216) and on a 64-token decode step:
+    HBM-bound; algorithmic bytes = T * (qkv row read 10,240 + q row written 8,192 + k and v
+    rows written 2 * 1,024) + the cos/sin rows read."""
+    import numpy as np
+    g = ea.AttnGeometry()
+    nb = 20000
+    kc = torch.zeros((nb, 16, 8, 64), dtype=torch.bfloat16, device="cuda:0")
+    vc = torch.zeros_like(kc)
+    table = torch.from_numpy(ea.yarn_cos_sin(8192)).to("cuda:0")
+    out = []
+    for T in (4216, 64):
+        qkv = torch.randn((T, 5120), device="cuda:0").to(torch.bfloat16)
+        pos = torch.randint(0, 8192, (T,), dtype=torch.int32, device="cuda:0")
+        slots = torch.randperm(nb * 16, device="cuda:0")[:T].to(torch.int64)
+        q = torch.empty((T, 64, 64), dtype=torch.bfloat16, device="cuda:0")
+        fn = lambda i: ea.rope_kv_write(g, qkv, pos, table, kc, vc, slots, q_out=q)
+        for i in range(5):
+            fn(i)
+        ms = event_ms(fn, steps, torch)
+        nbytes = T * (10240 + 8192 + 2048 + 256)
+        r = {"config": f"rope_kv_write_{T}_tokens", "ms": ms, "alg_bytes": nbytes,
+             "GBps": nbytes / ms / 1e6}
+        log(f"[bench] rope_kv_write, {T} tokens: {ms*1e3:.1f} us per call, "
+            f"{r['GBps']:.0f} GB/s = {100*r['GBps']/HBM_PEAK_GBS:.1f}% HBM")
+        out.append(r)
+    return out
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -356,6 +385,7 @@ def main():
             w5 = None
             torch.cuda.empty_cache()
         extra.append(sched_bench(synth, ea))
+        extra.extend(rope_bench(torch, ea, synth))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)

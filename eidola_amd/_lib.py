@@ -95,7 +95,7 @@ class BatchInfo(C.Structure):
     ]
 
 
-EXPORTS = ("eid_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
+EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
            "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
                  "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
@@ -125,6 +125,9 @@ def load_library():
     P = C.c_void_p
     lib.eid_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, P, P, C.c_int32, P, P, P]
     lib.eid_kv_write.restype = C.c_int32
+    lib.eid_rope_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, C.c_int32, P, P, P, P,
+                                      C.c_int32, P, P, P]
+    lib.eid_rope_kv_write.restype = C.c_int32
     for name in ("eid_attn_decode", "eid_attn_varlen", "eid_lse_merge"):
         fn = getattr(lib, name)
         fn.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs), P]

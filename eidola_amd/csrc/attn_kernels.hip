@@ -1019,6 +1019,82 @@ __global__ __launch_bounds__(128) void kv_write_kernel(const uint16_t *__restric
 }
 
 // ---------------------------------------------------------------------------------------
+// Fused rotary embedding + QKV split + slot-mapped KV write: the step in front of the
+// attention path.  grid = num_tokens, block = 4 * (Hq + 2 Hkv) threads: a thread takes 8
+// dims d..d+7 and their partners d+32.. of one head row (the half-split rotation pairs
+// dim i with dim i + 32), so it moves two 16-byte pieces in and two out.
+//   o1 = fma(-x2, sin, x1 * cos),  o2 = fma(x1, sin, x2 * cos)      (fp32, one rounding each
+//   for the product and the fused step), rounded to bf16 nearest-even; K rows then go into
+//   the cache exactly as kv_write_kernel stores a bf16 row (bit copy, or fp8 quantisation
+//   of the bf16-rounded value), V rows are moved without rotation.
+// ---------------------------------------------------------------------------------------
+template <bool FP8>
+__global__ __launch_bounds__(1024) void rope_kv_write_kernel(
+    const uint16_t *__restrict__ qkv, const int32_t *__restrict__ positions,
+    const float *__restrict__ cos_sin, const int max_pos, uint16_t *__restrict__ q_out,
+    uint8_t *__restrict__ k_cache, uint8_t *__restrict__ v_cache,
+    const int64_t *__restrict__ slot_mapping, const float *__restrict__ k_scale,
+    const float *__restrict__ v_scale, const int Hq, const int Hkv, const int64_t num_slots) {
+  const int t = blockIdx.x;
+  const int head = threadIdx.x >> 2, piece = threadIdx.x & 3;  // head row of [q | k | v]
+  const size_t row = (size_t)(Hq + 2 * Hkv) * kHeadDim;
+  const uint16_t *src = qkv + (size_t)t * row + (size_t)head * kHeadDim + 8 * piece;
+  const u32x4 r1 = *(const u32x4 *)src, r2 = *(const u32x4 *)(src + 32);
+  const bool is_v = head >= Hq + Hkv;
+  u32x4 o1 = r1, o2 = r2;
+  if (!is_v) {
+    const int pos = min(max(positions[t], 0), max_pos - 1);  // out-of-range stays in the table
+    const float *cs = cos_sin + (size_t)pos * kHeadDim + 8 * piece;
+    float c[8], sn[8];
+    *(f32x4 *)&c[0] = *(const f32x4 *)cs;
+    *(f32x4 *)&c[4] = *(const f32x4 *)(cs + 4);
+    *(f32x4 *)&sn[0] = *(const f32x4 *)(cs + 32);
+    *(f32x4 *)&sn[4] = *(const f32x4 *)(cs + 36);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float a[2], b[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const float x1 = bf16_bits_to_f32((r1[j] >> (16 * h)) & 0xffffu);
+        const float x2 = bf16_bits_to_f32((r2[j] >> (16 * h)) & 0xffffu);
+        const float cc = c[2 * j + h], ss = sn[2 * j + h];
+        a[h] = __builtin_fmaf(-x2, ss, __fmul_rn(x1, cc));
+        b[h] = __builtin_fmaf(x1, ss, __fmul_rn(x2, cc));
+      }
+      o1[j] = pack_bf16(a[0], a[1]);
+      o2[j] = pack_bf16(b[0], b[1]);
+    }
+  }
+  if (head < Hq) {
+    uint16_t *dst = q_out + ((size_t)t * Hq + head) * kHeadDim + 8 * piece;
+    *(u32x4 *)dst = o1;
+    *(u32x4 *)(dst + 32) = o2;
+    return;
+  }
+  const int64_t slot = slot_mapping[t];
+  if (slot < 0 || slot >= num_slots) return;
+  const int kh = is_v ? head - Hq - Hkv : head - Hq;
+  uint8_t *cache = is_v ? v_cache : k_cache;
+  const size_t elem = ((size_t)slot * Hkv + kh) * kHeadDim + 8 * piece;
+  if constexpr (FP8) {
+    const float sc = (is_v ? v_scale : k_scale)[kh];
+    u32x2 q1 = {0, 0}, q2 = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float x1 = __fdiv_rn(bf16_bits_to_f32((o1[j >> 1] >> ((j & 1) * 16)) & 0xffffu), sc);
+      const float x2 = __fdiv_rn(bf16_bits_to_f32((o2[j >> 1] >> ((j & 1) * 16)) & 0xffffu), sc);
+      q1[j >> 2] |= fp8_e4m3_encode(x1) << ((j & 3) * 8);
+      q2[j >> 2] |= fp8_e4m3_encode(x2) << ((j & 3) * 8);
+    }
+    *(u32x2 *)(cache + elem) = q1;
+    *(u32x2 *)(cache + elem + 32) = q2;
+  } else {
+    *(u32x4 *)(cache + elem * 2) = o1;
+    *(u32x4 *)(cache + (elem + 32) * 2) = o2;
+  }
+}
+
+// ---------------------------------------------------------------------------------------
 // Host-side launchers (called from the C ABI after validation).
 // ---------------------------------------------------------------------------------------
 // Workgroups of kernel `fn` the whole device holds at once (cached per instantiation),
@@ -1169,6 +1245,24 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
 hipError_t launch_merge(const AttnParams &p, hipStream_t st) {
   dim3 grid(p.num_q_heads / 4, p.num_seqs * p.ws_rows);
   lse_merge_kernel<<<grid, 256, 0, st>>>(p);
+  return hipGetLastError();
+}
+
+hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
+                                const float *cos_sin, int max_pos, uint16_t *q_out,
+                                uint8_t *k_cache, uint8_t *v_cache, const int64_t *slot_mapping,
+                                const float *k_scale, const float *v_scale, int Hq, int Hkv,
+                                int64_t num_slots, int num_tokens, bool fp8, hipStream_t st) {
+  if (num_tokens == 0) return hipSuccess;
+  const int block = 4 * (Hq + 2 * Hkv);
+  if (fp8)
+    rope_kv_write_kernel<true><<<num_tokens, block, 0, st>>>(qkv, positions, cos_sin, max_pos,
+                                                            q_out, k_cache, v_cache, slot_mapping,
+                                                            k_scale, v_scale, Hq, Hkv, num_slots);
+  else
+    rope_kv_write_kernel<false><<<num_tokens, block, 0, st>>>(qkv, positions, cos_sin, max_pos,
+                                                             q_out, k_cache, v_cache, slot_mapping,
+                                                             k_scale, v_scale, Hq, Hkv, num_slots);
   return hipGetLastError();
 }
 

@@ -14,6 +14,11 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
 int splitkv_fill(int ntiles, bool fp8, int Hkv);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
+hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
+                                const float *cos_sin, int max_pos, uint16_t *q_out,
+                                uint8_t *k_cache, uint8_t *v_cache, const int64_t *slot_mapping,
+                                const float *k_scale, const float *v_scale, int Hq, int Hkv,
+                                int64_t num_slots, int num_tokens, bool fp8, hipStream_t st);
 hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
                            uint8_t *v_cache, const int64_t *slot_mapping, const float *k_scale,
                            const float *v_scale, int Hkv, int64_t num_slots, int num_tokens,
@@ -226,6 +231,36 @@ int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v
       v_scale, desc->num_kv_heads, desc->num_blocks * desc->block_size, num_tokens, fp8,
       static_cast<hipStream_t>(hip_stream));
   if (e != hipSuccess) return hip_fail(e, "kv_write launch");
+  return EID_OK;
+}
+
+int32_t eid_rope_kv_write(const eid_attn_desc *desc, const void *qkv, const int32_t *positions,
+                          const float *cos_sin, int32_t max_pos, void *q_out, void *k_cache,
+                          void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
+                          const float *k_scale, const float *v_scale, void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_geometry(desc)) return rc;
+  if (4 * (desc->num_q_heads + 2 * desc->num_kv_heads) > 1024)
+    return fail(EID_ERR_UNSUPPORTED, "num_kv_heads %d too large for one workgroup per token",
+                desc->num_kv_heads);
+  if (num_tokens < 0) return fail(EID_ERR_INVALID_ARG, "num_tokens %d < 0", num_tokens);
+  if (max_pos <= 0) return fail(EID_ERR_INVALID_ARG, "max_pos %d must be positive", max_pos);
+  if (num_tokens == 0) return EID_OK;
+  if (!qkv || !positions || !cos_sin || !q_out || !k_cache || !v_cache || !slot_mapping)
+    return fail(EID_ERR_INVALID_ARG,
+                "qkv, positions, cos_sin, q_out, k_cache, v_cache, slot_mapping must be non-NULL");
+  if (!aligned16(qkv) || !aligned16(cos_sin) || !aligned16(q_out) || !aligned16(k_cache) ||
+      !aligned16(v_cache))
+    return fail(EID_ERR_INVALID_ARG, "qkv, cos_sin, q_out, k_cache and v_cache must be 16-byte aligned");
+  const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  if (fp8 && (!k_scale || !v_scale)) return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
+  hipError_t e = eid::launch_rope_kv_write(
+      static_cast<const uint16_t *>(qkv), positions, cos_sin, max_pos,
+      static_cast<uint16_t *>(q_out), static_cast<uint8_t *>(k_cache),
+      static_cast<uint8_t *>(v_cache), slot_mapping, k_scale, v_scale, desc->num_q_heads,
+      desc->num_kv_heads, desc->num_blocks * desc->block_size, num_tokens, fp8,
+      static_cast<hipStream_t>(hip_stream));
+  if (e != hipSuccess) return hip_fail(e, "rope_kv_write launch");
   return EID_OK;
 }
 

@@ -117,6 +117,66 @@ def kv_write(geom, k_new, v_new, k_cache, v_cache, slot_mapping, k_scale=None, v
                                       _ptr(v_scale), _stream()))
 
 
+def rope_kv_write(geom, qkv, positions, cos_sin, k_cache, v_cache, slot_mapping, k_scale=None,
+                  v_scale=None, q_out=None):
+    """Fused RoPE + QKV split + slot-mapped KV write.  qkv is [T, (Hq + 2 Hkv) * D] bf16,
+    cos_sin [max_pos, D] fp32 (per position D/2 cosines then D/2 sines); returns q_out
+    [T, Hq, D] bf16."""
+    _require(qkv, "qkv", torch.bfloat16, 2)
+    _require(positions, "positions", torch.int32, 1)
+    _require(cos_sin, "cos_sin", torch.float32, 2)
+    k_cache = _cache_view(k_cache, geom, "k_cache")
+    v_cache = _cache_view(v_cache, geom, "v_cache")
+    _require(slot_mapping, "slot_mapping", torch.int64, 1)
+    T = qkv.shape[0]
+    if qkv.shape[1] != (geom.num_q_heads + 2 * geom.num_kv_heads) * geom.head_dim:
+        raise ValueError("qkv must be [T, (num_q_heads + 2 num_kv_heads) * head_dim]")
+    if positions.shape[0] != T or slot_mapping.shape[0] != T:
+        raise ValueError("positions and slot_mapping must have one entry per token")
+    if cos_sin.shape[1] != geom.head_dim:
+        raise ValueError("cos_sin must be [max_pos, head_dim]")
+    if geom.kv_dtype == KV_FP8_E4M3:
+        _require(k_scale, "k_scale", torch.float32, 1)
+        _require(v_scale, "v_scale", torch.float32, 1)
+    if q_out is None:
+        q_out = torch.empty((T, geom.num_q_heads, geom.head_dim), dtype=torch.bfloat16,
+                            device=qkv.device)
+    else:
+        _require(q_out, "q_out", torch.bfloat16, 3)
+    desc = make_desc(geom, num_seqs=1, num_q_tokens=1, max_q_len=1, max_kv_len=1,
+                     max_blocks_per_seq=1, num_blocks=k_cache.shape[0])
+    check(load_library().eid_rope_kv_write(
+        C.byref(desc), _ptr(qkv), _ptr(positions), _ptr(cos_sin), cos_sin.shape[0], _ptr(q_out),
+        _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), T, _ptr(k_scale), _ptr(v_scale),
+        _stream()))
+    return q_out
+
+
+def yarn_cos_sin(max_pos, head_dim=64, base=150000.0, scaling_factor=32.0,
+                 initial_context=4096.0, ntk_alpha=1.0, ntk_beta=32.0):
+    """[max_pos, head_dim] fp32 table for eid_rope_kv_write (numpy): per position head_dim/2
+    cosines then head_dim/2 sines with YaRN "NTK-by-parts" frequency blending and the
+    attention-temperature factor 0.1 ln(scaling_factor) + 1 folded in, as the published
+    gpt-oss model definition describes its rotary embedding (defaults are that model's
+    configuration).  scaling_factor <= 1 gives plain RoPE."""
+    import numpy as np
+    half = head_dim // 2
+    freq = base ** (np.arange(0, head_dim, 2, dtype=np.float64) / head_dim)
+    if scaling_factor > 1.0:
+        concentration = 0.1 * np.log(scaling_factor) + 1.0
+        low = half * np.log(initial_context / (ntk_beta * 2 * np.pi)) / np.log(base)
+        high = half * np.log(initial_context / (ntk_alpha * 2 * np.pi)) / np.log(base)
+        ramp = (np.arange(half, dtype=np.float64) - low) / (high - low)
+        mask = 1.0 - np.clip(ramp, 0.0, 1.0)
+        inv_freq = (1.0 / (scaling_factor * freq)) * (1.0 - mask) + (1.0 / freq) * mask
+    else:
+        concentration = 1.0
+        inv_freq = 1.0 / freq
+    ang = np.arange(max_pos, dtype=np.float64)[:, None] * inv_freq[None, :]
+    return np.concatenate([np.cos(ang) * concentration, np.sin(ang) * concentration],
+                          axis=1).astype(np.float32)
+
+
 def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q,
                max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace,
                return_lse, sum_kv_len=0):

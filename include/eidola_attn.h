@@ -121,6 +121,29 @@ int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v
                      void *hip_stream);
 
 /*
+ * The step in front of K1, fused with it: rotary embedding of q and k (half-split pairing,
+ * dim i with dim i + 32), split of the projection output into q / k / v, and the slot-mapped
+ * KV write, in one pass over the new tokens.
+ *   qkv        [num_tokens, (Hq + 2 Hkv) * 64] bf16: per token the q heads, then the k heads,
+ *              then the v heads
+ *   positions  [num_tokens] int32, absolute position of each token; values outside
+ *              [0, max_pos) are clamped into the table
+ *   cos_sin    [max_pos, 64] fp32: per position 32 cosines then 32 sines, already multiplied
+ *              by whatever attention-temperature factor the model's RoPE scaling prescribes
+ *   q_out      [num_tokens, Hq, 64] bf16
+ * Arithmetic (fixed, so that results are reproducible bit for bit): with x1 = x[i],
+ * x2 = x[i + 32] in fp32, o[i] = fma(-x2, sin_i, x1 * cos_i), o[i + 32] = fma(x1, sin_i,
+ * x2 * cos_i), each rounded to bf16 nearest-even; the rotated k row and the v row are then
+ * stored exactly as eid_kv_write stores a bf16 row (fp8: quantised from the bf16 value).
+ * Tokens with slot -1 still produce q_out.  Reference counterpart: none.  Engine call site:
+ * once per layer per step after the QKV projection, instead of a RoPE kernel + eid_kv_write.
+ */
+int32_t eid_rope_kv_write(const eid_attn_desc *desc, const void *qkv, const int32_t *positions,
+                          const float *cos_sin, int32_t max_pos, void *q_out, void *k_cache,
+                          void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
+                          const float *k_scale, const float *v_scale, void *hip_stream);
+
+/*
  * Stages K2+K4 — decode attention: every sequence contributes exactly one query row
  * (num_q_tokens == num_seqs, max_q_len == 1).  Split-KV over partitions of
  * `partition_size` tokens with the per-head sink folded into the denominator once, in

@@ -39,6 +39,9 @@ def lib():
         L.orc_fp8_e4m3_decode.restype = C.c_float
         L.orc_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, P, P, C.c_int32, P, P]
         L.orc_kv_write.restype = C.c_int
+        L.orc_rope_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, C.c_int32, P, P, P, P,
+                                        C.c_int32, P, P]
+        L.orc_rope_kv_write.restype = C.c_int
         L.orc_attn_f64.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs), P, P]
         L.orc_attn_f64.restype = C.c_int
         L.orc_splitkv_partials_f64.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs),
@@ -98,6 +101,25 @@ def kv_write(desc, k_new, v_new, k_cache, v_cache, slot_mapping, k_scale=None, v
                             _p(sm), len(sm), _p(ks), _p(vs))
     if rc:
         raise ValueError("slot out of range")
+
+
+def rope_kv_write(desc, qkv, positions, cos_sin, k_cache, v_cache, slot_mapping, k_scale=None,
+                  v_scale=None):
+    """Fused RoPE + split + KV write; caches are updated in place, q_out [T,Hq,D] (bf16 bits)
+    is returned."""
+    qkv = _c(qkv, np.uint16)
+    pos = _c(positions, np.int32)
+    cs = _c(cos_sin, np.float32)
+    sm = _c(slot_mapping, np.int64)
+    ks, vs = _c(k_scale, np.float32), _c(v_scale, np.float32)
+    assert k_cache.flags.c_contiguous and v_cache.flags.c_contiguous
+    T = len(sm)
+    q_out = np.zeros((T, desc.num_q_heads, desc.head_dim), dtype=np.uint16)
+    rc = lib().orc_rope_kv_write(C.byref(desc), _p(qkv), _p(pos), _p(cs), cs.shape[0], _p(q_out),
+                                 _p(k_cache), _p(v_cache), _p(sm), T, _p(ks), _p(vs))
+    if rc:
+        raise ValueError("slot out of range")
+    return q_out
 
 
 def attn_f64(desc, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, sinks=None,

@@ -134,6 +134,62 @@ int orc_kv_write(const eid_attn_desc *d, const uint16_t *k_new, const uint16_t *
   return 0;
 }
 
+/* Fused rotary embedding + QKV split + KV write: same contract as eid_rope_kv_write
+ * (include/eidola_attn.h).  Half-split pairing (dim i with dim i + D/2); per pair, in fp32,
+ *   o1 = fma(-x2, sin, x1 * cos),  o2 = fma(x1, sin, x2 * cos),  each rounded to bf16 RNE;
+ * the rotated k row and the v row then go through orc_kv_write's rule.  Reference
+ * counterpart: none (the reference holds no model code).  `volatile` keeps the product a
+ * separately rounded fp32 value whatever the compiler's contraction settings are. */
+int orc_rope_kv_write(const eid_attn_desc *d, const uint16_t *qkv, const int32_t *positions,
+                      const float *cos_sin, int32_t max_pos, uint16_t *q_out, void *k_cache,
+                      void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
+                      const float *k_scale, const float *v_scale) {
+  const int Hq = d->num_q_heads, Hkv = d->num_kv_heads, D = d->head_dim, half = D / 2;
+  const int64_t nslots = d->num_blocks * d->block_size;
+  const size_t row = (size_t)(Hq + 2 * Hkv) * D;
+  for (int t = 0; t < num_tokens; t++) {
+    int pos = positions[t];
+    if (pos < 0) pos = 0;
+    if (pos > max_pos - 1) pos = max_pos - 1;
+    const float *cs = cos_sin + (size_t)pos * D;
+    const int64_t slot = slot_mapping[t];
+    if (slot >= nslots) return -1;
+    for (int h = 0; h < Hq + 2 * Hkv; h++) {
+      const uint16_t *src = qkv + (size_t)t * row + (size_t)h * D;
+      uint16_t o[256];
+      if (h < Hq + Hkv) {
+        for (int i = 0; i < half; i++) {
+          const float x1 = orc_bf16_to_f32(src[i]), x2 = orc_bf16_to_f32(src[i + half]);
+          volatile float p1 = x1 * cs[i], p2 = x2 * cs[i];
+          o[i] = orc_f32_to_bf16(fmaf(-x2, cs[half + i], p1));
+          o[i + half] = orc_f32_to_bf16(fmaf(x1, cs[half + i], p2));
+        }
+      } else {
+        memcpy(o, src, (size_t)D * sizeof(uint16_t));
+      }
+      if (h < Hq) {
+        memcpy(q_out + ((size_t)t * Hq + h) * D, o, (size_t)D * sizeof(uint16_t));
+        continue;
+      }
+      if (slot < 0) continue;
+      const int is_v = h >= Hq + Hkv;
+      const int kh = is_v ? h - Hq - Hkv : h - Hq;
+      void *cache = is_v ? v_cache : k_cache;
+      const float *scale = is_v ? v_scale : k_scale;
+      for (int x = 0; x < D; x++) {
+        const size_t dst = ((size_t)slot * Hkv + kh) * D + x;
+        if (d->kv_dtype == EID_KV_FP8_E4M3) {
+          volatile float qv = orc_bf16_to_f32(o[x]) / scale[kh];
+          ((uint8_t *)cache)[dst] = orc_fp8_e4m3_encode(qv);
+        } else {
+          ((uint16_t *)cache)[dst] = o[x];
+        }
+      }
+    }
+  }
+  return 0;
+}
+
 /* ------------------------------------------------------------------ definitional fp64 */
 
 /*  s_j = scale * <q, k_j> (* k_scale);  m = max(max_j s_j, sink);

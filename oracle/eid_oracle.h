@@ -37,6 +37,13 @@ int orc_kv_write(const eid_attn_desc *d, const uint16_t *k_new, const uint16_t *
                  void *k_cache, void *v_cache, const int64_t *slot_mapping,
                  int32_t num_tokens, const float *k_scale, const float *v_scale);
 
+/* Fused RoPE + QKV split + KV write: same contract as eid_rope_kv_write.  Returns 0, or -1
+ * on an out-of-range slot. */
+int orc_rope_kv_write(const eid_attn_desc *d, const uint16_t *qkv, const int32_t *positions,
+                      const float *cos_sin, int32_t max_pos, uint16_t *q_out, void *k_cache,
+                      void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
+                      const float *k_scale, const float *v_scale);
+
 /* Definitional attention in fp64 from the stored bf16/fp8 bits.
  * out64: [T, Hq, D] doubles; lse64: [T, Hq] doubles or NULL.
  * cu_seqlens_q may be NULL (then q_len = 1 for every sequence). */
