@@ -74,11 +74,11 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
       vf[mt][pr].w[2] = b2[0];
       vf[mt][pr].w[3] = b2[1];
     }
-  // S^T = K Q^T (raw scores, fp32).  With four row tiles the scores of tile nt + 1 are
-  // issued before the softmax of tile nt, so that the matrix pipe has work while the
-  // vector ALU runs the softmax.
-  constexpr bool kPipe = false;  // (four-tile pipelining needs 16 more VGPRs than the prefill kernel has)
-  auto scores = [&](const int nt, f32x4 (&S)[4]) {
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    // S^T = K Q^T (raw scores, fp32); the prefill kernel raises its priority around MFMA
+    // clusters so that the matrix pipe is fed first when both of a SIMD's waves are ready
+    f32x4 S[4];
     if (NT == 4) __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -87,19 +87,6 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
       S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
     }
     if (NT == 4) __builtin_amdgcn_s_setprio(0);
-  };
-  f32x4 Snext[4];
-  if (kPipe) scores(0, Snext);
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    f32x4 S[4];
-    if (kPipe) {
-#pragma unroll
-      for (int b = 0; b < 4; ++b) S[b] = Snext[b];
-      if (nt + 1 < NT) scores(nt + 1, Snext);
-    } else {
-      scores(nt, S);
-    }
     if (need_mask) {
       int pos, lo;
       ri.bounds(nt, pos, lo);
@@ -645,6 +632,93 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   // the merge launch that follows reads the partition from here instead of re-deriving it
   if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
   splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds);
+}
+
+// ---------------------------------------------------------------------------------------
+// Short-span kernel: when no sequence spans more than 8 chunks (sliding-window layers, short
+// contexts) a sequence is too short to be worth partitioning across workgroups, and one
+// wave walking its 2-3 chunks one after the other is pure latency.  Here a workgroup owns
+// one (sequence, KV head) and its 8 waves take one 64-token chunk each, all in flight at
+// once; the eight (m, l, acc) partials meet in LDS (each wave's V staging area is reused for
+// its fp32 accumulators) and the 512 threads combine them with the sink and write the
+// output.  grid = (num_seqs, Hkv); sequences of another q_len class leave at once.
+// ---------------------------------------------------------------------------------------
+constexpr int kShortWaves = 8;
+constexpr int kShortSpanMax = kShortWaves * kChunk;
+
+template <int NT, bool FP8>
+__global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan_kernel(const AttnParams p) {
+  constexpr int kRows = NT * 16;
+  constexpr int kPartBytes = kRows * kHeadDim * 4;  // one wave's fp32 accumulators
+  constexpr int kWaveBytes = kPartBytes > kWaveLdsBytes ? kPartBytes : kWaveLdsBytes;
+  __shared__ __align__(16) uint8_t lds[kShortWaves * kWaveBytes];
+  __shared__ float ml_lds[kShortWaves][kRows][2];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i16 = lane & 15, g = lane >> 4;
+  const int s = blockIdx.x, kvh = blockIdx.y;
+  const SeqView v = view_seq(p, s);
+  if (v.span <= 0) return;  // not of this class, or malformed: the whole workgroup leaves
+  const int L = v.seq_len, qlen = v.qlen, row0 = v.row0;
+  const int kb = kv_begin(L, qlen, p.window);
+  const int pos0 = L - qlen;
+  const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
+  const int nw = min(kShortWaves, (L - kb + kChunk - 1) / kChunk);  // waves with a chunk
+  const int t0 = kb + wave * kChunk;
+  if (wave < nw) {
+    Frag8 qf[NT][2];
+    RowInfo ri;
+    load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
+    float m[NT];
+    f32x4 lacc[NT], acc[NT][4];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      m[nt] = kNegBig;
+      lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    uint8_t *mine = lds + wave * kWaveBytes;
+    attend<NT, FP8>(p, s, kvh, t0, min(t0 + kChunk, L), L, pos0, lo_last, qf, ri, mine, m, lacc, acc);
+    // the V tile is consumed: the same bytes now carry this wave's accumulators, row-major
+    float *part = reinterpret_cast<float *>(mine);
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+        *(f32x4 *)(part + (nt * 16 + i16) * kHeadDim + 16 * mt + 4 * g) = acc[nt][mt];
+      if (g == 0) {
+        ml_lds[wave][nt * 16 + i16][0] = m[nt];
+        ml_lds[wave][nt * 16 + i16][1] = lacc[nt][0];
+      }
+    }
+  }
+  __syncthreads();
+  // combine: 32 threads per row, two dims each
+  const float vs = FP8 ? p.v_scale[kvh] : 1.0f;
+  const int d2 = (tid & 31) * 2;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int r = nt * 16 + (tid >> 5);
+    const int t = r >> 3;
+    if (t >= qlen) continue;
+    const int head = kvh * kGroup + (r & 7);
+    const float sink2 = p.sinks ? p.sinks[head] * kLog2e : -INFINITY;
+    float M = sink2;
+    for (int w = 0; w < nw; ++w) M = fmaxf(M, ml_lds[w][r][0]);
+    float den = fast_exp2(sink2 - M), o0 = 0.f, o1 = 0.f;
+    for (int w = 0; w < nw; ++w) {
+      const float wgt = fast_exp2(ml_lds[w][r][0] - M);
+      den += wgt * ml_lds[w][r][1];
+      const float2 a = *(const float2 *)(lds + w * kWaveBytes + ((size_t)r * kHeadDim + d2) * 4);
+      o0 += wgt * a.x;
+      o1 += wgt * a.y;
+    }
+    const float inv = vs / den;
+    const size_t orow = (size_t)(row0 + t) * p.num_q_heads + head;
+    *(uint32_t *)(p.out + orow * kHeadDim + d2) = pack_bf16(o0 * inv, o1 * inv);
+    if (p.lse && d2 == 0) p.lse[orow] = (M + __log2f(den)) * kLn2;
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1208,6 +1282,32 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
 
 // Item count of the one-workgroup-per-CU tier of the run-time partition rule.
 static int fill_lo(int target_items) { return min(target_items, device_cus()); }
+
+// Short-span launch: see shortspan_kernel.  The caller has checked that no sequence spans
+// more than kShortSpanMax tokens.
+hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
+  dim3 grid(p.num_seqs, p.num_kv_heads);
+  if (fp8) {
+    if (ntiles == 1) shortspan_kernel<1, true><<<grid, kShortWaves * 64, 0, st>>>(p);
+    else shortspan_kernel<3, true><<<grid, kShortWaves * 64, 0, st>>>(p);
+  } else {
+    if (ntiles == 1) shortspan_kernel<1, false><<<grid, kShortWaves * 64, 0, st>>>(p);
+    else shortspan_kernel<3, false><<<grid, kShortWaves * 64, 0, st>>>(p);
+  }
+  return hipGetLastError();
+}
+// Whether the short-span kernel should serve a launch: spans within its reach, and no more
+// workgroups (one per sequence and KV head) than the device holds at once; beyond that the
+// split-KV kernel's one workgroup per sequence makes fewer, better filled rounds.
+bool shortspan_applies(int ntiles, bool fp8, int num_seqs, int Hkv, int max_span) {
+  if (max_span > kShortSpanMax) return false;
+  static const int fill[2][2] = {
+      {device_fill(shortspan_kernel<1, false>, kShortWaves * 64),
+       device_fill(shortspan_kernel<1, true>, kShortWaves * 64)},
+      {device_fill(shortspan_kernel<3, false>, kShortWaves * 64),
+       device_fill(shortspan_kernel<3, true>, kShortWaves * 64)}};
+  return (long long)num_seqs * Hkv <= fill[ntiles == 1 ? 0 : 1][fp8 ? 1 : 0];
+}
 
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same

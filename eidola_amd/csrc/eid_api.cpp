@@ -12,6 +12,8 @@
 namespace eid {
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st);
 int splitkv_fill(int ntiles, bool fp8, int Hkv);
+hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
+bool shortspan_applies(int ntiles, bool fp8, int num_seqs, int Hkv, int max_span);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
 hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
@@ -279,7 +281,11 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  hipError_t e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
+  // spans of at most 8 chunks: one workgroup per (sequence, KV head), a chunk per wave
+  const bool short_span = pl.nparts_max == 1 &&
+      eid::shortspan_applies(1, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
+  hipError_t e = short_span ? eid::launch_shortspan(p, 1, fp8, st)
+                            : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (args->split_done_event) {
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
@@ -308,13 +314,18 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= eid::kShortQMax;
   const bool only_prefill = uniform && desc->max_q_len > eid::kShortQMax;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
+  const bool short1 = pl.nparts_max == 1 &&
+      eid::shortspan_applies(1, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
+  const bool short3 = pl.nparts_max == 1 &&
+      eid::shortspan_applies(3, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
   if (!only_verify && !only_prefill) {
     p.qlen_lo = 1;
     p.qlen_hi = 2;
     p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
-    e = eid::launch_splitkv(p, 1, fp8, plan_slots, st);
+    e = short1 ? eid::launch_shortspan(p, 1, fp8, st)
+               : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
     if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   }
   if (args->split_done_event) {
@@ -329,7 +340,8 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     p.qlen_lo = 3;
     p.qlen_hi = eid::kShortQMax;
     p.target_items = eid::splitkv_fill(3, fp8, desc->num_kv_heads);
-    e = eid::launch_splitkv(p, 3, fp8, plan_slots + 2, st);
+    e = short3 ? eid::launch_shortspan(p, 3, fp8, st)
+               : eid::launch_splitkv(p, 3, fp8, plan_slots + 2, st);
     if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
     if (pl.nparts_max > 1) {
       e = eid::launch_merge(p, st);
