@@ -285,6 +285,50 @@ def test_fp8_kv_attention(G, q_len):
     assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs), ref, f"fp8 q_len={q_len}")
 
 
+# ---------------------------------------------------------------- short-span kernel
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+@pytest.mark.parametrize("window,seq_lens,q_lens", [
+    (128, [1, 15, 16, 17, 129, 400, 1500, 3000], [1] * 8),            # windowed decode
+    (0, [1, 63, 64, 65, 300, 511, 512, 7], [1, 1, 1, 1, 1, 1, 1, 2]), # short contexts, 8 chunks
+    (40, [200, 77, 90, 1000], [5, 3, 6, 4]),                          # verify rows, windowed
+    (64, [300, 50, 900, 12, 640], [1, 5, 2, 6, 1]),                   # classes mixed
+])
+def test_short_spans_one_chunk_per_wave(G, kv_dtype, window, seq_lens, q_lens):
+    """No sequence spans more than 8 chunks and the batch is small: the attention entry
+    points take the kernel that gives every wave one chunk and merges in LDS.  Outputs and
+    lse against the oracle, for both cache types and every q_len class."""
+    b = make_batch(seq_lens, q_lens, window=window, kv_dtype=kv_dtype)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True)
+    assert_close(out, ref, f"short spans w={window}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+def test_short_span_and_split_kv_kernels_agree_across_the_fill_boundary(G):
+    """64 windowed decodes fill the device exactly at one workgroup per (sequence, KV head);
+    65 fall back to the split-KV kernel.  The first 64 rows must agree between the two."""
+    rng = np.random.default_rng(8)
+    L = rng.integers(1, 2000, size=65)
+    b65 = make_batch(L, [1] * 65, window=128, seed=4)
+    q, k, v, sinks = logical_tensors(b65)
+    kc_d, vc_d = G.gpu_caches(b65, k, v)
+    o65 = G.run_attn(b65, q, kc_d, vc_d, sinks)
+    b64 = make_batch(L[:64], [1] * 64, window=128, seed=4)
+    b64.block_table[:] = b65.block_table[:64]
+    o64 = G.run_attn(b64, q[:64], kc_d, vc_d, sinks)
+    a = synth.bf16_bits_to_f32(o64).astype(np.float64)
+    c = synth.bf16_bits_to_f32(o65[:64]).astype(np.float64)
+    assert np.abs(a - c).max() <= 4e-3
+    kc, vc = cpu_caches(b65, k, v)
+    ref, _ = oracle_out(b65, q, kc, vc, sinks)
+    assert_close(o65, ref, "65 windowed decodes")
+    assert_close(o64, ref[:64], "64 windowed decodes")
+
+
 def test_fp8_every_code_dequantises_exactly(G):
     """One-key attention returns v0 * sigmoid(s0 - sink): with a huge negative sink the
     output is the dequantised V row itself, for all 254 finite codes."""
