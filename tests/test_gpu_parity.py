@@ -411,6 +411,34 @@ def test_split_done_event_is_recorded_between_the_phases(G):
     assert 0.0 < e0.elapsed_time(e1) <= e0.elapsed_time(e2)
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_seeded_random_batches(G, seed):
+    """Random shapes across every dispatch decision at once: number of sequences, q_len
+    classes, context lengths, window, partition mode, cache type, launch hint."""
+    rng = np.random.default_rng(1000 + seed)
+    S = int(rng.integers(1, 41))
+    q_lens = rng.choice([1, 1, 1, 2, 3, 5, 6, 7, 20, 33, 64, 100], size=S)
+    ctx = rng.integers(0, int(rng.choice([60, 400, 3000])), size=S)
+    seq_lens = q_lens + ctx
+    window = int(rng.choice([0, 0, 16, 128, 500]))
+    partition = int(rng.choice([0, 0, 64, 256, 1024]))
+    kv_dtype = KV_FP8_E4M3 if rng.random() < 0.35 else KV_BF16
+    b = make_batch(seq_lens, q_lens, window=window, partition=partition, kv_dtype=kv_dtype,
+                   seed=seed)
+    q, k, v, sinks = logical_tensors(b)
+    if rng.random() < 0.2:
+        sinks = None
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True,
+                          hint=bool(rng.random() < 0.5))
+    what = f"seed {seed}: S={S} w={window} P={partition} dtype={kv_dtype} q={sorted(set(q_lens.tolist()))}"
+    assert_close(out, ref, what)
+    assert np.allclose(lse, ref_lse, atol=3e-3), what
+
+
 # ---------------------------------------------------------------- benchmark configurations
 def _sample_check(G, b, q_d, kc_d, vc_d, sinks, out_d, seqs, what, ks=None, vs=None):
     sub, kc, vc = G.compact_to_cpu(b, kc_d, vc_d, seqs)
