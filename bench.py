@@ -136,6 +136,39 @@ class Workload:
         self.attn[i % self.n]()
 
 
+def graph_step_ms(w, steps, torch):
+    """The same steps replayed from a HIP graph: all page sets' steps (kv_write + attention)
+    are captured once on a side stream and the graph is replayed, which removes the host's
+    launch cost from short steps.  Returns milliseconds per step, or None if capture fails."""
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(w.n):
+                w.step(i)                      # warm-up on the capture stream
+            side.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                for i in range(w.n):
+                    w.step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        reps = max(1, steps // w.n)
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / (reps * w.n)
+    except Exception as ex:  # capture is an extra; the eager numbers stand without it
+        log(f"[bench] graph capture unavailable: {ex}")
+        return None
+
+
 def measure(w, steps, warmup, torch, synth, label):
     b = w.batches[0]
     for i in range(warmup):
@@ -145,11 +178,12 @@ def measure(w, steps, warmup, torch, synth, label):
     ms_merge = event_ms(lambda i: w.merge[i % w.n](), steps, torch)
     ms_write = event_ms(w.kv_write, steps, torch)
     ms_split = split_kernel_ms(w, steps, torch)
+    ms_graph = graph_step_ms(w, steps, torch)
     work = synth.algorithmic_work(b)
     work_w = synth.algorithmic_work(b, include_kv_write=True)
     r = {
         "config": label, "ms_per_step": ms_step, "ms_attn": ms_attn, "ms_merge": ms_merge,
-        "ms_kv_write": ms_write, "ms_split": ms_split, "alg_bytes": work["bytes"], "alg_flops": work["flops"],
+        "ms_kv_write": ms_write, "ms_split": ms_split, "ms_per_step_graph": ms_graph, "alg_bytes": work["bytes"], "alg_flops": work["flops"],
         "q_tokens": work["q_tokens"], "ctx_tokens": work["ctx_tokens"],
         "step_GBps": work_w["bytes"] / ms_step / 1e6,
         "attn_GBps": work["bytes"] / ms_attn / 1e6,
@@ -161,7 +195,8 @@ def measure(w, steps, warmup, torch, synth, label):
     # (meaningless when no sequence of the first class ran: reported as None)
     part = int(w.attn[0]._keep[-1][:4].view(torch.int32).item())
     r["partition"] = part if 64 <= part <= 4096 and part % 64 == 0 else None
-    log(f"[bench] {label}: step {ms_step*1e3:.1f} us (attn {ms_attn*1e3:.1f}, split-KV "
+    gtxt = f", graph replay {ms_graph*1e3:.1f}" if ms_graph else ""
+    log(f"[bench] {label}: step {ms_step*1e3:.1f} us{gtxt} (attn {ms_attn*1e3:.1f}, split-KV "
         f"{ms_split*1e3:.1f}, merge {ms_merge*1e3:.1f}, kv_write {ms_write*1e3:.1f}); attn {r['attn_GBps']:.0f} GB/s = "
         f"{100*r['attn_GBps']/HBM_PEAK_GBS:.1f}% HBM, {r['attn_TFLOPs']:.1f} TFLOP/s; "
         f"partition {r['partition']}")

@@ -551,3 +551,45 @@ def test_config5_verify_full_size(G, layer):
     order = np.argsort(b.seq_lens)
     _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [int(order[0]), int(order[64]), int(order[-1])],
                   f"config5 layer {layer}")
+
+
+def test_step_replayed_from_a_hip_graph(G):
+    """kv_write + decode attention captured into a HIP graph and replayed: every replay must
+    reproduce the eager result bit for bit, with eager work and synchronisations in between
+    (the library enqueues kernels only: no memset nodes, no allocation)."""
+    b = make_batch([700, 33, 2500, 129], [1, 1, 1, 1])
+    q, k, v, sinks = logical_tensors(b)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    k_new = G.bf16_dev(synth.normal_bf16((4, 8, 64), 77, synth.TID_K))
+    v_new = G.bf16_dev(synth.normal_bf16((4, 8, 64), 77, synth.TID_V))
+    slots = G.dev(np.array([b.all_slots(s)[-1] for s in range(4)], dtype=np.int64))
+    call = ea.prepare("eid_attn_decode", b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table),
+                      G.dev(b.seq_lens), max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
+                      sum_kv_len=int(b.seq_lens.sum()))
+
+    def step():
+        ea.kv_write(b.geom, k_new, v_new, kc_d, vc_d, slots)
+        call()
+
+    step()
+    torch.cuda.synchronize()
+    eager = call.out.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for i in range(4):
+        call.out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(call.out, eager), f"replay {i}"
+        step()                      # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(call.out, eager)
