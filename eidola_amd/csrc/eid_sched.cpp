@@ -9,6 +9,7 @@
 //             ids of its partly filled last block (they are hashed when the block fills)
 #include <cstdarg>
 #include <cstdint>
+#include <algorithm>
 #include <cstring>
 #include <new>
 #include <unordered_map>
@@ -60,6 +61,7 @@ struct Seq {
   uint64_t chain = kRootHash;  // hash of the last full block while `chained`
   bool chained = true;         // every full block so far has been hashed
   std::vector<int32_t> tail;   // token ids of the partly filled last block
+  uint64_t stamp = 0;          // eid_sched::stamp of the last build_batch call that listed it
 };
 
 }  // namespace
@@ -72,6 +74,7 @@ struct eid_sched {
   std::vector<Block> blocks;
   std::vector<int32_t> block_tokens;  // [nblocks][bs], prefix reuse only
   int64_t free_head = -1, free_tail = -1, free_count = 0;
+  uint64_t stamp = 0;  // build_batch call counter
   std::unordered_map<uint64_t, int64_t> index;
   std::unordered_map<int64_t, Seq> seqs;
 
@@ -134,12 +137,17 @@ int32_t eid_sched_create(const eid_sched_config *cfg, eid_sched **out) {
   if (cfg->max_blocks_per_seq <= 0) return fail(EID_ERR_INVALID_ARG, "max_blocks_per_seq must be positive");
   eid_sched *s = new (std::nothrow) eid_sched;
   if (!s) return fail(EID_ERR_INVALID_ARG, "out of host memory");
-  s->bs = cfg->block_size;
-  s->nblocks = cfg->num_blocks;
-  s->max_blocks_per_seq = cfg->max_blocks_per_seq;
-  s->reuse = cfg->prefix_reuse != 0;
-  s->blocks.resize((size_t)s->nblocks);
-  if (s->reuse) s->block_tokens.assign((size_t)s->nblocks * s->bs, 0);
+  try {  // no C++ exception may cross the C ABI
+    s->bs = cfg->block_size;
+    s->nblocks = cfg->num_blocks;
+    s->max_blocks_per_seq = cfg->max_blocks_per_seq;
+    s->reuse = cfg->prefix_reuse != 0;
+    s->blocks.resize((size_t)s->nblocks);
+    if (s->reuse) s->block_tokens.assign((size_t)s->nblocks * s->bs, 0);
+  } catch (...) {
+    delete s;
+    return fail(EID_ERR_INVALID_ARG, "out of host memory for %lld blocks", (long long)cfg->num_blocks);
+  }
   for (int64_t b = 0; b < s->nblocks; ++b) s->free_push_back(b);
   *out = s;
   return EID_OK;
@@ -154,6 +162,12 @@ int32_t eid_sched_add_seq(eid_sched *s, int64_t seq_id, const int32_t *prompt, i
   if (n < 0) return fail(EID_ERR_INVALID_ARG, "prompt length %d is negative", n);
   if (s->seqs.count(seq_id)) return fail(EID_ERR_INVALID_ARG, "sequence %lld already exists", (long long)seq_id);
   Seq q;
+  try {  // every allocation happens before the first block reference is taken
+    q.blocks.reserve((size_t)std::min<int64_t>(s->max_blocks_per_seq, (int64_t)n / s->bs + 1));
+    q.tail.reserve((size_t)s->bs);
+  } catch (...) {
+    return fail(EID_ERR_INVALID_ARG, "out of host memory");
+  }
   if (s->reuse && prompt && n > 1) {
     const int max_match = (n - 1) / s->bs;  // at least one token stays to be computed
     for (int b = 0; b < max_match && b < s->max_blocks_per_seq; ++b) {
@@ -169,8 +183,17 @@ int32_t eid_sched_add_seq(eid_sched *s, int64_t seq_id, const int32_t *prompt, i
       q.len += s->bs;
     }
   }
-  if (cached_tokens) *cached_tokens = q.len;
-  s->seqs.emplace(seq_id, std::move(q));
+  const int32_t cached = q.len;
+  std::vector<int64_t> taken;
+  try {
+    taken = q.blocks;
+    s->seqs.emplace(seq_id, std::move(q));
+  } catch (...) {  // give the references back: the call changes nothing when it fails
+    const std::vector<int64_t> &held = taken.empty() ? q.blocks : taken;
+    for (size_t i = held.size(); i-- > 0;) s->release(held[i]);
+    return fail(EID_ERR_INVALID_ARG, "out of host memory");
+  }
+  if (cached_tokens) *cached_tokens = cached;
   return EID_OK;
 }
 
@@ -213,14 +236,20 @@ int32_t eid_sched_build_batch(eid_sched *s, const int64_t *seq_ids, const int32_
   const int bs = s->bs;
   // pass 1: validate, count the blocks the step needs; nothing is modified
   int64_t need = 0, total_q = 0;
-  std::vector<Seq *> sq((size_t)num_seqs);
+  std::vector<Seq *> sq;
+  try {
+    sq.resize((size_t)num_seqs);
+  } catch (...) {
+    return fail(EID_ERR_INVALID_ARG, "out of host memory");
+  }
+  const uint64_t stamp = ++s->stamp;  // marks the sequences of this call: finds duplicates in O(1)
   for (int i = 0; i < num_seqs; ++i) {
     auto it = s->seqs.find(seq_ids[i]);
     if (it == s->seqs.end()) return fail(EID_ERR_INVALID_ARG, "sequence %lld unknown", (long long)seq_ids[i]);
     if (q_lens[i] < 1) return fail(EID_ERR_INVALID_ARG, "q_lens[%d] = %d must be >= 1", i, q_lens[i]);
     Seq *q = &it->second;
-    for (int j = 0; j < i; ++j)
-      if (sq[(size_t)j] == q) return fail(EID_ERR_INVALID_ARG, "sequence %lld listed twice", (long long)seq_ids[i]);
+    if (q->stamp == stamp) return fail(EID_ERR_INVALID_ARG, "sequence %lld listed twice", (long long)seq_ids[i]);
+    q->stamp = stamp;
     sq[(size_t)i] = q;
     const int64_t new_len = (int64_t)q->len + q_lens[i];
     const int64_t nb = (new_len + bs - 1) / bs;
@@ -228,6 +257,12 @@ int32_t eid_sched_build_batch(eid_sched *s, const int64_t *seq_ids, const int32_
       return fail(EID_ERR_INVALID_ARG, "sequence %lld would need %lld blocks (max_blocks_per_seq %d)",
                   (long long)seq_ids[i], (long long)nb, s->max_blocks_per_seq);
     need += nb - (int64_t)q->blocks.size();
+    try {  // capacity only: pass 2 must not allocate, so it cannot fail half way
+      q->blocks.reserve((size_t)nb);
+      q->tail.reserve((size_t)bs);
+    } catch (...) {
+      return fail(EID_ERR_INVALID_ARG, "out of host memory");
+    }
     total_q += q_lens[i];
     if (total_q > 0x7fffffff) return fail(EID_ERR_INVALID_ARG, "more than 2^31 query tokens");
   }
@@ -260,7 +295,11 @@ int32_t eid_sched_build_batch(eid_sched *s, const int64_t *seq_ids, const int32_
           B.hash = h;
           B.parent = q.chain;
           std::memcpy(&s->block_tokens[(size_t)blk * bs], q.tail.data(), sizeof(int32_t) * bs);
-          if (s->index.emplace(h, blk).second) B.indexed = true;  // first copy of a prefix wins
+          try {
+            if (s->index.emplace(h, blk).second) B.indexed = true;  // first copy of a prefix wins
+          } catch (...) {
+            // no memory for the index node: the block simply stays unshared
+          }
           q.chain = h;
           q.tail.clear();
         }
