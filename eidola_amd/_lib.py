@@ -96,6 +96,7 @@ class BatchInfo(C.Structure):
 
 
 EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
+           "eid_o_proj",
            "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
                  "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
@@ -128,6 +129,8 @@ def load_library():
     lib.eid_rope_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, C.c_int32, P, P, P, P,
                                       C.c_int32, P, P, P]
     lib.eid_rope_kv_write.restype = C.c_int32
+    lib.eid_o_proj.argtypes = [P, P, P, P, P, C.c_int32, C.c_int32, C.c_int32, P]
+    lib.eid_o_proj.restype = C.c_int32
     for name in ("eid_attn_decode", "eid_attn_varlen", "eid_lse_merge"):
         fn = getattr(lib, name)
         fn.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs), P]

@@ -21,6 +21,9 @@ hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
                                 uint8_t *k_cache, uint8_t *v_cache, const int64_t *slot_mapping,
                                 const float *k_scale, const float *v_scale, int Hq, int Hkv,
                                 int64_t num_slots, int num_tokens, bool fp8, hipStream_t st);
+hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
+                         const uint16_t *resid, uint16_t *out, int T, int N, int K,
+                         hipStream_t st);
 hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
                            uint8_t *v_cache, const int64_t *slot_mapping, const float *k_scale,
                            const float *v_scale, int Hkv, int64_t num_slots, int num_tokens,
@@ -374,6 +377,34 @@ int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args, void
     p.plan_slot = static_cast<int32_t *>(args->workspace) + (desc->max_q_len <= 2 ? 0 : 2);
   hipError_t e = eid::launch_merge(p, static_cast<hipStream_t>(hip_stream));
   if (e != hipSuccess) return hip_fail(e, "merge launch");
+  return EID_OK;
+}
+
+int32_t eid_o_proj(const void *attn_out, const void *weight, const void *bias,
+                   const void *residual, void *out, int32_t num_tokens, int32_t out_features,
+                   int32_t in_features, void *hip_stream) {
+  g_err[0] = 0;
+  if (num_tokens < 0) return fail(EID_ERR_INVALID_ARG, "num_tokens %d < 0", num_tokens);
+  if (in_features <= 0 || in_features % 64 != 0)
+    return fail(EID_ERR_UNSUPPORTED, "in_features %d must be a positive multiple of 64", in_features);
+  if (out_features <= 0 || out_features % 16 != 0)
+    return fail(EID_ERR_UNSUPPORTED, "out_features %d must be a positive multiple of 16", out_features);
+  if ((int64_t)num_tokens * out_features > (int64_t)0x7fffffff * 64 ||
+      (int64_t)out_features * in_features > (int64_t)0x7fffffff * 64)
+    return fail(EID_ERR_UNSUPPORTED, "matrix too large");
+  if (num_tokens == 0) return EID_OK;
+  if (!attn_out || !weight || !out)
+    return fail(EID_ERR_INVALID_ARG, "attn_out, weight and out must be non-NULL");
+  if (!aligned16(attn_out) || !aligned16(weight) || !aligned16(out) || !aligned16(bias) ||
+      !aligned16(residual))
+    return fail(EID_ERR_INVALID_ARG, "attn_out, weight, bias, residual and out must be 16-byte aligned");
+  if (out == attn_out) return fail(EID_ERR_INVALID_ARG, "out must not alias attn_out");
+  hipError_t e = eid::launch_o_proj(
+      static_cast<const uint16_t *>(attn_out), static_cast<const uint16_t *>(weight),
+      static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(residual),
+      static_cast<uint16_t *>(out), num_tokens, out_features, in_features,
+      static_cast<hipStream_t>(hip_stream));
+  if (e != hipSuccess) return hip_fail(e, "o_proj launch");
   return EID_OK;
 }
 

@@ -152,6 +152,38 @@ def rope_kv_write(geom, qkv, positions, cos_sin, k_cache, v_cache, slot_mapping,
     return q_out
 
 
+def o_proj(attn_out, weight, bias=None, residual=None, out=None):
+    """Output projection after attention: attn_out [T, Hq, D] (or [T, K]) bf16, weight [N, K]
+    bf16 (out_features x in_features), optional bias [N] and residual [T, N] bf16; returns
+    out [T, N] bf16 = attn_out @ weight^T + bias + residual (fp32 sums, one bf16 rounding).
+    `out` may be the residual buffer itself."""
+    if attn_out.dim() == 3:
+        attn_out = attn_out.reshape(attn_out.shape[0], -1)
+    _require(attn_out, "attn_out", torch.bfloat16, 2)
+    _require(weight, "weight", torch.bfloat16, 2)
+    T, K = attn_out.shape
+    N = weight.shape[0]
+    if weight.shape[1] != K:
+        raise ValueError("weight must be [out_features, in_features] with in_features = %d" % K)
+    if bias is not None:
+        _require(bias, "bias", torch.bfloat16, 1)
+        if bias.shape[0] != N:
+            raise ValueError("bias must be [out_features]")
+    if residual is not None:
+        _require(residual, "residual", torch.bfloat16, 2)
+        if tuple(residual.shape) != (T, N):
+            raise ValueError("residual must be [T, out_features]")
+    if out is None:
+        out = torch.empty((T, N), dtype=torch.bfloat16, device=attn_out.device)
+    else:
+        _require(out, "out", torch.bfloat16, 2)
+        if tuple(out.shape) != (T, N):
+            raise ValueError("out must be [T, out_features]")
+    check(load_library().eid_o_proj(_ptr(attn_out), _ptr(weight), _ptr(bias), _ptr(residual),
+                                    _ptr(out), T, N, K, _stream()))
+    return out
+
+
 def yarn_cos_sin(max_pos, head_dim=64, base=150000.0, scaling_factor=32.0,
                  initial_context=4096.0, ntk_alpha=1.0, ntk_beta=32.0):
     """[max_pos, head_dim] fp32 table for eid_rope_kv_write (numpy): per position head_dim/2

@@ -182,6 +182,30 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
 int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
                       void *hip_stream);
 
+/*
+ * The step behind the path: output projection with bias and residual epilogue,
+ *   out[t, n] = bf16( sum_k attn_out[t, k] * weight[n, k] + bias[n] + residual[t, n] ),
+ * products and sums in fp32, one rounding to bf16 (nearest-even) at the end.
+ *   attn_out  [num_tokens, in_features] bf16: the `out` of eid_attn_decode / eid_attn_varlen
+ *             as it stands ([num_q_tokens, Hq, 64], in_features = Hq * 64, index
+ *             head * 64 + dim): token-major rows are the K-contiguous operand the matrix
+ *             units want, so no head-major variant of the attention output exists
+ *   weight    [out_features, in_features] bf16, in_features contiguous (the usual order of
+ *             a linear layer's weight)
+ *   bias      [out_features] bf16 or NULL
+ *   residual  [num_tokens, out_features] bf16 or NULL; may be the same buffer as `out`
+ *   out       [num_tokens, out_features] bf16
+ * in_features must be a multiple of 64, out_features a multiple of 16; all pointers 16-byte
+ * aligned.  Up to 64 tokens the weight is streamed once (HBM-bound), beyond that a tiled
+ * matrix-core kernel runs.  The order of the fp32 additions differs between the two and from
+ * a sequential sum; results agree with an exactly rounded result to within fp32 summation
+ * error before the bf16 rounding.  Reference counterpart: none.  Engine call site: per layer
+ * per step, right after attention, on the same stream.
+ */
+int32_t eid_o_proj(const void *attn_out, const void *weight, const void *bias,
+                   const void *residual, void *out, int32_t num_tokens, int32_t out_features,
+                   int32_t in_features, void *hip_stream);
+
 /* Bytes of workspace eid_attn_decode / eid_attn_varlen / eid_lse_merge need for desc.
  * Returns 0 for an invalid desc. */
 size_t eid_workspace_bytes(const eid_attn_desc *desc);

@@ -42,6 +42,10 @@ def lib():
         L.orc_rope_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, C.c_int32, P, P, P, P,
                                         C.c_int32, P, P]
         L.orc_rope_kv_write.restype = C.c_int
+        L.orc_o_proj.argtypes = [P, P, P, P, P, P, C.c_int32, C.c_int32, C.c_int32]
+        L.orc_o_proj.restype = None
+        L.orc_f64_to_bf16.argtypes = [C.c_double]
+        L.orc_f64_to_bf16.restype = C.c_uint16
         L.orc_attn_f64.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs), P, P]
         L.orc_attn_f64.restype = C.c_int
         L.orc_splitkv_partials_f64.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs),
@@ -120,6 +124,20 @@ def rope_kv_write(desc, qkv, positions, cos_sin, k_cache, v_cache, slot_mapping,
     if rc:
         raise ValueError("slot out of range")
     return q_out
+
+
+def o_proj(a, w, bias=None, residual=None):
+    """Output projection; a [T,K], w [N,K], bias [N], residual [T,N] as bf16 bits (uint16).
+    Returns (out bf16 bits [T,N], exact float64 [T,N])."""
+    a, w = _c(a, np.uint16), _c(w, np.uint16)
+    b, r = _c(bias, np.uint16), _c(residual, np.uint16)
+    T, K = a.shape
+    N = w.shape[0]
+    assert w.shape[1] == K
+    out = np.zeros((T, N), dtype=np.uint16)
+    exact = np.zeros((T, N), dtype=np.float64)
+    lib().orc_o_proj(_p(a), _p(w), _p(b), _p(r), _p(out), _p(exact), T, N, K)
+    return out, exact
 
 
 def attn_f64(desc, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, sinks=None,

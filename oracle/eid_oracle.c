@@ -32,6 +32,27 @@ uint16_t orc_f32_to_bf16(float f) {
   return (uint16_t)(u >> 16);
 }
 
+/* Nearest bf16 to a double, ties to even, decided in double arithmetic: the two bf16
+ * neighbours of x are found from its fp32 truncation, so no second rounding intervenes. */
+uint16_t orc_f64_to_bf16(double x) {
+  if (isnan(x)) return 0x7FC0u;
+  const double ax = fabs(x);
+  const uint16_t sign = signbit(x) ? 0x8000u : 0u;
+  if (ax >= 3.3961775292304225e38) return (uint16_t)(sign | 0x7F80u); /* >= max + half ulp */
+  /* largest bf16 magnitude <= ax: search by bits (monotone for non-negative values) */
+  uint32_t lo = 0, hi = 0x7F7Fu;
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi + 1) >> 1;
+    if ((double)orc_bf16_to_f32((uint16_t)mid) <= ax) lo = mid; else hi = mid - 1;
+  }
+  const double below = (double)orc_bf16_to_f32((uint16_t)lo);
+  if (below == ax || lo == 0x7F7Fu) return (uint16_t)(sign | lo);
+  const double above = (double)orc_bf16_to_f32((uint16_t)(lo + 1));
+  const double d_lo = ax - below, d_hi = above - ax; /* exact: neighbours within a factor 2 */
+  uint32_t pick = d_lo < d_hi ? lo : d_hi < d_lo ? lo + 1 : ((lo & 1u) ? lo + 1 : lo);
+  return (uint16_t)(sign | pick);
+}
+
 /* OCP e4m3fn: 1 sign, 4 exponent (bias 7), 3 mantissa; no infinities; S.1111.111 = NaN;
  * largest finite 448 = 1.75 * 2^8; subnormals are multiples of 2^-9. */
 float orc_fp8_e4m3_decode(uint8_t b) {
@@ -422,4 +443,26 @@ int orc_attn_bf16(const eid_attn_desc *d, const eid_attn_args *a, int num_thread
     }
   }
   return 0;
+}
+
+/* ------------------------------------------------------------------ output projection */
+
+/* out[t][n] = bf16(sum_k a[t][k] w[n][k] + bias[n] + residual[t][n]).  Every product of two
+ * bf16 values is exact in double; the sum of K of them is accumulated in double (relative
+ * error ~ K 2^-53, far below the bf16 grid). */
+void orc_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
+                const uint16_t *residual, uint16_t *out, double *exact64, int32_t T, int32_t N,
+                int32_t K) {
+#pragma omp parallel for schedule(static)
+  for (int32_t t = 0; t < T; ++t) {
+    for (int32_t n = 0; n < N; ++n) {
+      const uint16_t *ar = a + (size_t)t * K, *wr = w + (size_t)n * K;
+      double s = 0.0;
+      for (int32_t k = 0; k < K; ++k) s += (double)orc_bf16_to_f32(ar[k]) * (double)orc_bf16_to_f32(wr[k]);
+      if (bias) s += (double)orc_bf16_to_f32(bias[n]);
+      if (residual) s += (double)orc_bf16_to_f32(residual[(size_t)t * N + n]);
+      if (exact64) exact64[(size_t)t * N + n] = s;
+      if (out) out[(size_t)t * N + n] = orc_f64_to_bf16(s);
+    }
+  }
 }

@@ -44,6 +44,15 @@ int orc_rope_kv_write(const eid_attn_desc *d, const uint16_t *qkv, const int32_t
                       void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
                       const float *k_scale, const float *v_scale);
 
+/* Output projection with bias and residual: same contract as eid_o_proj.
+ * exact64 (may be NULL) receives the unrounded values [T, N]: the fp64 sum of the exact
+ * bf16 x bf16 products, plus bias, plus residual; out (may be NULL) receives them rounded to
+ * bf16 once, nearest-even, straight from the double (no detour through fp32). */
+void orc_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
+                const uint16_t *residual, uint16_t *out, double *exact64, int32_t T, int32_t N,
+                int32_t K);
+uint16_t orc_f64_to_bf16(double x);                /* round-to-nearest-even, NaN -> quiet NaN */
+
 /* Definitional attention in fp64 from the stored bf16/fp8 bits.
  * out64: [T, Hq, D] doubles; lse64: [T, Hq] doubles or NULL.
  * cu_seqlens_q may be NULL (then q_len = 1 for every sequence). */

@@ -49,9 +49,10 @@ def gpu_caches(batch, k, v, k_scale=None, v_scale=None):
 
 
 def run_attn(batch, q, kc_d, vc_d, sinks, k_scale=None, v_scale=None, *, decode=None,
-             return_lse=False, geom=None, hint=False):
+             return_lse=False, geom=None, hint=False, return_device=False):
     """Calls eid_attn_decode (all q_len == 1) or eid_attn_varlen through the C ABI; with
-    `hint` the host-side sum of seq_lens is passed as desc.sum_kv_len."""
+    `hint` the host-side sum of seq_lens is passed as desc.sum_kv_len.  `return_device`
+    hands back the output tensor itself instead of its bits on the host."""
     geom = geom or batch.geom
     if decode is None:
         decode = batch.max_q_len == 1
@@ -65,6 +66,8 @@ def run_attn(batch, q, kc_d, vc_d, sinks, k_scale=None, v_scale=None, *, decode=
         r = ea.attn_varlen(geom, bf16_dev(q), kc_d, vc_d, bt, sl, dev(batch.cu_seqlens_q),
                            max_q_len=batch.max_q_len, **kw)
     torch.cuda.synchronize()
+    if return_device:
+        return r[0] if return_lse else r
     if return_lse:
         return bits_host(r[0]), r[1].cpu().numpy()
     return bits_host(r)

@@ -130,6 +130,19 @@ def test_kv_write_validation_without_a_gpu():
     assert lib.eid_last_error() != b""
 
 
+def test_o_proj_validation_without_a_gpu():
+    lib = ea.load_library()
+    ok = 0x1000
+    assert lib.eid_o_proj(None, None, None, None, None, 0, 2880, 4096, None) == 0
+    assert lib.eid_o_proj(ok, ok, None, None, None, 4, 2880, 4096, None) == _lib.EID_ERR_INVALID_ARG
+    assert lib.eid_o_proj(ok, ok, None, None, ok, -1, 2880, 4096, None) == _lib.EID_ERR_INVALID_ARG
+    assert lib.eid_o_proj(ok, ok, None, None, ok, 4, 2880, 4100, None) == _lib.EID_ERR_UNSUPPORTED
+    assert lib.eid_o_proj(ok, ok, None, None, ok, 4, 2888, 4096, None) == _lib.EID_ERR_UNSUPPORTED
+    assert lib.eid_o_proj(ok, ok, ok + 8, None, ok + 0x100, 4, 2880, 4096, None) == _lib.EID_ERR_INVALID_ARG
+    assert lib.eid_o_proj(ok, ok, None, None, ok, 4, 2880, 4096, None) == _lib.EID_ERR_INVALID_ARG  # out aliases attn_out
+    assert b"alias" in lib.eid_last_error()
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "lib_path", lambda: str(tmp_path / "nope.so"))
