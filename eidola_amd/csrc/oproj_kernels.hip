@@ -57,63 +57,118 @@ __device__ __forceinline__ void oproj_store(const f32x4 acc, const uint16_t *bia
 }
 
 constexpr int kSkWaves = 8;
-constexpr int kSkChunk = 64;   // K elements per chunk: one 128-byte line of every weight row
-constexpr int kSkBatch = 8;    // chunks whose weight loads a wave issues back to back
+constexpr int kSkChunk = 64;                       // K elements per chunk: one 128-byte line per row
+constexpr int kSkSlab = kSkWaves * kSkChunk;       // K elements per round: one chunk per wave
+constexpr int kSkRounds = 8;                       // rounds whose weight loads are issued at once
+constexpr int kSkRowBytes = kSkSlab * 2 + 16;      // LDS row of an activation slab, padded
 
 }  // namespace
 
 // ---------------------------------------------------------------------------------------
-// Skinny kernel.  grid = N / 16, block = 512.  TT = number of 16-token tiles (T <= 16 TT).
-// Wave w takes chunks w, w + 8, w + 16, ... of the K dimension.  Requires K % 64 == 0.
+// Streaming kernel.  grid = N / 16, block = 512.  TT = number of 16-token tiles (T <= 16 TT).
+// K is walked in rounds of 512 elements; in round r wave w owns chunk 8 r + w.
+//   weights      each wave loads the fragments of its chunks of 8 rounds (all of K = 4096)
+//                back to back, straight from memory: 16 KiB in flight per wave
+//   activations  every workgroup needs all of a[T, K].  Loading its MFMA fragments straight
+//                from memory (16 rows x 64 bytes per instruction, rows 2 K bytes apart) runs
+//                at a fraction of the cache bandwidth, so a slab of a round (16 TT rows x
+//                1 KiB) is fetched with whole-row loads (one row per wave instruction), kept
+//                two rounds ahead in registers, passed through a double-buffered LDS tile
+//                and read from there as fragments.
+// The eight K shares meet in LDS (reusing the slab tiles).  Requires K % 64 == 0.
 // ---------------------------------------------------------------------------------------
 template <int TT>
 __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
     uint16_t *out, const int T, const int N, const int K) {
-  __shared__ f32x4 red[kSkWaves][TT][64];
+  constexpr int kRows = TT * 16;
+  constexpr int kLd = kRows / kSkWaves;  // slab rows per wave = loads per thread and slab
+  constexpr int kTileBytes = kRows * kSkRowBytes;
+  static_assert(2 * kTileBytes >= (int)sizeof(f32x4) * kSkWaves * TT * 64, "reduction reuses the tiles");
+  __shared__ __align__(16) uint8_t lds[2 * kTileBytes];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16;
   const int nchunks = K / kSkChunk;
+  const int R = (nchunks + kSkWaves - 1) / kSkWaves;
 
   const uint16_t *wp = w + (size_t)(n0 + i16) * K + g * 8;
-  const uint16_t *ap[TT];
+  // slab loader: wave w fetches rows w, w + 8, ...; a lane 16 bytes of the row's 1 KiB
+  const uint16_t *arow[kLd];
 #pragma unroll
-  for (int tt = 0; tt < TT; ++tt) ap[tt] = a + (size_t)min(tt * 16 + i16, T - 1) * K + g * 8;
+  for (int j = 0; j < kLd; ++j) arow[j] = a + (size_t)min(wave + kSkWaves * j, T - 1) * K;
+  u32x4 ar[2][kLd];
+  auto a_fetch = [&](const int st, const int r) {
+    int col = r * kSkSlab + lane * 8;
+    col = col < K ? col : 0;  // past the end of a short last slab: any valid address
+#pragma unroll
+    for (int j = 0; j < kLd; ++j) ar[st][j] = ld16(arow[j] + col);
+  };
+  const uint32_t st_off = (uint32_t)wave * kSkRowBytes + lane * 16;
+  auto a_stash = [&](const int st, const int buf) {
+#pragma unroll
+    for (int j = 0; j < kLd; ++j)
+      *(u32x4 *)(&lds[buf * kTileBytes + st_off + j * kSkWaves * kSkRowBytes]) = ar[st][j];
+  };
+  const uint32_t rd_off = (uint32_t)i16 * kSkRowBytes + wave * 128 + g * 16;
 
   f32x4 acc[TT];
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) acc[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  for (int c0 = wave; c0 < nchunks; c0 += kSkWaves * kSkBatch) {
-    // the whole batch of weight fragments first: 2 KiB per chunk and wave in flight
-    Frag8 wf[kSkBatch][2];
+  // Rounds rb .. rb + 7.  Every load is issued unconditionally (clamped): a load under a
+  // branch would leave the count of loads in flight unknown where the paths join, and the
+  // waits that follow would then drain all of them.
+  constexpr bool kEarlyW = TT < 4;
+  Frag8 wf[kSkRounds][2];
+  auto w_fetch = [&](const int rb) {
 #pragma unroll
-    for (int j = 0; j < kSkBatch; ++j) {
-      const int c = min(c0 + j * kSkWaves, nchunks - 1);  // a repeated chunk is skipped below
+    for (int j = 0; j < kSkRounds; ++j) {
+      const int c = min((rb + j) * kSkWaves + wave, nchunks - 1);
       wf[j][0].u = ld16(wp + c * kSkChunk);
       wf[j][1].u = ld16(wp + c * kSkChunk + 32);
     }
+  };
+  auto batch = [&](const int rb) {
+    if (rb > 0 || !kEarlyW) w_fetch(rb);  // else the first batch's weights are on their way
 #pragma unroll
-    for (int j = 0; j < kSkBatch; ++j) {
-      const int c = c0 + j * kSkWaves;
-      if (c < nchunks) {  // wave-uniform
-        Frag8 af[TT][2];
+    for (int j = 0; j < kSkRounds; ++j) {
+      const int par = j & 1;  // = (rb + j) % 2: rb is a multiple of 8
+      const int r = rb + j;
+      // LDS tile `par` holds slab r, register stage par ^ 1 slab r + 1 (in flight)
+      a_fetch(par, min(r + 2, R - 1));
+      if (r * kSkWaves + wave < nchunks) {  // wave-uniform
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
-          af[tt][0].u = ld16(ap[tt] + c * kSkChunk);
-          af[tt][1].u = ld16(ap[tt] + c * kSkChunk + 32);
-        }
-#pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-          acc[tt] = mfma16x32(wf[j][0], af[tt][0], acc[tt]);
-          acc[tt] = mfma16x32(wf[j][1], af[tt][1], acc[tt]);
+          Frag8 a0, a1;
+          const uint8_t *src = &lds[par * kTileBytes + rd_off + tt * 16 * kSkRowBytes];
+          a0.u = *(const u32x4 *)src;
+          a1.u = *(const u32x4 *)(src + 64);
+          acc[tt] = mfma16x32(wf[j][0], a0, acc[tt]);
+          acc[tt] = mfma16x32(wf[j][1], a1, acc[tt]);
         }
       }
+      a_stash(par ^ 1, par ^ 1);
+      __syncthreads();
     }
+  };
+
+  // The weight stream should start before anything waits; with four token tiles the
+  // registers do not stretch to holding it across the first slab's hand-over.
+  a_fetch(0, 0);  // the small, cache-resident slab first: it gates the first round
+  if (kEarlyW) w_fetch(0);
+  a_fetch(1, min(1, R - 1));
+  a_stash(0, 0);
+  __syncthreads();
+  if (R <= kSkRounds) {
+    batch(0);  // straight-line code for K <= 4096
+  } else {
+    for (int rb = 0; rb < R; rb += kSkRounds) batch(rb);
   }
+
+  f32x4(*red)[TT][64] = reinterpret_cast<f32x4(*)[TT][64]>(lds);  // all tile reads are done
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) red[wave][tt][lane] = acc[tt];
   __syncthreads();
@@ -186,22 +241,6 @@ __global__ __launch_bounds__(256, 2) void oproj_tiled_kernel(
     asrc[j] = a + (size_t)min(m0 + ld_row + 32 * j, T - 1) * K + ld_seg * 8;
   }
   const uint32_t st_off = (uint32_t)ld_row * kTlRowBytes + ld_seg * 16;
-  u32x4 wr[4], ar[4];
-  auto fetch = [&](const int k0) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      wr[j] = ld16(wsrc[j] + k0);
-      ar[j] = ld16(asrc[j] + k0);
-    }
-  };
-  auto stash = [&](const int buf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      *(u32x4 *)(&lds_w[buf][st_off + j * 32 * kTlRowBytes]) = wr[j];
-      *(u32x4 *)(&lds_a[buf][st_off + j * 32 * kTlRowBytes]) = ar[j];
-    }
-  };
-
   f32x4 acc[4][4];  // [feature tile][token tile]
 #pragma unroll
   for (int ft = 0; ft < 4; ++ft)
@@ -211,28 +250,54 @@ __global__ __launch_bounds__(256, 2) void oproj_tiled_kernel(
   const uint32_t rd_w = (uint32_t)(wn * 64 + i16) * kTlRowBytes + g * 16;
   const uint32_t rd_a = (uint32_t)(wm * 64 + i16) * kTlRowBytes + g * 16;
 
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  int cur = 0;
-  for (int k0 = 0; k0 < K; k0 += kTlK, cur ^= 1) {
-    const bool has_next = k0 + kTlK < K;
-    if (has_next) fetch(k0 + kTlK);
+  // Two register stages: the loads of K step i + 2 are issued while step i is computed and
+  // are only needed (moved to LDS) at the end of step i + 1, so every global load has two
+  // full steps to arrive.
+  u32x4 wr[2][4], ar[2][4];
+  auto fetch = [&](const int st, const int k0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      wr[st][j] = ld16(wsrc[j] + k0);
+      ar[st][j] = ld16(asrc[j] + k0);
+    }
+  };
+  auto stash = [&](const int st, const int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      *(u32x4 *)(&lds_w[buf][st_off + j * 32 * kTlRowBytes]) = wr[st][j];
+      *(u32x4 *)(&lds_a[buf][st_off + j * 32 * kTlRowBytes]) = ar[st][j];
+    }
+  };
+  const int nk = K / kTlK;
+  auto step = [&](const int par, const int i) {  // par = i % 2, a literal at both call sites
+    // unconditional (the last steps refetch the final slab and never use it): a fetch under
+    // a branch would leave the number of loads in flight unknown at the join and force the
+    // LDS stores below to wait for all of them
+    fetch(par, min(i + 2, nk - 1) * kTlK);
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       Frag8 wf[4], af[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        wf[i].u = *(const u32x4 *)(&lds_w[cur][rd_w + i * 16 * kTlRowBytes + ks * 64]);
-        af[i].u = *(const u32x4 *)(&lds_a[cur][rd_a + i * 16 * kTlRowBytes + ks * 64]);
+      for (int x = 0; x < 4; ++x) {
+        wf[x].u = *(const u32x4 *)(&lds_w[par][rd_w + x * 16 * kTlRowBytes + ks * 64]);
+        af[x].u = *(const u32x4 *)(&lds_a[par][rd_a + x * 16 * kTlRowBytes + ks * 64]);
       }
 #pragma unroll
       for (int ft = 0; ft < 4; ++ft)
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) acc[ft][tt] = mfma16x32(wf[ft], af[tt], acc[ft][tt]);
     }
-    if (has_next) stash(cur ^ 1);
+    if (i + 1 < nk) stash(par ^ 1, par ^ 1);
     __syncthreads();
+  };
+
+  fetch(0, 0);
+  fetch(1, min(1, nk - 1) * kTlK);
+  stash(0, 0);
+  __syncthreads();
+  for (int i = 0; i < nk; i += 2) {
+    step(0, i);
+    if (i + 1 < nk) step(1, i + 1);
   }
 
 #pragma unroll
