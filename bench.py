@@ -273,6 +273,52 @@ def rope_bench(torch, ea, synth, steps=50):
     return out
 
 
+def oproj_bench(torch, ea):
+    """eid_o_proj on gpt-oss's shape (4096 -> 2880, bias + residual) for a 64-token decode
+    step, a 256-token batch and config 3's 4,216 tokens.  16 weight copies (377 MB, more than
+    the last-level cache) are used in turn, as the layers of a model would be; 16 launches
+    are captured in a HIP graph and its replay timed with events, so the figure is device
+    time, not Python call overhead.  Up to 64 tokens the kernel is HBM-bound (algorithmic
+    bytes = weight + activations in + residual in + out), beyond that MFMA-bound
+    (2 T N K flops).  torch.addmm (hipBLASLt) on the same buffers is timed beside it."""
+    N, K, L = 2880, 4096, 16
+    ws = [torch.randn(N, K, device="cuda:0").to(torch.bfloat16) * 0.02 for _ in range(L)]
+    bias = torch.randn(N, device="cuda:0").to(torch.bfloat16)
+    out = []
+    for T in (64, 256, 4216):
+        x = torch.randn(T, K, device="cuda:0").to(torch.bfloat16)
+        res = torch.randn(T, N, device="cuda:0").to(torch.bfloat16)
+        y = torch.empty(T, N, dtype=torch.bfloat16, device="cuda:0")
+        fns = {"eid": lambda i: ea.o_proj(x, ws[i], bias, res, out=y),
+               "hipblaslt": lambda i: torch.addmm(res, x, ws[i].t(), out=y)}
+        r = {"config": f"o_proj_{T}_tokens", "flops": 2.0 * T * N * K,
+             "alg_bytes": 2 * (N * K + T * K + 2 * T * N + N)}
+        for name, fn in fns.items():
+            for i in range(2):
+                fn(i)
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                fn(0)
+                torch.cuda.synchronize()
+                with torch.cuda.graph(graph, stream=side):
+                    for i in range(L):
+                        fn(i)
+            torch.cuda.synchronize()
+            graph.replay()
+            ms = event_ms(lambda i: graph.replay(), 5, torch) / L
+            r[name + "_ms"] = ms
+        r["GBps"] = r["alg_bytes"] / r["eid_ms"] / 1e6
+        r["TFLOPs"] = r["flops"] / r["eid_ms"] / 1e9
+        log(f"[bench] o_proj, {T} tokens: {r['eid_ms']*1e3:.1f} us per call "
+            f"({r['GBps']:.0f} GB/s = {100*r['GBps']/HBM_PEAK_GBS:.1f}% HBM, "
+            f"{r['TFLOPs']:.0f} TFLOP/s = {100*r['TFLOPs']/2500:.1f}% of bf16 MFMA peak); "
+            f"hipBLASLt {r['hipblaslt_ms']*1e3:.1f} us")
+        out.append(r)
+    return out
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -421,6 +467,7 @@ def main():
             torch.cuda.empty_cache()
         extra.append(sched_bench(synth, ea))
         extra.extend(rope_bench(torch, ea, synth))
+        extra.extend(oproj_bench(torch, ea))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)

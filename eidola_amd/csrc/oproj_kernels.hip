@@ -201,19 +201,24 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 // Requires K % 64 == 0 and N % 16 == 0.
 // ---------------------------------------------------------------------------------------
 namespace {
-constexpr int kTlTile = 128;
 constexpr int kTlK = 64;
 constexpr int kTlRowBytes = 144;
-constexpr int kTlTileBytes = kTlTile * kTlRowBytes;
 }  // namespace
 
-__global__ __launch_bounds__(256, 2) void oproj_tiled_kernel(
+// WT = 16-row MFMA tiles per wave and dimension: 4 gives the 128 x 128 workgroup tile, 2 a
+// 64 x 64 one for batches too small to fill the device with the big tile (its K loop is as
+// long, but four workgroups share a CU).
+template <int WT>
+__global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
     uint16_t *out, const int T, const int N, const int K, const int tiles_m,
     const int tiles_n) {
-  __shared__ __align__(16) uint8_t lds_w[2][kTlTileBytes];
-  __shared__ __align__(16) uint8_t lds_a[2][kTlTileBytes];
+  constexpr int kTile = 32 * WT;  // rows of a workgroup tile in either dimension
+  constexpr int kWave = 16 * WT;  // rows of a wave tile
+  constexpr int kTileBytes = kTile * kTlRowBytes;
+  __shared__ __align__(16) uint8_t lds_w[2][kTileBytes];
+  __shared__ __align__(16) uint8_t lds_a[2][kTileBytes];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
@@ -230,40 +235,40 @@ __global__ __launch_bounds__(256, 2) void oproj_tiled_kernel(
   const int rows = min(tiles_m - first_m, 8);
   const int in_group = logical % group_size;
   const int tm = first_m + in_group % rows, tn = in_group / rows;
-  const int m0 = tm * kTlTile, n0 = tn * kTlTile;
+  const int m0 = tm * kTile, n0 = tn * kTile;
 
   // loader: a wave instruction covers 8 rows x 128 bytes (full lines)
   const int ld_row = tid >> 3, ld_seg = tid & 7;  // rows ld_row + 32 j
-  const uint16_t *wsrc[4], *asrc[4];
+  const uint16_t *wsrc[WT], *asrc[WT];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < WT; ++j) {
     wsrc[j] = w + (size_t)min(n0 + ld_row + 32 * j, N - 1) * K + ld_seg * 8;
     asrc[j] = a + (size_t)min(m0 + ld_row + 32 * j, T - 1) * K + ld_seg * 8;
   }
   const uint32_t st_off = (uint32_t)ld_row * kTlRowBytes + ld_seg * 16;
-  f32x4 acc[4][4];  // [feature tile][token tile]
+  f32x4 acc[WT][WT];  // [feature tile][token tile]
 #pragma unroll
-  for (int ft = 0; ft < 4; ++ft)
+  for (int ft = 0; ft < WT; ++ft)
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) acc[ft][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int tt = 0; tt < WT; ++tt) acc[ft][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const uint32_t rd_w = (uint32_t)(wn * 64 + i16) * kTlRowBytes + g * 16;
-  const uint32_t rd_a = (uint32_t)(wm * 64 + i16) * kTlRowBytes + g * 16;
+  const uint32_t rd_w = (uint32_t)(wn * kWave + i16) * kTlRowBytes + g * 16;
+  const uint32_t rd_a = (uint32_t)(wm * kWave + i16) * kTlRowBytes + g * 16;
 
   // Two register stages: the loads of K step i + 2 are issued while step i is computed and
   // are only needed (moved to LDS) at the end of step i + 1, so every global load has two
   // full steps to arrive.
-  u32x4 wr[2][4], ar[2][4];
+  u32x4 wr[2][WT], ar[2][WT];
   auto fetch = [&](const int st, const int k0) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < WT; ++j) {
       wr[st][j] = ld16(wsrc[j] + k0);
       ar[st][j] = ld16(asrc[j] + k0);
     }
   };
   auto stash = [&](const int st, const int buf) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < WT; ++j) {
       *(u32x4 *)(&lds_w[buf][st_off + j * 32 * kTlRowBytes]) = wr[st][j];
       *(u32x4 *)(&lds_a[buf][st_off + j * 32 * kTlRowBytes]) = ar[st][j];
     }
@@ -276,16 +281,16 @@ __global__ __launch_bounds__(256, 2) void oproj_tiled_kernel(
     fetch(par, min(i + 2, nk - 1) * kTlK);
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
-      Frag8 wf[4], af[4];
+      Frag8 wf[WT], af[WT];
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
+      for (int x = 0; x < WT; ++x) {
         wf[x].u = *(const u32x4 *)(&lds_w[par][rd_w + x * 16 * kTlRowBytes + ks * 64]);
         af[x].u = *(const u32x4 *)(&lds_a[par][rd_a + x * 16 * kTlRowBytes + ks * 64]);
       }
 #pragma unroll
-      for (int ft = 0; ft < 4; ++ft)
+      for (int ft = 0; ft < WT; ++ft)
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) acc[ft][tt] = mfma16x32(wf[ft], af[tt], acc[ft][tt]);
+        for (int tt = 0; tt < WT; ++tt) acc[ft][tt] = mfma16x32(wf[ft], af[tt], acc[ft][tt]);
     }
     if (i + 1 < nk) stash(par ^ 1, par ^ 1);
     __syncthreads();
@@ -301,16 +306,18 @@ __global__ __launch_bounds__(256, 2) void oproj_tiled_kernel(
   }
 
 #pragma unroll
-  for (int tt = 0; tt < 4; ++tt) {
-    const int t = m0 + wm * 64 + tt * 16 + i16;
+  for (int tt = 0; tt < WT; ++tt) {
+    const int t = m0 + wm * kWave + tt * 16 + i16;
     if (t >= T) continue;
 #pragma unroll
-    for (int ft = 0; ft < 4; ++ft) {
-      const int n = n0 + wn * 64 + ft * 16 + 4 * g;
+    for (int ft = 0; ft < WT; ++ft) {
+      const int n = n0 + wn * kWave + ft * 16 + 4 * g;
       if (n < N) oproj_store(acc[ft][tt], bias, resid, out, (size_t)t * N, n);
     }
   }
 }
+
+int device_cus();  // attn_kernels.hip
 
 hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
                          const uint16_t *resid, uint16_t *out, int T, int N, int K,
@@ -328,9 +335,18 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
       oproj_skinny_kernel<4><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     return hipGetLastError();
   }
-  const int tiles_m = (T + kTlTile - 1) / kTlTile, tiles_n = (N + kTlTile - 1) / kTlTile;
-  oproj_tiled_kernel<<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K, tiles_m,
-                                                       tiles_n);
+  // The 128 x 128 tile once it gives most CUs a workgroup, else 64 x 64 (measured
+  // crossover for 2880 x 4096: between 1,024 and 1,500 tokens, 184 and 276 big tiles).
+  const int big = ((T + 127) / 128) * ((N + 127) / 128);
+  if (4 * big >= 3 * device_cus()) {
+    const int tiles_m = (T + 127) / 128, tiles_n = (N + 127) / 128;
+    oproj_tiled_kernel<4><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                            tiles_m, tiles_n);
+  } else {
+    const int tiles_m = (T + 63) / 64, tiles_n = (N + 63) / 64;
+    oproj_tiled_kernel<2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                            tiles_m, tiles_n);
+  }
   return hipGetLastError();
 }
 
