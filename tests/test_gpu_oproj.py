@@ -6,7 +6,7 @@ tolerance is therefore
 
 (the second term bounds the fp32 summation error of 4096 terms with a wide margin), and at
 least 98 % of the outputs must be the oracle's bf16 bit for bit (the rest sit next to a
-rounding boundary).  Covered: both kernels and every tile count of the streaming one, ragged
+rounding boundary).  Covered: all three kernels and every tile count of the streaming one, ragged
 token and feature counts, bias / residual present or not, the residual updated in place, a
 poison canary around the output, and attention followed by the projection."""
 import numpy as np
@@ -79,8 +79,11 @@ def test_streaming_kernel_shapes(G, T, N, K, with_bias, with_res):
     _run(G, T, N, K, with_bias, with_res, seed=T + N)
 
 
+# the 64 x 64 tile (few workgroups) and the 128 x 128 tile (the last three: 276, 288 and 286
+# big tiles), with ragged token counts and feature counts that end inside a tile
 @pytest.mark.parametrize("T,N,K", [(65, 2880, 4096), (128, 128, 64), (129, 16, 128), (200, 144, 576),
-                                   (257, 2880, 512), (1000, 1040, 1024), (2048, 256, 256)])
+                                   (257, 2880, 512), (1000, 1040, 1024), (2048, 256, 256),
+                                   (1500, 2880, 512), (1025, 4096, 128), (2790, 1648, 192)])
 @pytest.mark.parametrize("with_bias,with_res", [(False, False), (True, True)])
 def test_tiled_kernel_shapes(G, T, N, K, with_bias, with_res):
     _run(G, T, N, K, with_bias, with_res, seed=T + K)
