@@ -3,8 +3,10 @@
 
 A step = one pass of the hot path over one synthetic batch of BASELINE.json's decode
 configuration (configs[1], full-attention variant): the slot-mapped KV write of the 64 new
-tokens followed by split-KV decode attention + merge, all inputs resident in HBM.  Page
-sets rotate between steps so the 256 MB Infinity Cache cannot serve the KV stream.
+tokens and split-KV decode attention + merge, all inputs resident in HBM: one
+eid_attn_decode call that is handed the new rows (k_new / v_new) and writes them into the
+cache itself, or with --unfused eid_kv_write followed by eid_attn_decode.  Page sets rotate
+between steps so the 256 MB Infinity Cache cannot serve the KV stream.
 
 Prints ONE JSON line on stdout.  `--all` additionally measures the other configurations
 and writes them (one JSON object per line) to the file given by --report.
@@ -60,18 +62,22 @@ def split_kernel_ms(w, steps, torch):
         pairs.append((a, b))
     torch.cuda.synchronize()
     for i, (a, b) in enumerate(pairs):
-        w.kv_write(i)
-        c = w.attn[i % w.n]
+        if w.fused:
+            c = w.fused[i % w.n]
+        else:
+            w.kv_write(i)
+            c = w.attn[i % w.n]
         a.record()
         c.args.split_done_event = b.cuda_event
         c()
     torch.cuda.synchronize()
-    for c in w.attn:
+    for c in w.attn + w.fused:
         c.args.split_done_event = None
     return sum(a.elapsed_time(b) for a, b in pairs) / steps
 
 
 NO_HINT = False  # --no-hint: do not pass the host-side sum of seq_lens to the library
+UNFUSED = False  # --unfused: decode steps as two launches (eid_kv_write, eid_attn_decode)
 
 
 class Workload:
@@ -110,7 +116,7 @@ class Workload:
         self.tables = [torch.from_numpy(b.block_table).to(dev) for b in self.batches]
         fn = "eid_attn_decode" if kind == "decode" else "eid_attn_varlen"
         ws = None
-        self.attn, self.merge = [], []
+        self.attn, self.merge, self.fused = [], [], []
         for bt in self.tables:
             # the scheduler's host-side copy of seq_lens gives the sum for free; the library
             # sizes the split-KV launch with it
@@ -122,6 +128,12 @@ class Workload:
             ws = c._keep[-1]
             self.attn.append(c)
             kw["workspace"] = ws
+            if kind == "decode" and not UNFUSED:
+                # the decode step as ONE call: the newest token's KV rows go in with the call,
+                # which writes them into the cache itself (stage K1 fused into K2)
+                self.fused.append(ea.prepare(fn, g, self.q, self.k_cache, self.v_cache, bt,
+                                             self.seq_lens, None, k_new=self.k_new,
+                                             v_new=self.v_new, **kw))
             self.merge.append(ea.prepare("eid_lse_merge", g, self.q, self.k_cache, self.v_cache,
                                          bt, self.seq_lens, cu, **kw))
         self.ea = ea
@@ -132,6 +144,13 @@ class Workload:
                          self.slots[i % self.n], self.k_scale, self.v_scale)
 
     def step(self, i):
+        """One pass of the hot path over one batch: KV write of the new tokens, attention."""
+        if self.fused:
+            self.fused[i % self.n]()
+        else:
+            self.step_unfused(i)
+
+    def step_unfused(self, i):
         self.kv_write(i)
         self.attn[i % self.n]()
 
@@ -174,6 +193,7 @@ def measure(w, steps, warmup, torch, synth, label):
     for i in range(warmup):
         w.step(i)
     ms_step = event_ms(w.step, steps, torch)
+    ms_unfused = event_ms(w.step_unfused, steps, torch) if w.fused else ms_step
     ms_attn = event_ms(lambda i: w.attn[i % w.n](), steps, torch)
     ms_merge = event_ms(lambda i: w.merge[i % w.n](), steps, torch)
     ms_write = event_ms(w.kv_write, steps, torch)
@@ -182,7 +202,8 @@ def measure(w, steps, warmup, torch, synth, label):
     work = synth.algorithmic_work(b)
     work_w = synth.algorithmic_work(b, include_kv_write=True)
     r = {
-        "config": label, "ms_per_step": ms_step, "ms_attn": ms_attn, "ms_merge": ms_merge,
+        "config": label, "ms_per_step": ms_step, "ms_per_step_two_launches": ms_unfused,
+        "fused_kv_write": bool(w.fused), "ms_attn": ms_attn, "ms_merge": ms_merge,
         "ms_kv_write": ms_write, "ms_split": ms_split, "ms_per_step_graph": ms_graph, "alg_bytes": work["bytes"], "alg_flops": work["flops"],
         "q_tokens": work["q_tokens"], "ctx_tokens": work["ctx_tokens"],
         "step_GBps": work_w["bytes"] / ms_step / 1e6,
@@ -196,6 +217,8 @@ def measure(w, steps, warmup, torch, synth, label):
     part = int(w.attn[0]._keep[-1][:4].view(torch.int32).item())
     r["partition"] = part if 64 <= part <= 4096 and part % 64 == 0 else None
     gtxt = f", graph replay {ms_graph*1e3:.1f}" if ms_graph else ""
+    if w.fused:
+        gtxt += f", as kv_write + attention {ms_unfused*1e3:.1f}"
     log(f"[bench] {label}: step {ms_step*1e3:.1f} us{gtxt} (attn {ms_attn*1e3:.1f}, split-KV "
         f"{ms_split*1e3:.1f}, merge {ms_merge*1e3:.1f}, kv_write {ms_write*1e3:.1f}); attn {r['attn_GBps']:.0f} GB/s = "
         f"{100*r['attn_GBps']/HBM_PEAK_GBS:.1f}% HBM, {r['attn_TFLOPs']:.1f} TFLOP/s; "
@@ -386,9 +409,13 @@ def main():
                     help="experiment: physically contiguous pages instead of a shuffled pool")
     ap.add_argument("--no-hint", action="store_true",
                     help="experiment: leave desc.sum_kv_len at 0 (grid sized from max_kv_len)")
+    ap.add_argument("--unfused", action="store_true",
+                    help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
+                         "instead of one eid_attn_decode call that takes k_new / v_new")
     a = ap.parse_args()
-    global NO_HINT
+    global NO_HINT, UNFUSED
     NO_HINT = a.no_hint
+    UNFUSED = a.unfused
     if a.gpus != 1:
         sys.exit("bench.py: this path runs on ONE MI355X (no sharding, no collectives); "
                  "--gpus must be 1")
@@ -412,7 +439,9 @@ def main():
         "data": "synthetic (seeded ragged batch, N(0,1) bf16 Q/K/V and sinks, random-permuted pages)",
         "config": {"workload": "configs[1] decode continuous batch, full attention: 64 seqs, "
                                "ctx U[1,8192], Hq64/Hkv8/D64, block 16, 300k-block pool; "
-                               "step = kv_write(64 tokens) + split-KV decode + LSE merge",
+                               "step = KV write of the 64 new tokens + split-KV decode + LSE merge"
+                               + ("" if a.unfused else " (one eid_attn_decode call: the write is "
+                                  "fused into the split-KV launch via k_new / v_new)"),
                    "partition_size": a.partition if a.partition else "run-time (workspace planned for >= %d)"
                    % ea.partition_size(w.attn[0].desc),
                    "sum_kv_len_hint": not a.no_hint,
@@ -420,7 +449,8 @@ def main():
         "pct_hbm_peak": 100 * r["step_GBps"] / HBM_PEAK_GBS,
         "tokens_per_s": r["q_tokens_per_s"], "ctx_tokens_per_s": r["ctx_tokens_per_s"],
         "breakdown_us": {"kv_write": r["ms_kv_write"] * 1e3, "attn_call": r["ms_attn"] * 1e3,
-                         "merge": r["ms_merge"] * 1e3},
+                         "merge": r["ms_merge"] * 1e3,
+                         "step_as_two_launches": r["ms_per_step_two_launches"] * 1e3},
         "roofline": {"bound": "hbm", "kernel": "splitkv_kernel<1,bf16,8 waves>",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,

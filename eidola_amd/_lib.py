@@ -72,6 +72,8 @@ class AttnArgs(C.Structure):
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
         ("split_done_event", C.c_void_p),
+        ("k_new", C.c_void_p),
+        ("v_new", C.c_void_p),
     ]
 
 

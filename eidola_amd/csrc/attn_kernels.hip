@@ -150,8 +150,45 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
   }
 }
 
+// Software round-to-nearest-even onto the OCP e4m3fn grid, saturating at +-448; NaN -> 0x7F.
+__device__ __forceinline__ uint32_t fp8_e4m3_encode(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return 0x7Fu;
+  if (a >= 0x43E00000u) return sign | 0x7Eu;  // |x| >= 448
+  if (a >= (121u << 23)) {                    // normal in e4m3: |x| >= 2^-6
+    uint32_t r = a + 0x7FFFFu + ((a >> 20) & 1u);
+    r >>= 20;  // exponent and 3 mantissa bits, carry propagated
+    return sign | (r - (120u << 3));
+  }
+  // subnormal: multiples of 2^-9; 8 rounds up into the smallest normal (0x08)
+  const float y = __uint_as_float(a) * 512.0f;
+  return sign | (uint32_t)__float2int_rn(y);
+}
+
+// 16 bf16 values -> 16 fp8-e4m3fn bytes, RNE of x / scale (the arithmetic of kv_write_kernel)
+__device__ __forceinline__ u32x4 quantize16_fp8(const u32x4 lo, const u32x4 hi, const float sc) {
+  u32x4 o = {0, 0, 0, 0};
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t wv = j < 8 ? lo[j >> 1] : hi[(j - 8) >> 1];
+    const uint32_t h = (wv >> ((j & 1) * 16)) & 0xffffu;
+    o[j >> 2] |= fp8_e4m3_encode(__fdiv_rn(bf16_bits_to_f32(h), sc)) << ((j & 3) * 8);
+  }
+  return o;
+}
+
 // One wavefront attends rows [16*NT) over keys [t_begin, t_end) of sequence `s`.
 // t_begin is a multiple of 16.  Tokens >= seq_len are never used (K masked, V zeroed).
+//
+// Fused KV write (decode, NT == 1, p.k_new set): the sequence's newest token, position
+// seq_len - 1, has not been written to the cache yet.  The wave whose key range contains it
+// takes that row from k_new / v_new instead of from the cache (the lane that would have
+// loaded it swaps its registers) and stores it into the cache on the way, in the format
+// kv_write_kernel would have used, so the step needs no separate write launch.  Key ranges
+// of different partitions are disjoint and every wave owns one KV head: exactly one lane
+// group writes each (sequence, head) row, and nobody else reads it in this launch.
 template <int NT, bool FP8>
 __device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
                                        const int t_begin, const int t_end, const int seq_len,
@@ -181,6 +218,9 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   // The ids of iteration i+1 are fetched while iteration i is in flight.
   constexpr int kPages = 4;
   constexpr int kIter = kChunk;
+  // position of the token this launch writes itself, if it lies in [t_begin, t_end); else -1
+  const int pos_new = (NT == 1 && p.k_new && seq_len - 1 >= t_begin && seq_len - 1 < t_end)
+                          ? seq_len - 1 : -1;
   int blk[kPages];
 #pragma unroll
   for (int b = 0; b < kPages; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
@@ -204,6 +244,45 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         for (int e = 0; e < kElt; ++e) {
           kraw[b][e] = ldg128(kp + 16 * e);
           vraw[b][e] = ldg128(vp + 16 * e);
+        }
+      }
+    }
+    if (NT == 1 && pos_new >= ti && pos_new < ti + kIter) {  // wave-uniform, once per sequence
+      // One 16-byte piece at a time (K then V), so that the rare path adds few live registers
+      // to a loop that runs at the register limit of two workgroups per CU.
+      const int b_new = (pos_new - ti) >> 4;
+      const bool mine = i16 == (pos_new & 15);
+      const size_t src = ((size_t)s * Hkv + kvh) * kHeadDim + g * 16;
+      size_t dst = lane_off;
+#pragma unroll
+      for (int b = 0; b < kPages; ++b)
+        if (b == b_new) dst += (size_t)blk[b] * page_bytes;
+#pragma unroll
+      for (int kv = 0; kv < 2; ++kv) {
+        const uint16_t *from = (kv ? p.v_new : p.k_new) + src;
+        uint8_t *to = const_cast<uint8_t *>(kv ? p.v_cache : p.k_cache) + dst;
+        if constexpr (FP8) {
+          const float sc = (kv ? p.v_scale : p.k_scale)[kvh];
+          const u32x4 x = quantize16_fp8(*(const u32x4 *)from, *(const u32x4 *)(from + 8), sc);
+          if (mine) {
+            *(u32x4 *)to = x;
+#pragma unroll
+            for (int b = 0; b < kPages; ++b)
+              if (b == b_new) (kv ? vraw[b][0] : kraw[b][0]) = x;
+          }
+          asm volatile("" ::: "memory");
+        } else {
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            const u32x4 x = *(const u32x4 *)(from + 8 * e);
+            if (mine) {
+              *(u32x4 *)(to + 16 * e) = x;
+#pragma unroll
+              for (int b = 0; b < kPages; ++b)
+                if (b == b_new) (kv ? vraw[b][e * (kElt - 1)] : kraw[b][e * (kElt - 1)]) = x;
+            }
+            asm volatile("" ::: "memory");
+          }
         }
       }
     }
@@ -1040,23 +1119,6 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
 // Slot-mapped KV write.  grid = num_tokens, block = 128: thread e moves 8 elements of the
 // token's K row (first Hkv*8 threads) or V row (next Hkv*8 threads).
 // ---------------------------------------------------------------------------------------
-// Software round-to-nearest-even onto the OCP e4m3fn grid, saturating at +-448; NaN -> 0x7F.
-__device__ __forceinline__ uint32_t fp8_e4m3_encode(float x) {
-  const uint32_t u = __float_as_uint(x);
-  const uint32_t sign = (u >> 24) & 0x80u;
-  const uint32_t a = u & 0x7fffffffu;
-  if (a > 0x7f800000u) return 0x7Fu;
-  if (a >= 0x43E00000u) return sign | 0x7Eu;  // |x| >= 448
-  if (a >= (121u << 23)) {                    // normal in e4m3: |x| >= 2^-6
-    uint32_t r = a + 0x7FFFFu + ((a >> 20) & 1u);
-    r >>= 20;  // exponent and 3 mantissa bits, carry propagated
-    return sign | (r - (120u << 3));
-  }
-  // subnormal: multiples of 2^-9; 8 rounds up into the smallest normal (0x08)
-  const float y = __uint_as_float(a) * 512.0f;
-  return sign | (uint32_t)__float2int_rn(y);
-}
-
 template <bool FP8>
 __global__ __launch_bounds__(128) void kv_write_kernel(const uint16_t *__restrict__ k_new,
                                                        const uint16_t *__restrict__ v_new,

@@ -173,6 +173,8 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.sinks = a->sinks;
   p.k_scale = a->k_scale;
   p.v_scale = a->v_scale;
+  p.k_new = nullptr;  // set by eid_attn_decode only
+  p.v_new = nullptr;
   uint8_t *ws = static_cast<uint8_t *>(a->workspace);
   p.plan = nullptr;
   p.plan_slot = nullptr;
@@ -280,6 +282,12 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   p.cu_seqlens_q = nullptr;  // one row per sequence by contract
   p.qlen_lo = 1;
   p.qlen_hi = 1;
+  if ((args->k_new != nullptr) != (args->v_new != nullptr))
+    return fail(EID_ERR_INVALID_ARG, "k_new and v_new must both be given or both be NULL");
+  if (!aligned16(args->k_new) || !aligned16(args->v_new))
+    return fail(EID_ERR_INVALID_ARG, "k_new and v_new must be 16-byte aligned");
+  p.k_new = static_cast<const uint16_t *>(args->k_new);  // fused write of the newest token
+  p.v_new = static_cast<const uint16_t *>(args->v_new);
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
@@ -305,6 +313,8 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   g_err[0] = 0;
   if (int32_t rc = check_attn_desc(desc)) return rc;
   if (int32_t rc = check_attn_args(desc, args, true, true)) return rc;
+  if (args->k_new || args->v_new)
+    return fail(EID_ERR_INVALID_ARG, "k_new / v_new are taken by eid_attn_decode only");
   const Plan pl = make_plan(desc);
   eid::AttnParams p = make_params(desc, args, pl);
   hipStream_t st = static_cast<hipStream_t>(hip_stream);

@@ -22,6 +22,8 @@ struct AttnParams {
   float *lse;
   const uint8_t *k_cache;
   const uint8_t *v_cache;
+  const uint16_t *k_new;  // decode only, may be NULL: [num_seqs, Hkv, 64] bf16 rows of the newest
+  const uint16_t *v_new;  // token of every sequence, written into the caches by this launch
   const int32_t *block_table;
   const int32_t *cu_seqlens_q;  // may be null: q_len == 1 everywhere
   const int32_t *seq_lens;

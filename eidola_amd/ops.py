@@ -211,7 +211,7 @@ def yarn_cos_sin(max_pos, head_dim=64, base=150000.0, scaling_factor=32.0,
 
 def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q,
                max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace,
-               return_lse, sum_kv_len=0):
+               return_lse, sum_kv_len=0, k_new=None, v_new=None):
     _require(q, "q", torch.bfloat16, 3)
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
@@ -261,6 +261,12 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
     args.v_scale = v_scale.data_ptr() if v_scale is not None else None
     args.workspace = workspace.data_ptr()
     args.workspace_bytes = workspace.numel() * workspace.element_size()
+    for name, t in (("k_new", k_new), ("v_new", v_new)):
+        if t is not None:
+            _require(t, name, torch.bfloat16, 3)
+            if tuple(t.shape) != (S, geom.num_kv_heads, geom.head_dim):
+                raise ValueError(f"{name} must be [num_seqs, num_kv_heads, head_dim]")
+            setattr(args, name, t.data_ptr())
     check(getattr(lib, fn_name)(C.byref(desc), C.byref(args), _stream()))
     return (out, lse) if return_lse else out
 
@@ -285,7 +291,7 @@ class PreparedCall:
 
 def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, *,
             max_q_len=1, max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
-            workspace=None, sum_kv_len=0):
+            workspace=None, sum_kv_len=0, k_new=None, v_new=None):
     """Build a PreparedCall for "eid_attn_decode" / "eid_attn_varlen" / "eid_lse_merge"."""
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
@@ -314,19 +320,23 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
     args.v_scale = v_scale.data_ptr() if v_scale is not None else None
     args.workspace = workspace.data_ptr()
     args.workspace_bytes = workspace.numel()
+    args.k_new = k_new.data_ptr() if k_new is not None else None
+    args.v_new = v_new.data_ptr() if v_new is not None else None
     keep = (q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, sinks, k_scale, v_scale,
-            workspace)
+            k_new, v_new, workspace)  # workspace stays last: callers share it via _keep[-1]
     return PreparedCall(fn_name, desc, args, keep, out, lse)
 
 
 def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, sinks=None,
                 k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
-                return_lse=False, sum_kv_len=0):
+                return_lse=False, sum_kv_len=0, k_new=None, v_new=None):
     """Stages K2+K4: one query row per sequence (q is [num_seqs, Hq, D]).  `sum_kv_len` is the
-    optional host-side sum of seq_lens (any upper bound): it sizes the launch to the work."""
+    optional host-side sum of seq_lens (any upper bound): it sizes the launch to the work.
+    With `k_new` / `v_new` ([num_seqs, Hkv, D] bf16: the newest token of every sequence, not
+    yet in the cache) the call writes those rows into the caches itself (stage K1 fused)."""
     return _attn_call("eid_attn_decode", geom, q, k_cache, v_cache, block_table, seq_lens, None,
                       1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse,
-                      sum_kv_len)
+                      sum_kv_len, k_new, v_new)
 
 
 def attn_varlen(geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, *, max_q_len,

@@ -105,6 +105,13 @@ typedef struct eid_attn_args {
                              stream right after the split-KV launch of the q_len <= 2 class,
                              i.e. before its merge, so that a caller who records an event of
                              his own before the call can time that kernel by itself */
+  const void *k_new;    /* eid_attn_decode only, optional (both or neither): [num_seqs, Hkv, 64] */
+  const void *v_new;    /* bf16 rows of every sequence's newest token (position seq_lens[s]-1),
+                           NOT yet in the cache.  The call then writes them into k_cache /
+                           v_cache itself (same bits as eid_kv_write to slot
+                           block_table[s][pos/16]*16 + pos%16) and attends to them from
+                           registers: the step needs no separate eid_kv_write launch.
+                           k_cache / v_cache are written in that case. */
 } eid_attn_args;
 
 /*
