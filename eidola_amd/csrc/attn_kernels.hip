@@ -12,6 +12,7 @@
 //   O^T[dim][row] += V^T[dim][token] . P^T[token][row], with V staged row-major in LDS and
 //        read back transposed by ds_read_b64_tr_b16.
 // "row" = (query token, query head of the KV group): 8 heads share every K/V byte.
+#include <atomic>
 #include "eid_device.h"
 #include "eid_params.h"
 
@@ -1328,7 +1329,25 @@ static long long item_bound(const AttnParams &p) {
 template <int NT, bool FP8, int WAVES>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
   dim3 grid((unsigned)item_bound(p), p.num_kv_heads / WAVES);
-  splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, 0, st>>>(p);
+  // One 8-wave workgroup per CU.  A second resident workgroup adds nothing for a kernel that
+  // streams from HBM (measured: the same or up to 4 % slower with two), while half of the
+  // CU's registers left free let a prefill workgroup of a mixed batch run beside it.  The
+  // cap is a request for unused dynamic LDS: two such workgroups no longer fit a CU's 160 KB,
+  // one plus a prefill workgroup does.
+  constexpr int kPad = WAVES == 8 ? 16384 : 0;
+  if (kPad > 0) {  // once per device: allow the kernel its dynamic LDS on top of the static tile
+    static std::atomic<bool> allowed[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
+      e = hipFuncSetAttribute((const void *)splitkv_kernel<NT, FP8, WAVES>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kPad);
+      if (e != hipSuccess) return e;
+      if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
+    }
+  }
+  splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, kPad, st>>>(p);
   return hipGetLastError();
 }
 

@@ -195,6 +195,32 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   return p;
 }
 
+// Helper stream of the calling thread on the current device: the prefill launch of a mixed
+// batch runs there, beside the split-KV launches on the caller's stream (fork and join by
+// events, so the caller sees one stream's worth of ordering).  Created on first use at the
+// default priority and kept for the life of the thread; nullptr if creation fails (the call
+// then runs its launches one after the other).
+struct Helper {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  bool tried = false, ok = false;
+};
+Helper *helper_stream() {
+  constexpr int kMaxDevices = 64;
+  thread_local Helper helpers[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  Helper &h = helpers[dev];
+  if (!h.tried) {
+    h.tried = true;
+    h.ok = hipStreamCreateWithFlags(&h.stream, hipStreamNonBlocking) == hipSuccess &&
+           hipEventCreateWithFlags(&h.fork, hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&h.join, hipEventDisableTiming) == hipSuccess;
+    if (!h.ok) (void)hipGetLastError();  // not sticky: the sequential path follows
+  }
+  return h.ok ? &h : nullptr;
+}
+
 int32_t hip_fail(hipError_t e, const char *what) {
   return fail(EID_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
@@ -331,6 +357,17 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
       eid::shortspan_applies(1, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
   const bool short3 = pl.nparts_max == 1 &&
       eid::shortspan_applies(3, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
+  // Mixed batch: the MFMA-bound prefill launch and the HBM-bound split-KV launches use
+  // different halves of the machine, so they run side by side: prefill on the thread's
+  // helper stream, forked from and joined back into the caller's stream.
+  const bool has_prefill = desc->max_q_len > eid::kShortQMax;
+  static const bool serial = getenv("EID_SERIAL_CLASSES") != nullptr;  // for A/B measurements
+  Helper *hs = (has_prefill && !only_prefill && !serial) ? helper_stream() : nullptr;
+  if (hs) {
+    e = hipEventRecord(hs->fork, st);
+    if (e == hipSuccess) e = hipStreamWaitEvent(hs->stream, hs->fork, 0);
+    if (e != hipSuccess) return hip_fail(e, "fork to the helper stream");
+  }
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
   if (!only_verify && !only_prefill) {
@@ -340,6 +377,14 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     e = short1 ? eid::launch_shortspan(p, 1, fp8, st)
                : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
     if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+  }
+  if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
+    eid::AttnParams pp = p;
+    pp.qlen_lo = eid::kShortQMax + 1;
+    pp.qlen_hi = 0x7fffffff;
+    e = eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream);
+    if (e == hipSuccess) e = hipEventRecord(hs->join, hs->stream);
+    if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
   }
   if (args->split_done_event) {
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
@@ -361,7 +406,10 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
       if (e != hipSuccess) return hip_fail(e, "merge launch");
     }
   }
-  if (desc->max_q_len > eid::kShortQMax) {  // long chunks: MFMA prefill kernel
+  if (hs) {
+    e = hipStreamWaitEvent(st, hs->join, 0);
+    if (e != hipSuccess) return hip_fail(e, "join of the helper stream");
+  } else if (has_prefill) {  // long chunks: MFMA prefill kernel
     p.qlen_lo = eid::kShortQMax + 1;
     p.qlen_hi = 0x7fffffff;
     e = eid::launch_prefill(p, desc->num_q_tokens, fp8, st);

@@ -593,3 +593,84 @@ def test_step_replayed_from_a_hip_graph(G):
         step()                      # eager work between replays
         torch.cuda.synchronize()
         assert torch.equal(call.out, eager)
+
+
+def _mixed_call(G, seed=41):
+    """A mixed batch (prefill chunks, verify rows, decodes): its prefill launch runs on the
+    library's helper stream beside the split-KV launches."""
+    b = make_batch([900, 64, 3000, 200, 1500, 77, 2600], [256, 1, 1, 5, 40, 1, 2], seed=seed)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    call = ea.prepare("eid_attn_varlen", b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table),
+                      G.dev(b.seq_lens), G.dev(b.cu_seqlens_q), max_q_len=b.max_q_len,
+                      max_kv_len=b.max_kv_len, sinks=G.dev(sinks), sum_kv_len=int(b.seq_lens.sum()))
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    return b, call, ref
+
+
+def test_mixed_batch_replayed_from_a_hip_graph(G):
+    """The fork to the helper stream and the join back are captured with the launches: every
+    replay must reproduce the eager result, with eager work in between."""
+    b, call, ref = _mixed_call(G)
+    call()
+    torch.cuda.synchronize()
+    eager = call.out.clone()
+    assert_close(G.bits_host(eager), ref, "mixed eager")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call()                      # the thread's helper stream exists before capture starts
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            call()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for i in range(4):
+        call.out.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(call.out, eager), f"replay {i}"
+        call()
+        torch.cuda.synchronize()
+        assert torch.equal(call.out, eager)
+
+
+def test_mixed_batches_from_two_host_threads(G):
+    """Two host threads, each with its own stream, workspace and output, issue mixed batches at
+    the same time: every thread owns its helper stream, results equal the single-threaded ones."""
+    import threading
+    cases = [_mixed_call(G, seed=51), _mixed_call(G, seed=52)]
+    want = []
+    for _, call, ref in cases:
+        call()
+        torch.cuda.synchronize()
+        assert_close(G.bits_host(call.out), ref, "mixed single-threaded")
+        want.append(call.out.clone())
+    errors = []
+
+    def worker(i):
+        try:
+            torch.cuda.set_device(0)
+            st = torch.cuda.Stream()
+            _, call, _ = cases[i]
+            for it in range(20):
+                call.out.zero_()            # on the default stream of this thread ...
+                st.wait_stream(torch.cuda.current_stream())
+                call(stream=st.cuda_stream)
+                st.synchronize()
+                if not torch.equal(call.out, want[i]):
+                    errors.append((i, it))
+                    return
+        except Exception as ex:  # surfaced below
+            errors.append((i, repr(ex)))
+
+    ts = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
