@@ -409,6 +409,9 @@ def main():
                     help="experiment: physically contiguous pages instead of a shuffled pool")
     ap.add_argument("--no-hint", action="store_true",
                     help="experiment: leave desc.sum_kv_len at 0 (grid sized from max_kv_len)")
+    ap.add_argument("--only", default="",
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj "
+                         "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
                          "instead of one eid_attn_decode call that takes k_new / v_new")
@@ -468,36 +471,47 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if a.all:
+        only = set(x for x in a.only.split(",") if x)
+        want = lambda name: not only or name in only
         w = None
         torch.cuda.empty_cache()
-        ww = Workload(lambda off: synth.config2(window=128, perm_offset=off), a.sets, 7, torch, ea,
-                      synth, "decode")
-        extra.append(measure(ww, a.steps, a.warmup, torch, synth, "config2_decode_w128"))
-        ww = None
-        torch.cuda.empty_cache()
-        w3 = Workload(lambda off: synth.config3(perm_offset=off), 4, 8, torch, ea, synth, "varlen")
-        r3 = measure(w3, max(20, a.steps // 4), a.warmup, torch, synth, "config3_mixed")
-        lw = synth.algorithmic_work(w3.batches[0], rows="long")
-        sw = synth.algorithmic_work(w3.batches[0], rows="short")
-        r3["prefill_flops"], r3["decode_rows_bytes"] = lw["flops"], sw["bytes"]
-        extra.append(r3)
-        w3 = None
-        torch.cuda.empty_cache()
-        w4 = Workload(lambda off: synth.config4(num_blocks=300_000, perm_offset=off), 3, 9, torch,
-                      ea, synth, "decode")
-        extra.append(measure(w4, max(20, a.steps // 2), a.warmup, torch, synth, "config4_fp8_decode"))
-        w4 = None
-        torch.cuda.empty_cache()
+        if want("2w"):
+            ww = Workload(lambda off: synth.config2(window=128, perm_offset=off), a.sets, 7, torch,
+                          ea, synth, "decode")
+            extra.append(measure(ww, a.steps, a.warmup, torch, synth, "config2_decode_w128"))
+            ww = None
+            torch.cuda.empty_cache()
+        if want("3"):
+            w3 = Workload(lambda off: synth.config3(perm_offset=off), 4, 8, torch, ea, synth, "varlen")
+            r3 = measure(w3, max(20, a.steps // 4), a.warmup, torch, synth, "config3_mixed")
+            lw = synth.algorithmic_work(w3.batches[0], rows="long")
+            sw = synth.algorithmic_work(w3.batches[0], rows="short")
+            r3["prefill_flops"], r3["decode_rows_bytes"] = lw["flops"], sw["bytes"]
+            extra.append(r3)
+            w3 = None
+            torch.cuda.empty_cache()
+        if want("4"):
+            w4 = Workload(lambda off: synth.config4(num_blocks=300_000, perm_offset=off), 3, 9,
+                          torch, ea, synth, "decode")
+            extra.append(measure(w4, max(20, a.steps // 2), a.warmup, torch, synth,
+                                 "config4_fp8_decode"))
+            w4 = None
+            torch.cuda.empty_cache()
         for layer in (0, 1):
+            if not want("5"):
+                break
             w5 = Workload(lambda off: synth.config5(layer=layer, num_blocks=900_000, perm_offset=off),
                           3, 10 + layer, torch, ea, synth, "varlen")
             extra.append(measure(w5, max(10, a.steps // 10), max(3, a.warmup // 4), torch, synth,
                                  f"config5_verify_layer{layer}"))
             w5 = None
             torch.cuda.empty_cache()
-        extra.append(sched_bench(synth, ea))
-        extra.extend(rope_bench(torch, ea, synth))
-        extra.extend(oproj_bench(torch, ea))
+        if want("sched"):
+            extra.append(sched_bench(synth, ea))
+        if want("rope"):
+            extra.extend(rope_bench(torch, ea, synth))
+        if want("oproj"):
+            extra.extend(oproj_bench(torch, ea))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)
