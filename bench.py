@@ -506,6 +506,15 @@ def main():
                                  f"config5_verify_layer{layer}"))
             w5 = None
             torch.cuda.empty_cache()
+            if layer == 0:
+                # BASELINE words this configuration with 512-token partitions; the same batch
+                # with the partition left to the library (desc.partition_size = 0)
+                w5 = Workload(lambda off: synth.config5(layer=0, num_blocks=900_000, perm_offset=off)
+                              .with_geom(partition_size=0), 3, 10, torch, ea, synth, "varlen")
+                extra.append(measure(w5, max(10, a.steps // 10), max(3, a.warmup // 4), torch,
+                                     synth, "config5_verify_layer0_runtime_partition"))
+                w5 = None
+                torch.cuda.empty_cache()
         if want("sched"):
             extra.append(sched_bench(synth, ea))
         if want("rope"):
