@@ -18,8 +18,9 @@
 //                        streamed once.  One workgroup per 16 features; its 8 waves deal the
 //                        K dimension in 64-element chunks, each wave keeps a whole batch of
 //                        weight loads in flight, the partial sums meet in LDS.
-//   oproj_tiled_kernel   any T.  MFMA-bound: 128 tokens x 128 features per workgroup, K in
-//                        steps of 64 through double-buffered, row-padded LDS tiles.
+//   oproj_tiled_kernel   any T.  128 x 128 (or, for batches too small to fill the device
+//                        with that, 64 x 64) tokens x features per workgroup, K in steps of
+//                        64 through double-buffered, row-padded LDS tiles.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
