@@ -481,6 +481,21 @@ __device__ __forceinline__ long long wave_total64(const long long v) {
   const long long c = wave_total((int)(v >> 44));
   return a + (b << 22) + (c << 44);
 }
+// Maximum over the 64 lanes of a value >= 0, wave-uniform (same DPP ladder as the scan; a lane
+// without a source takes 0).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_max(const int v) {
+  return max(v, __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ int wave_max(int v) {
+  v = dpp_max<0x111, 0xf>(v);
+  v = dpp_max<0x112, 0xf>(v);
+  v = dpp_max<0x114, 0xf>(v);
+  v = dpp_max<0x118, 0xf>(v);
+  v = dpp_max<0x142, 0xa>(v);
+  v = dpp_max<0x143, 0xc>(v);
+  return __builtin_amdgcn_readlane(v, 63);
+}
 // a / b for wave-uniform a >= 0, b > 0: the 64-bit division expands to some hundred
 // instructions, the 32-bit one to a third of that, and batches rarely need the former.
 __device__ __forceinline__ long long uniform_div(const long long a, const long long b) {
@@ -527,35 +542,46 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
   if (!p.dynamic_partition) return p.partition;
   const int lane = threadIdx.x & 63;
   long long total = first.span;
+  int longest = first.span;
   int active = __popcll(__ballot(first.span > 0));
   for (int s0 = 64; s0 < p.num_seqs; s0 += 64) {
     const SeqView v = view_seq(p, s0 + lane);
     total += v.span;
+    longest = max(longest, v.span);
     active += __popcll(__ballot(v.span > 0));
   }
   total = wave_total64(total);
+  longest = wave_max(longest);
   const long long T = max(p.target_items, 1);
   // (every value below is the same in all lanes and lives in scalar registers, and so does
   // everything derived from the partition)
   // Smallest multiple of 64 (>= the planning minimum, < the cap) whose exact item count
-  // is <= Tx, or 0 if there is none.
+  // is <= Tx, or 0 if there is none.  Two sizes are known to fit: the pessimistic bound
+  // total / (Tx - active) (every sequence may add one short item), and the longest span,
+  // which makes every sequence a single item (the only way when active == Tx).  The exact
+  // count falls as the partition grows, so the smallest fitting size below the better of
+  // the two is found by bisection (a handful of counts).
   auto single_fill = [&](const long long Tx) -> int {
-    if (active >= Tx) return 0;
-    // items <= total/P + active <= Tx
-    long long P = (uniform_div(total + (Tx - active) - 1, Tx - active) + 63) / 64 * 64;
-    P = max(P, (long long)p.partition);
-    if (P >= kDynPartitionCap) return 0;
-    // The bound is pessimistic by up to one item per sequence: walk down while the exact
-    // count still fits.
-    for (int step = 0; step < 4 && P - 64 >= p.partition; ++step) {
-      const int Pc = (int)P - 64;
+    if (active > Tx) return 0;
+    long long hi = ((long long)longest + 63) / 64 * 64;
+    if (active < Tx)
+      hi = min(hi, (uniform_div(total + (Tx - active) - 1, Tx - active) + 63) / 64 * 64);
+    hi = max(hi, (long long)p.partition);
+    if (hi >= kDynPartitionCap) return 0;
+    int lo_i = p.partition / 64, hi_i = (int)hi / 64 - 1, P = (int)hi;
+    while (lo_i <= hi_i) {
+      const int mid = (lo_i + hi_i) >> 1, Pc = mid * 64;
       int items = num_partitions(p, first.span, Pc);
       for (int s0 = 64; s0 < p.num_seqs; s0 += 64)
         items += num_partitions(p, view_seq(p, s0 + lane).span, Pc);
-      if (wave_total64(items) > Tx) break;
-      P = Pc;
+      if (wave_total64(items) <= Tx) {
+        P = Pc;
+        hi_i = mid - 1;
+      } else {
+        lo_i = mid + 1;
+      }
     }
-    return (int)P;
+    return P;
   };
   // one workgroup per CU if the batch is small enough for that, else one device fill
   if (p.target_items_lo < T) {
@@ -563,7 +589,19 @@ __device__ __forceinline__ int effective_partition(const AttnParams &p, const Se
     if (P) return P;
   }
   if (const int P = single_fill(T)) return P;
-  // more than one fill: aim at about three fills of equal items, within [floor, cap]
+  // More than one fill.  At least one sequence per CU and none longer than the cap: every
+  // sequence is one item (no partials, no merge); the dispatcher evens out ragged lengths
+  // over the rounds.
+  const int whole = (longest + 63) / 64 * 64;
+  if (active >= p.target_items_lo && whole <= kDynPartitionCap) return max(whole, p.partition);
+  // Nearly uniform lengths (longest within a quarter of the mean): equal pieces of every
+  // sequence, as few as the cap allows; there is no raggedness for small items to even out,
+  // and every item pays a prologue and a partial.
+  if ((long long)longest * active * 4 <= total * 5) {
+    const int pieces = (longest + kDynPartitionCap - 1) / kDynPartitionCap;
+    return max(((longest + pieces - 1) / pieces + 63) / 64 * 64, p.partition);
+  }
+  // Ragged: aim at about three fills of equal items, within [floor, cap]
   return (int)min((long long)kDynPartitionCap,
                   max((long long)kDynPartitionFloor, (uniform_div(total, 3 * T) + 63) / 64 * 64));
 }
@@ -1314,8 +1352,9 @@ static long long item_bound(const AttnParams &p) {
       auto takes_tier = [&](const long long Tx) {
         return S < Tx && ((sum + (Tx - S) - 1) / (Tx - S) + 63) / 64 * 64 < kDynPartitionCap;
       };
+      // (the equal-pieces rule for nearly uniform batches never goes below half the cap)
       const long long multi =
-          min(sum / kDynPartitionFloor, max(sum / kDynPartitionCap, 3 * T)) + S + 16;
+          min(sum / kDynPartitionFloor, max(2 * sum / kDynPartitionCap, 3 * T)) + S + 16;
       if (Tlo < T && takes_tier(Tlo)) items = min(items, Tlo);
       else if (takes_tier(T)) items = min(items, T);
       else items = min(items, max(T, multi));
@@ -1329,12 +1368,12 @@ static long long item_bound(const AttnParams &p) {
 template <int NT, bool FP8, int WAVES>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
   dim3 grid((unsigned)item_bound(p), p.num_kv_heads / WAVES);
-  // One 8-wave workgroup per CU.  A second resident workgroup adds nothing for a kernel that
-  // streams from HBM (measured: the same or up to 4 % slower with two), while half of the
-  // CU's registers left free let a prefill workgroup of a mixed batch run beside it.  The
-  // cap is a request for unused dynamic LDS: two such workgroups no longer fit a CU's 160 KB,
-  // one plus a prefill workgroup does.
-  constexpr int kPad = WAVES == 8 ? 16384 : 0;
+  // With a prefill launch beside it (mixed batch, p.share_cus): one 8-wave workgroup per CU.
+  // A second resident workgroup adds little to a kernel that streams from HBM (it only
+  // covers the prologues of many short items), while half of the CU's registers left free
+  // let a prefill workgroup run next to it.  The cap is a request for unused dynamic LDS: two
+  // such workgroups no longer fit a CU's 160 KB, one plus a prefill workgroup does.
+  const int kPad = (WAVES == 8 && p.share_cus) ? 16384 : 0;
   if (kPad > 0) {  // once per device: allow the kernel its dynamic LDS on top of the static tile
     static std::atomic<bool> allowed[64];
     int dev = 0;

@@ -21,6 +21,7 @@ hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
                                 uint8_t *k_cache, uint8_t *v_cache, const int64_t *slot_mapping,
                                 const float *k_scale, const float *v_scale, int Hq, int Hkv,
                                 int64_t num_slots, int num_tokens, bool fp8, hipStream_t st);
+int device_cus();
 hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
                          const uint16_t *resid, uint16_t *out, int T, int N, int K,
                          hipStream_t st);
@@ -127,9 +128,17 @@ Plan make_plan(const eid_attn_desc *d) {
   const int32_t span = max_span(d);
   // partition_size == 0: the kernels size the partition from the batch at run time, never
   // below kDynPartitionMin, which therefore bounds the partition count for the workspace.
-  const int32_t P = d->partition_size ? d->partition_size : eid::kDynPartitionMin;
-  pl.partition = P;
+  int32_t P = d->partition_size ? d->partition_size : eid::kDynPartitionMin;
   pl.dynamic = d->partition_size == 0;
+  // ... unless the host can already tell what they would choose: with at least one sequence
+  // per CU and no span beyond the partition cap, every sequence is one work item.  Planning
+  // it here makes the kernels map workgroup w to sequence w with no scan of seq_lens at all
+  // (with hundreds of sequences the scans are a fifth of the run time) and no partials.
+  if (pl.dynamic && d->num_seqs >= eid::device_cus() && span <= eid::kDynPartitionCap) {
+    P = (span + 63) / 64 * 64;
+    pl.dynamic = false;
+  }
+  pl.partition = P;
   pl.nparts_max = (span + P - 1) / P;
   pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
@@ -363,6 +372,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool has_prefill = desc->max_q_len > eid::kShortQMax;
   static const bool serial = getenv("EID_SERIAL_CLASSES") != nullptr;  // for A/B measurements
   Helper *hs = (has_prefill && !only_prefill && !serial) ? helper_stream() : nullptr;
+  p.share_cus = hs ? 1 : 0;
   if (hs) {
     e = hipEventRecord(hs->fork, st);
     if (e == hipSuccess) e = hipStreamWaitEvent(hs->stream, hs->fork, 0);

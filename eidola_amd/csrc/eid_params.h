@@ -41,6 +41,8 @@ struct AttnParams {
   int32_t qlen_lo, qlen_hi;  // this launch serves sequences with qlen_lo <= q_len <= qlen_hi
   int32_t dynamic_partition; // 1: kernels derive the partition from the batch (>= partition)
   int32_t target_items;      // workgroups the device holds at once (dynamic partition only)
+  int32_t share_cus;         // host-side launch flag: 1 = hold the split-KV kernel to one
+                             // workgroup per CU (a prefill launch runs beside it)
   float softmax_scale;
 };
 

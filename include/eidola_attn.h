@@ -217,8 +217,10 @@ int32_t eid_o_proj(const void *attn_out, const void *weight, const void *bias,
  * Returns 0 for an invalid desc. */
 size_t eid_workspace_bytes(const eid_attn_desc *desc);
 
-/* The partition size (tokens) the workspace is planned with: desc->partition_size, or the
- * lower bound 256 of the run-time choice when that is 0. */
+/* The partition size (tokens) the workspace is planned with: desc->partition_size; when that
+ * is 0, the lower bound 256 of the kernels' run-time choice, or, for a batch with at least
+ * one sequence per compute unit whose longest span fits one partition (2,048 tokens), that
+ * span rounded up to 64: every sequence is then one work item and no partials are written. */
 int32_t eid_partition_size(const eid_attn_desc *desc);
 
 /* Thread-local description of the last error on this thread; "" if none. */

@@ -48,6 +48,17 @@ def test_workspace_and_partition_planning():
                       max_q_len=5, max_kv_len=65536, max_blocks_per_seq=4096, num_blocks=300000)
     assert ea.partition_size(d5) == 512
     assert ea.workspace_bytes(d5) == 256 + 128 * 5 * 64 * 128 * (8 + 128)
+    # at least one sequence per CU (256 without a device to ask) and no span beyond 2,048
+    # tokens: every sequence is planned as one work item, and the workspace shrinks to it
+    dm = ea.make_desc(ea.AttnGeometry(), num_seqs=300, num_q_tokens=300, max_q_len=1,
+                      max_kv_len=1300, max_blocks_per_seq=82, num_blocks=300000)
+    assert ea.partition_size(dm) == 1344
+    assert ea.workspace_bytes(dm) == 256 + 300 * 64 * (8 + 128)
+    dm.max_kv_len, dm.max_blocks_per_seq = 2049, 129
+    assert ea.partition_size(dm) == 256
+    dm.num_seqs = dm.num_q_tokens = 255
+    dm.max_kv_len = 1300
+    assert ea.partition_size(dm) == 256
     dw = ea.make_desc(ea.AttnGeometry(window=128), num_seqs=64, num_q_tokens=64, max_q_len=1,
                       max_kv_len=8192, max_blocks_per_seq=512, num_blocks=300000)
     assert ea.workspace_bytes(dw) < ea.workspace_bytes(good_desc(num_seqs=64, num_q_tokens=64,

@@ -226,6 +226,42 @@ def test_many_sequences_cross_the_64_wide_scan(G):
         assert np.array_equal(G.run_attn(b, q, kc_d, vc_d, sinks, hint=True), out)
 
 
+@pytest.mark.parametrize("kind", ["decode", "mixed", "uniform", "one_long"])
+def test_at_least_one_sequence_per_cu(G, kind):
+    """300 and more sequences.  With no span beyond 2,048 tokens the host plans every sequence
+    as one work item (no partials); one longer sequence sends the batch back to the run-time
+    rule (several fills, or equal pieces when the lengths are uniform)."""
+    rng = np.random.default_rng(17)
+    S = 300
+    if kind == "decode":
+        q_lens = np.ones(S, np.int64)
+        seq_lens = rng.integers(1, 1300, size=S)
+    elif kind == "mixed":
+        q_lens = rng.choice([1, 1, 1, 2, 5, 6, 20], size=S)
+        seq_lens = q_lens + rng.integers(0, 900, size=S)
+    elif kind == "uniform":
+        q_lens = np.ones(S, np.int64)
+        seq_lens = np.full(S, 2304)            # beyond the cap: two equal pieces each
+    else:
+        q_lens = np.ones(S, np.int64)
+        seq_lens = rng.integers(1, 700, size=S)
+        seq_lens[123] = 5000
+    b = make_batch(seq_lens, q_lens, seed=19)
+    d = desc_of(b)
+    if kind in ("decode", "mixed"):
+        assert ea.partition_size(d) == (int(seq_lens.max()) + 63) // 64 * 64
+    else:
+        assert ea.partition_size(d) == 256      # run-time choice, planned from its lower bound
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True, hint=True)
+    assert_close(out, ref, f"300 sequences, {kind}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+    assert np.array_equal(G.run_attn(b, q, kc_d, vc_d, sinks), out)     # without the hint
+
+
 @pytest.mark.parametrize("hkv", [1, 4, 16])
 def test_other_kv_head_counts(G, hkv):
     b = make_batch([300, 40, 1, 77], [1, 5, 1, 40], num_kv_heads=hkv, partition=128)
