@@ -262,6 +262,25 @@ def test_at_least_one_sequence_per_cu(G, kind):
     assert np.array_equal(G.run_attn(b, q, kc_d, vc_d, sinks), out)     # without the hint
 
 
+def test_loose_max_kv_len_leaves_the_choice_to_the_kernels(G):
+    """300 short sequences declared with max_kv_len = 4,096: the host cannot plan whole
+    sequences, the kernels find out by themselves that every sequence is one item."""
+    rng = np.random.default_rng(23)
+    seq_lens = rng.integers(1, 700, size=300)
+    b = make_batch(seq_lens, np.ones(300, np.int64), seed=29)
+    q, k, v, sinks = logical_tensors(b)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    bt = np.zeros((300, 256), np.int32)
+    bt[:, :b.block_table.shape[1]] = b.block_table
+    for hint in (0, int(seq_lens.sum())):
+        out = ea.attn_decode(b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(bt), G.dev(b.seq_lens),
+                             max_kv_len=4096, sinks=G.dev(sinks), sum_kv_len=hint)
+        torch.cuda.synchronize()
+        assert_close(G.bits_host(out), ref, f"loose bound, hint {hint}")
+
+
 @pytest.mark.parametrize("hkv", [1, 4, 16])
 def test_other_kv_head_counts(G, hkv):
     b = make_batch([300, 40, 1, 77], [1, 5, 1, 40], num_kv_heads=hkv, partition=128)
