@@ -342,6 +342,38 @@ def oproj_bench(torch, ea):
     return out
 
 
+def prefill_bench(torch, ea, synth):
+    """Chunked prefill of ONE long prompt: a 512-token and a 2,048-token chunk behind 60,000
+    tokens of context (few query tiles, so the prefill kernel splits every tile's key range),
+    and an 8,192-token chunk without prior.  MFMA-bound: 16,384 FLOP per unmasked pair."""
+    import numpy as np
+    g = ea.AttnGeometry()
+    nb = 300_000
+    kc = torch.empty((nb, 16, 8, 64), dtype=torch.bfloat16, device="cuda:0")
+    vc = torch.empty_like(kc)
+    synth.fill_pool_gpu(g, kc, vc, 12)
+    sinks = torch.zeros(64, device="cuda:0")
+    out = []
+    for new, prior in ((512, 60_000), (2048, 60_000), (8192, 0)):
+        lens = np.array([new + prior], np.int32)
+        q = torch.randn((new, 64, 64), device="cuda:0").to(torch.bfloat16)
+        bt = torch.from_numpy(synth.build_block_table(lens, nb, 12)).to("cuda:0")
+        call = ea.prepare("eid_attn_varlen", g, q, kc, vc, bt, torch.from_numpy(lens).to("cuda:0"),
+                          torch.tensor([0, new], dtype=torch.int32, device="cuda:0"),
+                          max_q_len=new, max_kv_len=new + prior, sinks=sinks,
+                          sum_kv_len=new + prior)
+        for _ in range(3):
+            call()
+        ms = event_ms(lambda i: call(), 10, torch)
+        flops = 16384.0 * (new * prior + new * (new + 1) // 2)
+        r = {"config": f"prefill_{new}_new_after_{prior}", "ms": ms, "flops": flops,
+             "TFLOPs": flops / ms / 1e9}
+        log(f"[bench] prefill, {new} new tokens after {prior}: {ms*1e3:.1f} us, "
+            f"{r['TFLOPs']:.0f} TFLOP/s = {100*r['TFLOPs']/MFMA_BF16_PEAK_TFLOPS:.1f}% of bf16 MFMA peak")
+        out.append(r)
+    return out
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -410,7 +442,7 @@ def main():
     ap.add_argument("--no-hint", action="store_true",
                     help="experiment: leave desc.sum_kv_len at 0 (grid sized from max_kv_len)")
     ap.add_argument("--only", default="",
-                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj "
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill "
                          "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
@@ -521,6 +553,8 @@ def main():
             extra.extend(rope_bench(torch, ea, synth))
         if want("oproj"):
             extra.extend(oproj_bench(torch, ea))
+        if want("prefill"):
+            extra.extend(prefill_bench(torch, ea, synth))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)

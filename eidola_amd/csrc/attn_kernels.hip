@@ -922,11 +922,16 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int i16 = lane & 15, g = lane >> 4;
   const int Hkv = p.num_kv_heads;
   const int kvh = blockIdx.x % Hkv;
+  // Key-range split (few tiles, long contexts): `KS` consecutive units share one tile and
+  // take one part of its key range each.
+  const int KS = p.pf_splits;
+  const int unit = blockIdx.x / Hkv;
+  const int ks_part = KS > 1 ? unit % KS : 0;
   // one wave looks the item up, the others receive it through LDS
   __shared__ int item_lds[8];
   if (wave == 0) {
     int s0 = 0, tile0 = 0, row00 = 0, qlen0 = 0, L0 = 0;
-    const bool found = find_prefill_item(p, blockIdx.x / Hkv, s0, tile0, row00, qlen0, L0);
+    const bool found = find_prefill_item(p, KS > 1 ? unit / KS : unit, s0, tile0, row00, qlen0, L0);
     if (lane == 0) {
       item_lds[0] = found;
       item_lds[1] = s0;
@@ -949,8 +954,13 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int tq_wg = tile * kPfTok;
   const int pos_first_wg = pos0 + tq_wg;
   const int pos_last_wg = pos0 + min(tq_wg + kPfTok, qlen) - 1;
-  const int t_begin = (W > 0 ? max(0, pos_first_wg - W + 1) : 0) & ~(kBlock - 1);
-  const int t_end = pos_last_wg + 1;
+  int t_begin = (W > 0 ? max(0, pos_first_wg - W + 1) : 0) & ~(kBlock - 1);
+  int t_end = pos_last_wg + 1;
+  if (KS > 1) {  // this unit's part of the key range, in whole 64-token chunks
+    const int per = ((t_end - t_begin + KS - 1) / KS + kChunk - 1) / kChunk * kChunk;
+    t_begin += ks_part * per;
+    t_end = min(t_end, t_begin + per);  // may leave nothing: empty partials are written
+  }
   // this wave's rows
   const int tq0 = tq_wg + wave * kPfWaveTok;
   const bool wave_active = tq0 < qlen;
@@ -1034,8 +1044,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     *(u32x4 *)(&lds_v[buf][st_off_v + 16]) = v1;
   };
 
-  fetch(t_begin);
-  stash(t_begin, 0);
+  if (t_begin < t_end) {
+    fetch(t_begin);
+    stash(t_begin, 0);
+  }
   __syncthreads();
   int cur = 0;
   for (int tc = t_begin; tc < t_end; tc += kChunk, cur ^= 1) {
@@ -1056,8 +1068,62 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     if (has_next) stash(tc + kChunk, cur ^ 1);
     __syncthreads();
   }
-  if (wave_active) finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc);
+  if (!wave_active) return;
+  if (KS == 1) {
+    finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc);
+  } else {
+    // partials of this part, one cell per (query token, part, head): finish() addresses cells
+    // as (s * ws_rows + t), so the sequence's first row with one row per "sequence" gives the
+    // token's own index
+    AttnParams pp = p;
+    pp.ws_ml = p.pf_ml;
+    pp.ws_acc = p.pf_acc;
+    pp.ws_rows = 1;
+    pp.nparts_max = KS;
+    finish<NT, FP8>(pp, row0, kvh, row0, qlen, tq0, false, ks_part, m, lacc, acc);
+  }
 }
+
+// Merge of the key-range parts of the prefill kernel.  grid = (Hq / 4, num_q_tokens); one wave
+// per (query token, head), a lane per head dim.  Tokens of sequences outside the prefill class
+// (their rows come from the split-KV kernels) are left alone.
+__global__ __launch_bounds__(256) void prefill_merge_kernel(const AttnParams p) {
+  const int lane = threadIdx.x & 63;
+  const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int row = blockIdx.y;
+  // sequence of this row: last s with cu_seqlens_q[s] <= row
+  int lo = 0, hi = p.num_seqs - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (p.cu_seqlens_q[mid] <= row) lo = mid; else hi = mid - 1;
+  }
+  const int qlen = p.cu_seqlens_q[lo + 1] - p.cu_seqlens_q[lo];
+  if (qlen < p.qlen_lo || qlen > p.qlen_hi || p.seq_lens[lo] < qlen) return;
+  const int KS = p.pf_splits, Hq = p.num_q_heads;
+  const size_t base = (size_t)row * KS * Hq + head;
+  const float sink = p.sinks ? p.sinks[head] : -INFINITY;
+  float M = sink;
+  for (int j = 0; j < KS; ++j) {
+    const float2 ml = *(const float2 *)(p.pf_ml + (base + (size_t)j * Hq) * 2);
+    if (ml.y > 0.f) M = fmaxf(M, ml.x);
+  }
+  float den = fast_exp2((sink - M) * kLog2e), o = 0.f;
+  for (int j = 0; j < KS; ++j) {
+    const float2 ml = *(const float2 *)(p.pf_ml + (base + (size_t)j * Hq) * 2);
+    if (!(ml.y > 0.f)) continue;  // an empty part: its cell may hold anything
+    const float w = ml.y * fast_exp2((ml.x - M) * kLog2e);
+    den += w;
+    o += w * (float)p.pf_acc[(base + (size_t)j * Hq) * kHeadDim + lane];
+  }
+  // den > 0: a prefill row always sees its own key, so some part is non-empty
+  const size_t orow = (size_t)row * Hq + head;
+  const float r = o / den;
+  const uint32_t mine = __float_as_uint(r), next = __shfl_down(mine, 1);
+  if ((lane & 1) == 0)
+    *(uint32_t *)(p.out + orow * kHeadDim + lane) = pack_bf16(__uint_as_float(mine), __uint_as_float(next));
+  if (p.lse && lane == 0) p.lse[orow] = M + __log2f(den) * kLn2;
+}
+
 
 // ---------------------------------------------------------------------------------------
 // Cross-partition merge.  grid = (Hq / 4, num_seqs * ws_rows); one wave per (row, head).
@@ -1451,14 +1517,23 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   return launch_splitkv_t<3, false>(p, st);
 }
 
+// Upper bound on the prefill kernel's 32-token query tiles: every sequence rounds up by at most
+// one tile.
+long long prefill_tiles_bound(int num_q_tokens, int num_seqs) {
+  return (long long)num_q_tokens / kPfTok + num_seqs;
+}
+
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st) {
-  // upper bound on 32-token tiles: every sequence rounds up by at most one tile
-  const long long items = (long long)num_q_tokens / kPfTok + p.num_seqs;
+  const long long items = prefill_tiles_bound(num_q_tokens, p.num_seqs) * max(1, p.pf_splits);
   dim3 grid((unsigned)(items * p.num_kv_heads));
   if (fp8)
     prefill_kernel<true><<<grid, kPfWaves * 64, 0, st>>>(p);
   else
     prefill_kernel<false><<<grid, kPfWaves * 64, 0, st>>>(p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || p.pf_splits <= 1) return e;
+  dim3 mgrid(p.num_q_heads / 4, num_q_tokens);
+  prefill_merge_kernel<<<mgrid, 256, 0, st>>>(p);
   return hipGetLastError();
 }
 

@@ -22,6 +22,7 @@ hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
                                 const float *k_scale, const float *v_scale, int Hq, int Hkv,
                                 int64_t num_slots, int num_tokens, bool fp8, hipStream_t st);
 int device_cus();
+long long prefill_tiles_bound(int num_q_tokens, int num_seqs);
 hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
                          const uint16_t *resid, uint16_t *out, int T, int N, int K,
                          hipStream_t st);
@@ -112,6 +113,8 @@ struct Plan {
   int32_t partition, nparts_max, ws_rows;
   bool dynamic;
   size_t ml_bytes, acc_bytes;
+  int32_t pf_splits;             // key-range parts per prefill tile (1 = no split)
+  size_t pf_ml_bytes, pf_acc_bytes;
 };
 
 // Longest key span a split-KV sequence can have (from its first visible page to its end).
@@ -143,7 +146,26 @@ Plan make_plan(const eid_attn_desc *d) {
   pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
   pl.ml_bytes = (cells * 2 * sizeof(float) + 255) / 256 * 256;
-  pl.acc_bytes = cells * eid::kHeadDim * sizeof(_Float16);
+  pl.acc_bytes = (cells * eid::kHeadDim * sizeof(_Float16) + 255) / 256 * 256;
+  // Prefill rows: when the query tiles alone cannot fill the device (two workgroups per CU)
+  // and the context is long enough to share out, every tile's key range is split into parts
+  // of at least 512 keys that run side by side and are merged afterwards.
+  pl.pf_splits = 1;
+  pl.pf_ml_bytes = pl.pf_acc_bytes = 0;
+  if (d->max_q_len > eid::kShortQMax) {
+    const long long wgs = eid::prefill_tiles_bound(d->num_q_tokens, d->num_seqs) * d->num_kv_heads;
+    // (aim: the split that comes nearest to one fill; two fills were measured too: better for
+    // one 512-token chunk behind 60k tokens, worse for a 2,048-token chunk without a prior)
+    const long long fill = 2LL * eid::device_cus(), w1 = wgs > 0 ? wgs : 1;
+    const long long by_fill = (fill + w1 / 2) / w1, by_len = d->max_kv_len / 512;
+    const long long ks = by_fill < by_len ? by_fill : by_len;
+    pl.pf_splits = (int32_t)(ks < 1 ? 1 : ks > 8 ? 8 : ks);
+    if (pl.pf_splits > 1) {
+      const size_t pcells = (size_t)d->num_q_tokens * pl.pf_splits * d->num_q_heads;
+      pl.pf_ml_bytes = (pcells * 2 * sizeof(float) + 255) / 256 * 256;
+      pl.pf_acc_bytes = pcells * eid::kHeadDim * sizeof(_Float16);
+    }
+  }
   return pl;
 }
 
@@ -159,9 +181,10 @@ int32_t check_attn_args(const eid_attn_desc *d, const eid_attn_args *a, bool nee
   if (d->kv_dtype == EID_KV_FP8_E4M3 && need_q && (!a->k_scale || !a->v_scale))
     return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
   const Plan pl = make_plan(d);
-  if (!a->workspace || a->workspace_bytes < eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes)
-    return fail(EID_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given",
-                eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes,
+  const size_t need =
+      eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
+  if (!a->workspace || a->workspace_bytes < need)
+    return fail(EID_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need,
                 a->workspace ? a->workspace_bytes : (size_t)0);
   if ((reinterpret_cast<uintptr_t>(a->workspace) & 255u) != 0)
     return fail(EID_ERR_WORKSPACE, "workspace must be 256-byte aligned");
@@ -189,6 +212,11 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.plan_slot = nullptr;
   p.ws_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes);
   p.ws_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes);
+  p.pf_splits = pl.pf_splits;
+  p.pf_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes);
+  p.pf_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes +
+                                          pl.pf_ml_bytes);
+  p.num_q_tokens = d->num_q_tokens;
   p.sum_kv_len = d->sum_kv_len;
   p.num_seqs = d->num_seqs;
   p.num_q_heads = d->num_q_heads;
@@ -250,7 +278,7 @@ int32_t eid_partition_size(const eid_attn_desc *desc) {
 size_t eid_workspace_bytes(const eid_attn_desc *desc) {
   if (check_attn_desc(desc)) return 0;
   const Plan pl = make_plan(desc);
-  return eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes;
+  return eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
 }
 
 int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v_new,

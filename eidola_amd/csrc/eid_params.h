@@ -41,6 +41,11 @@ struct AttnParams {
   int32_t qlen_lo, qlen_hi;  // this launch serves sequences with qlen_lo <= q_len <= qlen_hi
   int32_t dynamic_partition; // 1: kernels derive the partition from the batch (>= partition)
   int32_t target_items;      // workgroups the device holds at once (dynamic partition only)
+  int32_t pf_splits;         // prefill kernel: every query tile's key range is split into this
+                             // many parts (1 = none); parts write partials to pf_ml / pf_acc
+  float *pf_ml;              // [num_q_tokens][pf_splits][Hq][2]   (m natural-log units, l)
+  _Float16 *pf_acc;          // [num_q_tokens][pf_splits][Hq][64]  part output, normalised
+  int32_t num_q_tokens;
   int32_t share_cus;         // host-side launch flag: 1 = hold the split-KV kernel to one
                              // workgroup per CU (a prefill launch runs beside it)
   float softmax_scale;

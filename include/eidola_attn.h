@@ -185,6 +185,10 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  *                                     at the next 256-byte boundary
  * (heads innermost: the 64 heads of one (row, partition) cell form one contiguous block,
  * which a split-KV workgroup writes with full-width stores)
+ * Behind these, when the batch holds prefill chunks whose query tiles cannot fill the device
+ * by themselves (few new tokens behind a long context), the same two arrays once more for the
+ * prefill rows, [num_q_tokens][K] cells with K <= 8 key-range parts per query tile; they are
+ * merged inside the call.  eid_workspace_bytes() accounts for all of it.
  */
 int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args,
                       void *hip_stream);

@@ -729,3 +729,27 @@ def test_mixed_batches_from_two_host_threads(G):
         t.join()
     torch.cuda.synchronize()
     assert not errors, errors
+
+
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+@pytest.mark.parametrize("window", [0, 700])
+def test_prefill_key_range_split(G, kv_dtype, window):
+    """Few query tiles over long contexts: the prefill kernel splits every tile's key range into
+    parts (here 8, 4 and 2 by the planning rule) that are merged afterwards.  Covered: a chunk
+    whose context is shorter than one part (empty parts), chunks without prior context, decode
+    and verify rows in the same batch (their tokens must be left alone by the merge), fp8."""
+    cases = [
+        ([5200], [200]),                                   # 8 parts
+        ([3000, 140, 40, 2600], [100, 100, 40, 7]),         # short contexts beside long ones
+        ([4000, 900, 2500, 64, 1800], [64, 1, 5, 64, 2]),   # mixed classes
+    ]
+    for seq_lens, q_lens in cases:
+        b = make_batch(seq_lens, q_lens, seed=43, window=window, kv_dtype=kv_dtype)
+        q, k, v, sinks = logical_tensors(b)
+        ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+        kc, vc = cpu_caches(b, k, v, ks, vs)
+        kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+        ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+        out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True)
+        assert_close(out, ref, f"split prefill {seq_lens} w={window}")
+        assert np.allclose(lse, ref_lse, atol=2e-3)
