@@ -374,6 +374,59 @@ def prefill_bench(torch, ea, synth):
     return out
 
 
+def small_batch_bench(torch, ea, synth):
+    """Decode steps of small batches (one to sixteen sequences), the latency regime: replayed
+    from a HIP graph over several page sets, KV write fused.  The figure is microseconds per
+    call; the bandwidth column only says how far from streaming the call is."""
+    import numpy as np
+    g = ea.AttnGeometry()
+    nb = 300_000
+    kc = torch.empty((nb, 16, 8, 64), dtype=torch.bfloat16, device="cuda:0")
+    vc = torch.empty_like(kc)
+    synth.fill_pool_gpu(g, kc, vc, 13)
+    sinks = torch.zeros(64, device="cuda:0")
+    out = []
+    for lens in ([512], [4096], [16384], [131072], [8192] * 4, [2048] * 16,
+                 [8000, 4000, 2000, 1000, 500, 250, 125, 64]):
+        lens = np.array(lens, np.int32)
+        B, total = len(lens), int(lens.sum())
+        q = torch.randn((B, 64, 64), device="cuda:0").to(torch.bfloat16)
+        kn = torch.randn((B, 8, 64), device="cuda:0").to(torch.bfloat16)
+        vn = torch.randn((B, 8, 64), device="cuda:0").to(torch.bfloat16)
+        sl = torch.from_numpy(lens).to("cuda:0")
+        nblk = int(((lens.astype(np.int64) + 15) // 16).sum())
+        nsets = max(1, min(8, nb // nblk))
+        calls, ws = [], None
+        for r in range(nsets):
+            bt = torch.from_numpy(synth.build_block_table(lens, nb, 13, perm_offset=r * nblk)).to("cuda:0")
+            c = ea.prepare("eid_attn_decode", g, q, kc, vc, bt, sl, None, max_kv_len=int(lens.max()),
+                           sinks=sinks, sum_kv_len=total, workspace=ws, k_new=kn, v_new=vn)
+            ws = c._keep[-1]
+            calls.append(c)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for c in calls:
+                c(stream=side.cuda_stream)
+            side.synchronize()
+            gr = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gr, stream=side):
+                for _ in range(4):
+                    for c in calls:
+                        c(stream=side.cuda_stream)
+        torch.cuda.synchronize()
+        gr.replay()
+        torch.cuda.synchronize()
+        us = event_ms(lambda i: gr.replay(), 5, torch) * 1e3 / (4 * nsets)
+        name = f"{B}x{int(lens.max())}" + ("" if lens.min() == lens.max() else "_ragged")
+        r = {"config": f"small_batch_decode_{name}", "us": us, "bytes": total * 2048,
+             "partition": ea.partition_size(calls[0].desc)}
+        log(f"[bench] small batch {name}: {us:.1f} us per decode call "
+            f"({total * 2048 / us / 1e3:.0f} GB/s); partition {r['partition']}")
+        out.append(r)
+    return out
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -442,7 +495,7 @@ def main():
     ap.add_argument("--no-hint", action="store_true",
                     help="experiment: leave desc.sum_kv_len at 0 (grid sized from max_kv_len)")
     ap.add_argument("--only", default="",
-                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill "
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small "
                          "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
@@ -555,6 +608,8 @@ def main():
             extra.extend(oproj_bench(torch, ea))
         if want("prefill"):
             extra.extend(prefill_bench(torch, ea, synth))
+        if want("small"):
+            extra.extend(small_batch_bench(torch, ea, synth))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)

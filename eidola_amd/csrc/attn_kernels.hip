@@ -753,16 +753,24 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
 }
 
 // ---------------------------------------------------------------------------------------
-// Short-span kernel: when no sequence spans more than 8 chunks (sliding-window layers, short
-// contexts) a sequence is too short to be worth partitioning across workgroups, and one
-// wave walking its 2-3 chunks one after the other is pure latency.  Here a workgroup owns
-// one (sequence, KV head) and its 8 waves take one 64-token chunk each, all in flight at
-// once; the eight (m, l, acc) partials meet in LDS (each wave's V staging area is reused for
-// its fp32 accumulators) and the 512 threads combine them with the sink and write the
-// output.  grid = (num_seqs, Hkv); sequences of another q_len class leave at once.
+// Short-span kernel: one wave per 64-token chunk.  When no sequence spans more than 8 chunks
+// (sliding-window layers, short contexts) a sequence is too short to be worth partitioning
+// across workgroups, and one wave walking its 2-3 chunks one after the other is pure latency.
+// Here a workgroup owns one (sequence, KV head) and its 8 waves take one chunk each, all in
+// flight at once; the eight (m, l, acc) partials meet in LDS (each wave's V staging area is
+// reused for its fp32 accumulators) and the 512 threads combine them with the sink and write
+// the output.  grid = (num_seqs, Hkv); sequences of another q_len class leave at once.
+//
+// The same kernel serves small batches of longer sequences (nparts_max > 1): the sequences
+// are cut into partitions of 8 chunks, a workgroup owns one (sequence, partition, KV head),
+// found by the same scan as the split-KV kernel's work items, and writes the partition's
+// (m, l) and normalised output to the workspace for the merge kernel.  The host takes this
+// path when all workgroups are resident at once, so that every chunk of the batch is in
+// flight from the start and the call lasts a few memory latencies, whatever the lengths.
+// grid = (bound on the items, Hkv).
 // ---------------------------------------------------------------------------------------
 constexpr int kShortWaves = 8;
-constexpr int kShortSpanMax = kShortWaves * kChunk;
+static_assert(kShortSpanMax == kShortWaves * kChunk, "one chunk per wave");
 
 template <int NT, bool FP8>
 __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan_kernel(const AttnParams p) {
@@ -774,15 +782,27 @@ __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
-  const int s = blockIdx.x, kvh = blockIdx.y;
-  const SeqView v = view_seq(p, s);
-  if (v.span <= 0) return;  // not of this class, or malformed: the whole workgroup leaves
-  const int L = v.seq_len, qlen = v.qlen, row0 = v.row0;
-  const int kb = kv_begin(L, qlen, p.window);
+  const int kvh = blockIdx.y;
+  int s = blockIdx.x, part = 0, nparts = 1, L, qlen, row0;
+  if (p.nparts_max == 1) {
+    const SeqView v = view_seq(p, s);
+    if (v.span <= 0) return;  // not of this class, or malformed: the whole workgroup leaves
+    L = v.seq_len, qlen = v.qlen, row0 = v.row0;
+  } else {
+    // partitions of kShortSpanMax keys (the host set p.partition to that): every wave looks
+    // the item up for itself, there is nothing else to do yet and no barrier to wait at
+    WorkItem it;
+    int P;
+    if (!find_work_item(p, blockIdx.x, P, it)) return;
+    s = it.seq, part = it.part, nparts = it.nparts;
+    L = it.seq_len, qlen = it.qlen, row0 = it.row0;
+  }
   const int pos0 = L - qlen;
   const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
-  const int nw = min(kShortWaves, (L - kb + kChunk - 1) / kChunk);  // waves with a chunk
-  const int t0 = kb + wave * kChunk;
+  const int tb = kv_begin(L, qlen, p.window) + part * kShortSpanMax;  // this workgroup's keys
+  const int te = min(tb + kShortSpanMax, L);
+  const int nw = min(kShortWaves, (te - tb + kChunk - 1) / kChunk);  // waves with a chunk
+  const int t0 = tb + wave * kChunk;
   if (wave < nw) {
     Frag8 qf[NT][2];
     RowInfo ri;
@@ -797,7 +817,7 @@ __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan
       for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     uint8_t *mine = lds + wave * kWaveBytes;
-    attend<NT, FP8>(p, s, kvh, t0, min(t0 + kChunk, L), L, pos0, lo_last, qf, ri, mine, m, lacc, acc);
+    attend<NT, FP8>(p, s, kvh, t0, min(t0 + kChunk, te), L, pos0, lo_last, qf, ri, mine, m, lacc, acc);
     // the V tile is consumed: the same bytes now carry this wave's accumulators, row-major
     float *part = reinterpret_cast<float *>(mine);
 #pragma unroll
@@ -821,6 +841,26 @@ __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan
     const int t = r >> 3;
     if (t >= qlen) continue;
     const int head = kvh * kGroup + (r & 7);
+    if (nparts > 1) {
+      // one of several partitions: its (m, l) and normalised output go to the workspace in
+      // the split-KV kernel's layout, for the same merge
+      float M = kNegBig;
+      for (int w = 0; w < nw; ++w) M = fmaxf(M, ml_lds[w][r][0]);
+      float l = 0.f, o0 = 0.f, o1 = 0.f;
+      for (int w = 0; w < nw; ++w) {
+        const float wgt = fast_exp2(ml_lds[w][r][0] - M);
+        l += wgt * ml_lds[w][r][1];
+        const float2 a = *(const float2 *)(lds + w * kWaveBytes + ((size_t)r * kHeadDim + d2) * 4);
+        o0 += wgt * a.x;
+        o1 += wgt * a.y;
+      }
+      const size_t idx = ((size_t)(s * p.ws_rows + t) * p.nparts_max + part) * p.num_q_heads + head;
+      if (d2 == 0) *(float2 *)(p.ws_ml + idx * 2) = make_float2(l > 0.f ? M * kLn2 : -INFINITY, l);
+      const float inv_l = l > 0.f ? vs / l : 0.f;
+      typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+      *(f16x2 *)(p.ws_acc + idx * kHeadDim + d2) = f16x2{(_Float16)(o0 * inv_l), (_Float16)(o1 * inv_l)};
+      continue;
+    }
     const float sink2 = p.sinks ? p.sinks[head] * kLog2e : -INFINITY;
     float M = sink2;
     for (int w = 0; w < nw; ++w) M = fmaxf(M, ml_lds[w][r][0]);
@@ -1134,11 +1174,30 @@ __global__ __launch_bounds__(256) void prefill_merge_kernel(const AttnParams p) 
 // are summed at the end.  Sequences finished by the split-KV kernel itself (one partition)
 // and sequences outside [qlen_lo, qlen_hi] are skipped.
 // ---------------------------------------------------------------------------------------
+//
+// EAGER (launches of a few rows, where the call is a chain of memory latencies): the (m, l)
+// pairs and the first 32 partitions' outputs are requested before the sequence's length, and
+// with it the number of partitions that were written, is known; cells beyond that number
+// are dropped once it is.
+template <bool EAGER>
 __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   const int lane = threadIdx.x & 63;
   const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int wsrow = blockIdx.y;
   const int s = wsrow / p.ws_rows, t = wsrow % p.ws_rows;
+  float2 ml_early = make_float2(-INFINITY, 0.f);
+  uint2 v_early[8];
+  if (EAGER) {
+    const size_t base = (size_t)wsrow * p.nparts_max * p.num_q_heads + head;
+    if (lane < p.nparts_max) ml_early = *(const float2 *)(p.ws_ml + (base + (size_t)lane * p.num_q_heads) * 2);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int c = 4 * j + (lane >> 4);
+      v_early[j] = make_uint2(0u, 0u);
+      if (c < p.nparts_max)
+        v_early[j] = *(const uint2 *)(p.ws_acc + (base + (size_t)c * p.num_q_heads) * kHeadDim + (lane & 15) * 4);
+    }
+  }
   int row0 = s, qlen = 1;
   if (p.cu_seqlens_q) {
     row0 = p.cu_seqlens_q[s];
@@ -1160,7 +1219,11 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   const float sink = p.sinks ? p.sinks[head] : -INFINITY;
   // the first 64 partitions' (m, l), kept for both passes
   float2 ml0 = make_float2(-INFINITY, 0.f);
-  if (lane < nparts) ml0 = *(const float2 *)(p.ws_ml + (base + lane * cstride) * 2);
+  if (EAGER) {
+    if (lane < nparts) ml0 = ml_early;
+  } else {
+    if (lane < nparts) ml0 = *(const float2 *)(p.ws_ml + (base + lane * cstride) * 2);
+  }
   // pass 1: global maximum over non-empty partitions and the sink
   float M = sink;
   if (ml0.y > 0.f) M = fmaxf(M, ml0.x);
@@ -1189,7 +1252,11 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
       for (int j = 0; j < 8; ++j) {
         const int c = c0 + 4 * (j0 + j) + g;
         v[j] = make_uint2(0u, 0u);  // never multiply an unwritten cell, it may hold a NaN
-        if (c < nparts) v[j] = *(const uint2 *)(acc_row + (size_t)c * cstride * kHeadDim);
+        if (EAGER && c0 == 0 && j0 == 0) {
+          if (c < nparts) v[j] = v_early[j];
+        } else {
+          if (c < nparts) v[j] = *(const uint2 *)(acc_row + (size_t)c * cstride * kHeadDim);
+        }
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -1469,10 +1536,19 @@ static hipError_t launch_splitkv_t(const AttnParams &p, hipStream_t st) {
 // Item count of the one-workgroup-per-CU tier of the run-time partition rule.
 static int fill_lo(int target_items) { return min(target_items, device_cus()); }
 
+// Upper bound on the (sequence, partition) pairs of a short-span launch: the host knows the
+// longest span, and perhaps the sum of the lengths (which bounds the spans without a window).
+long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window) {
+  long long items = (long long)num_seqs * nparts_max;
+  if (nparts_max > 1 && sum_kv_len > 0 && window == 0)
+    items = min(items, sum_kv_len / kShortSpanMax + num_seqs);
+  return items;
+}
+
 // Short-span launch: see shortspan_kernel.  The caller has checked that no sequence spans
 // more than kShortSpanMax tokens.
 hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
-  dim3 grid(p.num_seqs, p.num_kv_heads);
+  dim3 grid((unsigned)shortspan_items(p.num_seqs, p.nparts_max, p.sum_kv_len, p.window), p.num_kv_heads);
   if (fp8) {
     if (ntiles == 1) shortspan_kernel<1, true><<<grid, kShortWaves * 64, 0, st>>>(p);
     else shortspan_kernel<3, true><<<grid, kShortWaves * 64, 0, st>>>(p);
@@ -1482,17 +1558,17 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
   }
   return hipGetLastError();
 }
-// Whether the short-span kernel should serve a launch: spans within its reach, and no more
-// workgroups (one per sequence and KV head) than the device holds at once; beyond that the
-// split-KV kernel's one workgroup per sequence makes fewer, better filled rounds.
-bool shortspan_applies(int ntiles, bool fp8, int num_seqs, int Hkv, int max_span) {
-  if (max_span > kShortSpanMax) return false;
+// Whether the short-span kernel should serve a launch of `num_items` (sequence, 512-key
+// partition) pairs: no more workgroups (one per item and KV head) than the device holds at
+// once; beyond that the split-KV kernel's one workgroup per item with longer partitions makes
+// fewer, better filled rounds.
+bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
   static const int fill[2][2] = {
       {device_fill(shortspan_kernel<1, false>, kShortWaves * 64),
        device_fill(shortspan_kernel<1, true>, kShortWaves * 64)},
       {device_fill(shortspan_kernel<3, false>, kShortWaves * 64),
        device_fill(shortspan_kernel<3, true>, kShortWaves * 64)}};
-  return (long long)num_seqs * Hkv <= fill[ntiles == 1 ? 0 : 1][fp8 ? 1 : 0];
+  return num_items * Hkv <= fill[ntiles == 1 ? 0 : 1][fp8 ? 1 : 0];
 }
 
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
@@ -1537,9 +1613,14 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
   return hipGetLastError();
 }
 
+constexpr int kMergeEagerCells = 256;  // per head: 2 MiB of reads at most
 hipError_t launch_merge(const AttnParams &p, hipStream_t st) {
   dim3 grid(p.num_q_heads / 4, p.num_seqs * p.ws_rows);
-  lse_merge_kernel<<<grid, 256, 0, st>>>(p);
+  // speculating on cells that may not have been written is cheap for a few rows only
+  if ((long long)p.num_seqs * p.ws_rows * min(p.nparts_max, 32) <= kMergeEagerCells)
+    lse_merge_kernel<true><<<grid, 256, 0, st>>>(p);
+  else
+    lse_merge_kernel<false><<<grid, 256, 0, st>>>(p);
   return hipGetLastError();
 }
 

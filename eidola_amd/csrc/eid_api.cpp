@@ -4,6 +4,7 @@
 
 #include "../../include/eidola_attn.h"
 #include "eid_params.h"
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -13,7 +14,8 @@ namespace eid {
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st);
 int splitkv_fill(int ntiles, bool fp8, int Hkv);
 hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
-bool shortspan_applies(int ntiles, bool fp8, int num_seqs, int Hkv, int max_span);
+bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
+long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
 hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
@@ -141,6 +143,18 @@ Plan make_plan(const eid_attn_desc *d) {
     P = (span + 63) / 64 * 64;
     pl.dynamic = false;
   }
+  // Small batches: when every 64-key chunk of the batch can have a wave of its own at once
+  // (512-key partitions, one workgroup of eight waves per partition and KV head, all
+  // resident together), the call is a few memory latencies long instead of a serial walk.
+  if (pl.dynamic) {
+    const long long items = eid::shortspan_items(
+        d->num_seqs, (span + eid::kShortSpanMax - 1) / eid::kShortSpanMax, d->sum_kv_len, d->window);
+    if (eid::shortspan_applies(d->max_q_len <= 2 ? 1 : 3, d->kv_dtype == EID_KV_FP8_E4M3, items,
+                               d->num_kv_heads)) {
+      P = eid::kShortSpanMax;
+      pl.dynamic = false;
+    }
+  }
   pl.partition = P;
   pl.nparts_max = (span + P - 1) / P;
   pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
@@ -258,6 +272,18 @@ Helper *helper_stream() {
   return h.ok ? &h : nullptr;
 }
 
+// Whether the short-span kernel serves the split-KV rows of a call (q_len class of `ntiles`
+// 16-row tiles): spans within one workgroup's reach, or partitions of exactly that size, and
+// few enough of them.
+bool use_shortspan(const eid_attn_desc *d, const Plan &pl, int ntiles) {
+  if (pl.nparts_max == 1 ? max_span(d) > eid::kShortSpanMax
+                         : (pl.dynamic || pl.partition != eid::kShortSpanMax))
+    return false;
+  return eid::shortspan_applies(
+      ntiles, d->kv_dtype == EID_KV_FP8_E4M3,
+      eid::shortspan_items(d->num_seqs, pl.nparts_max, d->sum_kv_len, d->window), d->num_kv_heads);
+}
+
 int32_t hip_fail(hipError_t e, const char *what) {
   return fail(EID_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
@@ -356,8 +382,7 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   // spans of at most 8 chunks: one workgroup per (sequence, KV head), a chunk per wave
-  const bool short_span = pl.nparts_max == 1 &&
-      eid::shortspan_applies(1, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
+  const bool short_span = use_shortspan(desc, pl, 1);
   hipError_t e = short_span ? eid::launch_shortspan(p, 1, fp8, st)
                             : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
@@ -390,10 +415,13 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= eid::kShortQMax;
   const bool only_prefill = uniform && desc->max_q_len > eid::kShortQMax;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  const bool short1 = pl.nparts_max == 1 &&
-      eid::shortspan_applies(1, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
-  const bool short3 = pl.nparts_max == 1 &&
-      eid::shortspan_applies(3, fp8, desc->num_seqs, desc->num_kv_heads, max_span(desc));
+  const bool short1 = use_shortspan(desc, pl, 1), short3 = use_shortspan(desc, pl, 3);
+  auto launch_split = [&](const bool short_span, const int ntiles, int32_t *slot) {
+    if (!short_span) return eid::launch_splitkv(p, ntiles, fp8, slot, st);
+    p.plan = nullptr;  // the short-span kernel works with the host's partition
+    p.plan_slot = nullptr;
+    return eid::launch_shortspan(p, ntiles, fp8, st);
+  };
   // Mixed batch: the MFMA-bound prefill launch and the HBM-bound split-KV launches use
   // different halves of the machine, so they run side by side: prefill on the thread's
   // helper stream, forked from and joined back into the caller's stream.
@@ -412,8 +440,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     p.qlen_lo = 1;
     p.qlen_hi = 2;
     p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
-    e = short1 ? eid::launch_shortspan(p, 1, fp8, st)
-               : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
+    e = launch_split(short1, 1, plan_slots);
     if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   }
   if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
@@ -436,8 +463,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     p.qlen_lo = 3;
     p.qlen_hi = eid::kShortQMax;
     p.target_items = eid::splitkv_fill(3, fp8, desc->num_kv_heads);
-    e = short3 ? eid::launch_shortspan(p, 3, fp8, st)
-               : eid::launch_splitkv(p, 3, fp8, plan_slots + 2, st);
+    e = launch_split(short3, 3, plan_slots + 2);
     if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
     if (pl.nparts_max > 1) {
       e = eid::launch_merge(p, st);

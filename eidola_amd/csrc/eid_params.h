@@ -14,6 +14,7 @@ constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the
 constexpr int kDynPartitionMin = 256;   // lower bound (and workspace sizing) of the dynamic partition
 constexpr int kDynPartitionCap = 2048;  // a workgroup streams serially: keep its share bounded
 constexpr int kDynPartitionFloor = 512; // smallest partition when the batch needs several fills
+constexpr int kShortSpanMax = 512;      // keys one workgroup of the short-span kernel covers
 constexpr int kPlanBytes = 256;         // head of the workspace: two {partition, items} slots
 
 struct AttnParams {

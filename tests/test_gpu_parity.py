@@ -363,6 +363,53 @@ def test_short_spans_one_chunk_per_wave(G, kv_dtype, window, seq_lens, q_lens):
     assert np.allclose(lse, ref_lse, atol=2e-3)
 
 
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+@pytest.mark.parametrize("window,seq_lens,q_lens,hint", [
+    (0, [4096], [1], False),                                   # one sequence, 8 partitions
+    (0, [513, 1024, 1025, 2500], [1, 1, 1, 1], False),         # partition edges
+    (0, [20000, 300, 64, 1], [1, 1, 2, 1], True),              # ragged, sized by the sum
+    (0, [3000, 700, 5000], [5, 3, 6], False),                  # verify rows
+    (2000, [6000, 2100, 900], [1, 4, 1], False),               # window wider than a partition
+    (0, [2000, 1500, 116], [1, 5, 40], False),                 # next to a prefill chunk
+])
+def test_small_batches_in_partitions_of_512(G, kv_dtype, window, seq_lens, q_lens, hint):
+    """A batch small enough that every 64-key chunk gets a wave of its own at once: the entry
+    points cut the sequences into 512-key partitions, one workgroup of eight waves per
+    partition and KV head, and merge the partitions afterwards.  Outputs and lse against the
+    oracle; the planning is visible through eid_partition_size."""
+    b = make_batch(seq_lens, q_lens, window=window, kv_dtype=kv_dtype)
+    desc = desc_of(b)
+    desc.sum_kv_len = int(b.seq_lens.sum()) if hint else 0
+    assert ea.partition_size(desc) == 512
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, hint=hint)
+    assert_close(out, ref, f"small batch w={window}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+def test_small_batch_partitions_agree_with_the_split_kv_kernel(G):
+    """The same four sequences through the 512-key partitions of the small-batch path
+    (run-time partition) and through the split-KV kernel (the caller's partition of 256):
+    two different kernels and merge inputs, one result within rounding."""
+    b = make_batch([9000, 4000, 777, 512], [1] * 4, seed=12)
+    q, k, v, sinks = logical_tensors(b)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    a = G.run_attn(b, q, kc_d, vc_d, sinks)
+    from dataclasses import replace
+    c = G.run_attn(b, q, kc_d, vc_d, sinks, geom=replace(b.geom, partition_size=256))
+    fa = synth.bf16_bits_to_f32(a).astype(np.float64)
+    fc = synth.bf16_bits_to_f32(c).astype(np.float64)
+    assert np.abs(fa - fc).max() <= 4e-3
+    kc, vc = cpu_caches(b, k, v)
+    ref, _ = oracle_out(b, q, kc, vc, sinks)
+    assert_close(a, ref, "small batch, 512-key partitions")
+    assert_close(c, ref, "small batch, split-KV kernel")
+
+
 def test_short_span_and_split_kv_kernels_agree_across_the_fill_boundary(G):
     """64 windowed decodes fill the device exactly at one workgroup per (sequence, KV head);
     65 fall back to the split-KV kernel.  The first 64 rows must agree between the two."""
