@@ -224,7 +224,9 @@ size_t eid_workspace_bytes(const eid_attn_desc *desc);
 /* The partition size (tokens) the workspace is planned with: desc->partition_size; when that
  * is 0, the lower bound 256 of the kernels' run-time choice, or, for a batch with at least
  * one sequence per compute unit whose longest span fits one partition (2,048 tokens), that
- * span rounded up to 64: every sequence is then one work item and no partials are written. */
+ * span rounded up to 64: every sequence is then one work item and no partials are written;
+ * or, for a batch so small that every 64-token chunk gets a wavefront of its own at once
+ * (one workgroup of eight per 512 tokens and KV head, all resident together), 512. */
 int32_t eid_partition_size(const eid_attn_desc *desc);
 
 /* Thread-local description of the last error on this thread; "" if none. */
