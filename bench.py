@@ -76,7 +76,7 @@ def split_kernel_ms(w, steps, torch):
     return sum(a.elapsed_time(b) for a, b in pairs) / steps
 
 
-NO_HINT = False  # --no-hint: do not pass the host-side sum of seq_lens to the library
+NO_HINT = False  # --no-hint: do not pass host-side lengths (sum, seq_lens copy) to the library
 UNFUSED = False  # --unfused: decode steps as two launches (eid_kv_write, eid_attn_decode)
 
 
@@ -118,11 +118,13 @@ class Workload:
         ws = None
         self.attn, self.merge, self.fused = [], [], []
         for bt in self.tables:
-            # the scheduler's host-side copy of seq_lens gives the sum for free; the library
-            # sizes the split-KV launch with it
+            # the scheduler builds seq_lens / cu_seqlens_q on the host: the library gets those
+            # copies (and their sum) and plans the launches with them
             kw = dict(max_q_len=b0.max_q_len, max_kv_len=b0.max_kv_len, sinks=self.sinks,
                       k_scale=self.k_scale, v_scale=self.v_scale, workspace=ws,
-                      sum_kv_len=0 if NO_HINT else int(b0.seq_lens.sum()))
+                      sum_kv_len=0 if NO_HINT else int(b0.seq_lens.sum()),
+                      seq_lens_host=None if NO_HINT else b0.seq_lens,
+                      cu_seqlens_q_host=None if NO_HINT or kind != "varlen" else b0.cu_seqlens_q)
             cu = self.cu if kind == "varlen" else None
             c = ea.prepare(fn, g, self.q, self.k_cache, self.v_cache, bt, self.seq_lens, cu, **kw)
             ws = c._keep[-1]
@@ -400,7 +402,8 @@ def small_batch_bench(torch, ea, synth):
         for r in range(nsets):
             bt = torch.from_numpy(synth.build_block_table(lens, nb, 13, perm_offset=r * nblk)).to("cuda:0")
             c = ea.prepare("eid_attn_decode", g, q, kc, vc, bt, sl, None, max_kv_len=int(lens.max()),
-                           sinks=sinks, sum_kv_len=total, workspace=ws, k_new=kn, v_new=vn)
+                           sinks=sinks, sum_kv_len=total, seq_lens_host=lens, workspace=ws,
+                           k_new=kn, v_new=vn)
             ws = c._keep[-1]
             calls.append(c)
         side = torch.cuda.Stream()
@@ -493,7 +496,8 @@ def main():
     ap.add_argument("--no-shuffle", action="store_true",
                     help="experiment: physically contiguous pages instead of a shuffled pool")
     ap.add_argument("--no-hint", action="store_true",
-                    help="experiment: leave desc.sum_kv_len at 0 (grid sized from max_kv_len)")
+                    help="experiment: no host-side lengths for the library (desc.sum_kv_len = 0, no "
+                         "seq_lens_host): the kernels size and plan the launch themselves")
     ap.add_argument("--only", default="",
                     help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small "
                          "(default: everything), e.g. to profile one configuration")
@@ -532,7 +536,7 @@ def main():
                                   "fused into the split-KV launch via k_new / v_new)"),
                    "partition_size": a.partition if a.partition else "run-time (workspace planned for >= %d)"
                    % ea.partition_size(w.attn[0].desc),
-                   "sum_kv_len_hint": not a.no_hint,
+                   "sum_kv_len_hint": not a.no_hint, "seq_lens_host": not a.no_hint,
                    "page_sets_rotated": a.sets},
         "pct_hbm_peak": 100 * r["step_GBps"] / HBM_PEAK_GBS,
         "tokens_per_s": r["q_tokens_per_s"], "ctx_tokens_per_s": r["ctx_tokens_per_s"],

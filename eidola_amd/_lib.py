@@ -74,6 +74,8 @@ class AttnArgs(C.Structure):
         ("split_done_event", C.c_void_p),
         ("k_new", C.c_void_p),
         ("v_new", C.c_void_p),
+        ("seq_lens_host", C.c_void_p),
+        ("cu_seqlens_q_host", C.c_void_p),
     ]
 
 

@@ -1473,6 +1473,7 @@ int splitkv_fill(int ntiles, bool fp8, int Hkv) {
 // and with active, so if it is below the cap for (sum_kv_len, num_seqs) it is below the cap
 // for the real batch, and the tier Tx is taken.
 static long long item_bound(const AttnParams &p) {
+  if (p.exact_items > 0) return p.exact_items;
   const long long S = p.num_seqs, T = p.target_items, Tlo = p.target_items_lo;
   if (p.nparts_max == 1) return S;  // workgroup w serves sequence w
   long long items = S * p.nparts_max;
@@ -1548,7 +1549,10 @@ long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, in
 // Short-span launch: see shortspan_kernel.  The caller has checked that no sequence spans
 // more than kShortSpanMax tokens.
 hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
-  dim3 grid((unsigned)shortspan_items(p.num_seqs, p.nparts_max, p.sum_kv_len, p.window), p.num_kv_heads);
+  const long long items = p.exact_items > 0 && p.nparts_max > 1
+                              ? p.exact_items
+                              : shortspan_items(p.num_seqs, p.nparts_max, p.sum_kv_len, p.window);
+  dim3 grid((unsigned)items, p.num_kv_heads);
   if (fp8) {
     if (ntiles == 1) shortspan_kernel<1, true><<<grid, kShortWaves * 64, 0, st>>>(p);
     else shortspan_kernel<3, true><<<grid, kShortWaves * 64, 0, st>>>(p);
@@ -1578,7 +1582,7 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   p.target_items_lo = fill_lo(p.target_items);
   p.plan = nullptr;
   p.plan_slot = plan_slot;
-  if (p.nparts_max > 1 && item_bound(p) > 4LL * p.target_items) {
+  if (p.nparts_max > 1 && p.exact_items == 0 && item_bound(p) > 4LL * p.target_items) {
     AttnParams q = p;
     plan_kernel<<<1, 64, 0, st>>>(q, plan_slot);
     const hipError_t e = hipGetLastError();

@@ -9,6 +9,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <vector>
 
 namespace eid {
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st);
@@ -288,6 +289,121 @@ int32_t hip_fail(hipError_t e, const char *what) {
   return fail(EID_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+// ---- launch planning from the caller's host copies of seq_lens / cu_seqlens_q ----------
+
+// Key spans of the sequences of one q_len class, as the kernels see them (view_seq).
+struct ClassSpans {
+  std::vector<int32_t> spans;
+  long long total = 0;
+  int32_t longest = 0;
+  long long items(int32_t P, int32_t nparts_max) const {
+    long long n = 0;
+    for (const int32_t sp : spans) n += std::min((sp + P - 1) / P, nparts_max);
+    return n;
+  }
+};
+
+ClassSpans class_spans(const eid_attn_desc *d, const int32_t *seq_lens, const int32_t *cu,
+                       int32_t ws_rows, int32_t qlen_lo, int32_t qlen_hi) {
+  ClassSpans c;
+  for (int32_t s = 0; s < d->num_seqs; ++s) {
+    const int32_t L = seq_lens[s], qlen = cu ? cu[s + 1] - cu[s] : 1;
+    if (qlen < qlen_lo || qlen > qlen_hi || qlen > ws_rows || L < qlen) continue;
+    const int32_t span = L - eid::kv_begin(L, qlen, d->window);
+    if (span <= 0) continue;
+    c.spans.push_back(span);
+    c.total += span;
+    c.longest = std::max(c.longest, span);
+  }
+  return c;
+}
+
+// The partition the kernels' run-time rule would derive for these spans (the same tiers in the
+// same order: one workgroup per CU, one device fill, whole sequences, equal pieces of nearly
+// uniform batches, about three fills), computed once here instead of by every workgroup.
+int32_t host_partition(const ClassSpans &c, long long T, long long Tlo, int32_t Pmin,
+                       int32_t nparts_max) {
+  const long long active = (long long)c.spans.size(), cap = eid::kDynPartitionCap;
+  auto up64 = [](long long v) { return (v + 63) / 64 * 64; };
+  auto single_fill = [&](const long long Tx) -> int32_t {
+    if (active > Tx) return 0;
+    long long hi = up64(c.longest);
+    if (active < Tx) hi = std::min(hi, up64((c.total + (Tx - active) - 1) / (Tx - active)));
+    hi = std::max(hi, (long long)Pmin);
+    if (hi >= cap) return 0;
+    int32_t lo_i = Pmin / 64, hi_i = (int32_t)hi / 64 - 1, P = (int32_t)hi;
+    while (lo_i <= hi_i) {
+      const int32_t mid = (lo_i + hi_i) >> 1;
+      if (c.items(mid * 64, nparts_max) <= Tx) {
+        P = mid * 64;
+        hi_i = mid - 1;
+      } else {
+        lo_i = mid + 1;
+      }
+    }
+    return P;
+  };
+  if (Tlo < T)
+    if (const int32_t P = single_fill(std::max(Tlo, 1LL))) return P;
+  if (const int32_t P = single_fill(T)) return P;
+  const long long whole = up64(c.longest);
+  if (active >= Tlo && whole <= cap) return (int32_t)std::max(whole, (long long)Pmin);
+  if ((long long)c.longest * active * 4 <= c.total * 5) {
+    const long long pieces = (c.longest + cap - 1) / cap;
+    return (int32_t)std::max(up64((c.longest + pieces - 1) / pieces), (long long)Pmin);
+  }
+  return (int32_t)std::min(cap, std::max((long long)eid::kDynPartitionFloor, up64(c.total / (3 * T))));
+}
+
+// What the host decided for the split-KV launch of one q_len class.
+struct ClassPlan {
+  bool skip = false;      // no sequence of this class: launch nothing
+  bool short_span = false;
+  bool merge = false;     // some sequence has more than one partition
+};
+
+// Sets p.partition / p.dynamic_partition / p.exact_items for the class [qlen_lo, qlen_hi] and
+// says which kernel serves it.  Without host lengths this is the plan made from the
+// descriptor alone; with them, the run-time choices of the kernels are made here.
+ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan &pl,
+                     eid::AttnParams &p, int ntiles, int32_t qlen_lo, int32_t qlen_hi,
+                     bool decode) {
+  ClassPlan cp;
+  const bool fp8 = d->kv_dtype == EID_KV_FP8_E4M3;
+  p.qlen_lo = qlen_lo;
+  p.qlen_hi = qlen_hi;
+  p.partition = pl.partition;
+  p.dynamic_partition = pl.dynamic ? 1 : 0;
+  p.exact_items = 0;
+  p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads);
+  cp.short_span = use_shortspan(d, pl, ntiles);
+  cp.merge = pl.nparts_max > 1;
+  constexpr int32_t kHostPlanMaxSeqs = 8192;  // beyond that the host pass is no longer free
+  const int32_t *cu = decode ? nullptr : a->cu_seqlens_q_host;
+  if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs) return cp;
+  const ClassSpans c = class_spans(d, a->seq_lens_host, cu, pl.ws_rows, qlen_lo, qlen_hi);
+  if (c.spans.empty()) {
+    cp.skip = true;
+    return cp;
+  }
+  if (pl.nparts_max == 1) return cp;  // workgroup w serves sequence w: nothing to refine
+  if (pl.dynamic) {
+    const long long at512 = c.items(eid::kShortSpanMax, pl.nparts_max);
+    if (eid::shortspan_applies(ntiles, fp8, at512, d->num_kv_heads)) {
+      cp.short_span = true;  // small batch: one wave per chunk (see make_plan)
+      p.partition = eid::kShortSpanMax;
+    } else {
+      const long long T = p.target_items;
+      p.partition = host_partition(c, T, std::min<long long>(T, eid::device_cus()), pl.partition,
+                                   pl.nparts_max);
+    }
+    p.dynamic_partition = 0;
+  }
+  p.exact_items = c.items(p.partition, pl.nparts_max);
+  cp.merge = p.exact_items > (long long)c.spans.size();
+  return cp;
+}
+
 }  // namespace
 
 extern "C" {
@@ -369,8 +485,6 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const Plan pl = make_plan(desc);
   eid::AttnParams p = make_params(desc, args, pl);
   p.cu_seqlens_q = nullptr;  // one row per sequence by contract
-  p.qlen_lo = 1;
-  p.qlen_hi = 1;
   if ((args->k_new != nullptr) != (args->v_new != nullptr))
     return fail(EID_ERR_INVALID_ARG, "k_new and v_new must both be given or both be NULL");
   if (!aligned16(args->k_new) || !aligned16(args->v_new))
@@ -379,18 +493,19 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   p.v_new = static_cast<const uint16_t *>(args->v_new);
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
-  p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  // spans of at most 8 chunks: one workgroup per (sequence, KV head), a chunk per wave
-  const bool short_span = use_shortspan(desc, pl, 1);
-  hipError_t e = short_span ? eid::launch_shortspan(p, 1, fp8, st)
-                            : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
+  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true);
+  if (cp.skip) return EID_OK;  // (every sequence empty or malformed: nothing is written)
+  // spans of at most 8 chunks, or a small batch in partitions of that size: one workgroup
+  // per (sequence, partition, KV head), a chunk per wave
+  hipError_t e = cp.short_span ? eid::launch_shortspan(p, 1, fp8, st)
+                               : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (args->split_done_event) {
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
     if (e != hipSuccess) return hip_fail(e, "split_done_event record");
   }
-  if (pl.nparts_max > 1) {
+  if (cp.merge) {
     e = eid::launch_merge(p, st);
     if (e != hipSuccess) return hip_fail(e, "merge launch");
   }
@@ -415,9 +530,8 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= eid::kShortQMax;
   const bool only_prefill = uniform && desc->max_q_len > eid::kShortQMax;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  const bool short1 = use_shortspan(desc, pl, 1), short3 = use_shortspan(desc, pl, 3);
-  auto launch_split = [&](const bool short_span, const int ntiles, int32_t *slot) {
-    if (!short_span) return eid::launch_splitkv(p, ntiles, fp8, slot, st);
+  auto launch_split = [&](const ClassPlan &cp, const int ntiles, int32_t *slot) {
+    if (!cp.short_span) return eid::launch_splitkv(p, ntiles, fp8, slot, st);
     p.plan = nullptr;  // the short-span kernel works with the host's partition
     p.plan_slot = nullptr;
     return eid::launch_shortspan(p, ntiles, fp8, st);
@@ -436,12 +550,14 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   }
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
+  ClassPlan cp1;
+  cp1.skip = true;
   if (!only_verify && !only_prefill) {
-    p.qlen_lo = 1;
-    p.qlen_hi = 2;
-    p.target_items = eid::splitkv_fill(1, fp8, desc->num_kv_heads);
-    e = launch_split(short1, 1, plan_slots);
-    if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+    cp1 = plan_class(desc, args, pl, p, 1, 1, 2, false);
+    if (!cp1.skip) {
+      e = launch_split(cp1, 1, plan_slots);
+      if (e != hipSuccess) return hip_fail(e, "split-KV launch");
+    }
   }
   if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
     eid::AttnParams pp = p;
@@ -455,19 +571,19 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
     if (e != hipSuccess) return hip_fail(e, "split_done_event record");
   }
-  if (!only_verify && !only_prefill && pl.nparts_max > 1) {
+  if (!cp1.skip && cp1.merge) {
     e = eid::launch_merge(p, st);
     if (e != hipSuccess) return hip_fail(e, "merge launch");
   }
   if (desc->max_q_len > 2 && !only_prefill) {  // q_len 3..6: three tiles
-    p.qlen_lo = 3;
-    p.qlen_hi = eid::kShortQMax;
-    p.target_items = eid::splitkv_fill(3, fp8, desc->num_kv_heads);
-    e = launch_split(short3, 3, plan_slots + 2);
-    if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
-    if (pl.nparts_max > 1) {
-      e = eid::launch_merge(p, st);
-      if (e != hipSuccess) return hip_fail(e, "merge launch");
+    const ClassPlan cp3 = plan_class(desc, args, pl, p, 3, 3, eid::kShortQMax, false);
+    if (!cp3.skip) {
+      e = launch_split(cp3, 3, plan_slots + 2);
+      if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
+      if (cp3.merge) {
+        e = eid::launch_merge(p, st);
+        if (e != hipSuccess) return hip_fail(e, "merge launch");
+      }
     }
   }
   if (hs) {

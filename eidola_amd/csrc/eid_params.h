@@ -49,6 +49,8 @@ struct AttnParams {
   int32_t num_q_tokens;
   int32_t share_cus;         // host-side launch flag: 1 = hold the split-KV kernel to one
                              // workgroup per CU (a prefill launch runs beside it)
+  long long exact_items;     // host-side: the launch's exact number of work items when the host
+                             // has the sequence lengths, 0 = not known (a bound is launched)
   float softmax_scale;
 };
 

@@ -8,6 +8,7 @@ import ctypes as C
 import math
 from dataclasses import dataclass
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -191,7 +192,6 @@ def yarn_cos_sin(max_pos, head_dim=64, base=150000.0, scaling_factor=32.0,
     attention-temperature factor 0.1 ln(scaling_factor) + 1 folded in, as the published
     gpt-oss model definition describes its rotary embedding (defaults are that model's
     configuration).  scaling_factor <= 1 gives plain RoPE."""
-    import numpy as np
     half = head_dim // 2
     freq = base ** (np.arange(0, head_dim, 2, dtype=np.float64) / head_dim)
     if scaling_factor > 1.0:
@@ -209,9 +209,25 @@ def yarn_cos_sin(max_pos, head_dim=64, base=150000.0, scaling_factor=32.0,
                           axis=1).astype(np.float32)
 
 
+def _host_i32(a, name, n):
+    """A host copy of a length array as contiguous int32 numpy (the library reads it during
+    the call); accepts numpy arrays and CPU tensors."""
+    if a is None:
+        return None
+    if isinstance(a, torch.Tensor):
+        if a.is_cuda:
+            raise ValueError(f"{name} must live in host memory")
+        a = a.numpy()
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    if a.shape != (n,):
+        raise ValueError(f"{name} must have {n} entries")
+    return a
+
+
 def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q,
                max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace,
-               return_lse, sum_kv_len=0, k_new=None, v_new=None):
+               return_lse, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None,
+               cu_seqlens_q_host=None):
     _require(q, "q", torch.bfloat16, 3)
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
@@ -267,6 +283,10 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
             if tuple(t.shape) != (S, geom.num_kv_heads, geom.head_dim):
                 raise ValueError(f"{name} must be [num_seqs, num_kv_heads, head_dim]")
             setattr(args, name, t.data_ptr())
+    sl_h = _host_i32(seq_lens_host, "seq_lens_host", S)
+    cu_h = _host_i32(cu_seqlens_q_host, "cu_seqlens_q_host", S + 1)
+    args.seq_lens_host = sl_h.ctypes.data if sl_h is not None else None
+    args.cu_seqlens_q_host = cu_h.ctypes.data if cu_h is not None else None
     check(getattr(lib, fn_name)(C.byref(desc), C.byref(args), _stream()))
     return (out, lse) if return_lse else out
 
@@ -291,8 +311,11 @@ class PreparedCall:
 
 def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, *,
             max_q_len=1, max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
-            workspace=None, sum_kv_len=0, k_new=None, v_new=None):
-    """Build a PreparedCall for "eid_attn_decode" / "eid_attn_varlen" / "eid_lse_merge"."""
+            workspace=None, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None,
+            cu_seqlens_q_host=None):
+    """Build a PreparedCall for "eid_attn_decode" / "eid_attn_varlen" / "eid_lse_merge".
+    `seq_lens_host` / `cu_seqlens_q_host` (host copies of the two length arrays) are copied
+    and kept by the object."""
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
     _require(q, "q", torch.bfloat16, 3)
@@ -322,30 +345,42 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
     args.workspace_bytes = workspace.numel()
     args.k_new = k_new.data_ptr() if k_new is not None else None
     args.v_new = v_new.data_ptr() if v_new is not None else None
+    S = seq_lens.shape[0]
+    sl_h = _host_i32(seq_lens_host, "seq_lens_host", S)
+    cu_h = _host_i32(cu_seqlens_q_host, "cu_seqlens_q_host", S + 1)
+    sl_h = sl_h.copy() if sl_h is not None else None
+    cu_h = cu_h.copy() if cu_h is not None else None
+    args.seq_lens_host = sl_h.ctypes.data if sl_h is not None else None
+    args.cu_seqlens_q_host = cu_h.ctypes.data if cu_h is not None else None
     keep = (q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, sinks, k_scale, v_scale,
-            k_new, v_new, workspace)  # workspace stays last: callers share it via _keep[-1]
+            k_new, v_new, sl_h, cu_h,
+            workspace)  # workspace stays last: callers share it via _keep[-1]
     return PreparedCall(fn_name, desc, args, keep, out, lse)
 
 
 def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, sinks=None,
                 k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
-                return_lse=False, sum_kv_len=0, k_new=None, v_new=None):
+                return_lse=False, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None):
     """Stages K2+K4: one query row per sequence (q is [num_seqs, Hq, D]).  `sum_kv_len` is the
-    optional host-side sum of seq_lens (any upper bound): it sizes the launch to the work.
+    optional host-side sum of seq_lens (any upper bound): it sizes the launch to the work;
+    `seq_lens_host`, a host copy of seq_lens, lets the library plan the launch exactly.
     With `k_new` / `v_new` ([num_seqs, Hkv, D] bf16: the newest token of every sequence, not
     yet in the cache) the call writes those rows into the caches itself (stage K1 fused)."""
     return _attn_call("eid_attn_decode", geom, q, k_cache, v_cache, block_table, seq_lens, None,
                       1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse,
-                      sum_kv_len, k_new, v_new)
+                      sum_kv_len, k_new, v_new, seq_lens_host)
 
 
 def attn_varlen(geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, *, max_q_len,
                 max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
-                workspace=None, return_lse=False, sum_kv_len=0):
-    """Stages K2/K3+K4 on a ragged cu_seqlens batch (prefill chunks, verify rows, decodes)."""
+                workspace=None, return_lse=False, sum_kv_len=0, seq_lens_host=None,
+                cu_seqlens_q_host=None):
+    """Stages K2/K3+K4 on a ragged cu_seqlens batch (prefill chunks, verify rows, decodes).
+    With host copies of both length arrays the library plans the launches exactly."""
     return _attn_call("eid_attn_varlen", geom, q, k_cache, v_cache, block_table, seq_lens,
                       cu_seqlens_q, max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse,
-                      workspace, return_lse, sum_kv_len)
+                      workspace, return_lse, sum_kv_len, None, None, seq_lens_host,
+                      cu_seqlens_q_host)
 
 
 def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_len, max_kv_len,

@@ -112,6 +112,14 @@ typedef struct eid_attn_args {
                            block_table[s][pos/16]*16 + pos%16) and attends to them from
                            registers: the step needs no separate eid_kv_write launch.
                            k_cache / v_cache are written in that case. */
+  const int32_t *seq_lens_host;     /* optional HOST copies of seq_lens [num_seqs] and */
+  const int32_t *cu_seqlens_q_host; /* cu_seqlens_q [num_seqs + 1] (the latter is needed by
+                           eid_attn_varlen only), read before the call returns.  An engine's
+                           scheduler builds these arrays on the host anyway; with them the
+                           library plans the launches itself (partition size, exact grids,
+                           which kernels have work at all) instead of leaving that to every
+                           workgroup of the kernels.  They must equal the device arrays;
+                           results do not depend on whether they are given. */
 } eid_attn_args;
 
 /*

@@ -49,10 +49,11 @@ def gpu_caches(batch, k, v, k_scale=None, v_scale=None):
 
 
 def run_attn(batch, q, kc_d, vc_d, sinks, k_scale=None, v_scale=None, *, decode=None,
-             return_lse=False, geom=None, hint=False, return_device=False):
+             return_lse=False, geom=None, hint=False, return_device=False, host_lens=False):
     """Calls eid_attn_decode (all q_len == 1) or eid_attn_varlen through the C ABI; with
-    `hint` the host-side sum of seq_lens is passed as desc.sum_kv_len.  `return_device`
-    hands back the output tensor itself instead of its bits on the host."""
+    `hint` the host-side sum of seq_lens is passed as desc.sum_kv_len, with `host_lens` the
+    host copies of seq_lens / cu_seqlens_q as well.  `return_device` hands back the output
+    tensor itself instead of its bits on the host."""
     geom = geom or batch.geom
     if decode is None:
         decode = batch.max_q_len == 1
@@ -60,9 +61,13 @@ def run_attn(batch, q, kc_d, vc_d, sinks, k_scale=None, v_scale=None, *, decode=
               v_scale=dev(v_scale), return_lse=return_lse,
               sum_kv_len=int(batch.seq_lens.sum()) if hint else 0)
     bt, sl = dev(batch.block_table), dev(batch.seq_lens)
+    if host_lens:
+        kw["seq_lens_host"] = batch.seq_lens
     if decode:
         r = ea.attn_decode(geom, bf16_dev(q), kc_d, vc_d, bt, sl, **kw)
     else:
+        if host_lens:
+            kw["cu_seqlens_q_host"] = batch.cu_seqlens_q
         r = ea.attn_varlen(geom, bf16_dev(q), kc_d, vc_d, bt, sl, dev(batch.cu_seqlens_q),
                            max_q_len=batch.max_q_len, **kw)
     torch.cuda.synchronize()

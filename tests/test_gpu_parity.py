@@ -535,10 +535,43 @@ def test_seeded_random_batches(G, seed):
     kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
     ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
     out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True,
-                          hint=bool(rng.random() < 0.5))
+                          hint=bool(rng.random() < 0.5), host_lens=bool(rng.random() < 0.5))
     what = f"seed {seed}: S={S} w={window} P={partition} dtype={kv_dtype} q={sorted(set(q_lens.tolist()))}"
     assert_close(out, ref, what)
     assert np.allclose(lse, ref_lse, atol=3e-3), what
+
+
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+@pytest.mark.parametrize("window,partition,seq_lens,q_lens", [
+    (0, 0, [5000, 300, 9000, 40, 1, 2500], [1] * 6),                 # ragged decode
+    (0, 0, [20000, 300, 64, 1], [1, 1, 2, 1]),                       # small batch without the sum
+    (0, 0, [3000, 700, 5000, 900], [5, 3, 6, 4]),                    # verify rows only
+    (0, 0, [2000, 1500, 600, 116], [1, 1, 40, 70]),                  # decodes + prefill, no verify class
+    (0, 0, [900, 800], [100, 33]),                                   # prefill rows only
+    (128, 0, [6000, 2100, 900, 50], [1, 4, 1, 2]),                   # windowed: one partition each
+    (0, 256, [5000, 300, 9000, 40], [1, 1, 5, 2]),                   # the caller's partition
+    (0, 0, [33] * 70 + [7000] * 3, [1] * 73),                        # many short ones, few long
+])
+def test_host_copies_of_the_lengths_plan_the_launches(G, kv_dtype, window, partition, seq_lens,
+                                                      q_lens):
+    """With args.seq_lens_host / cu_seqlens_q_host the library picks partition sizes, exact
+    grids and the kernels that have work on the host.  Same results as without them (and as
+    the oracle), for every q_len class mix, including classes without a sequence."""
+    b = make_batch(seq_lens, q_lens, window=window, partition=partition, kv_dtype=kv_dtype)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    plain = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, host_lens=True)
+    assert_close(out, ref, "host lengths")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+    a = synth.bf16_bits_to_f32(out).astype(np.float64)
+    c = synth.bf16_bits_to_f32(plain).astype(np.float64)
+    assert np.abs(a - c).max() <= 4e-3
+    both = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, host_lens=True, hint=True)
+    assert np.array_equal(both, out)   # the sum adds nothing the arrays do not say
 
 
 # ---------------------------------------------------------------- benchmark configurations
@@ -590,6 +623,12 @@ def test_config2_full_size(G, window):
         oh = ea.attn_decode(*args, max_kv_len=b.max_kv_len, sinks=G.dev(sinks), sum_kv_len=hint)
         torch.cuda.synchronize()
         assert torch.equal(oh, out), hint
+    # host copy of seq_lens: the library derives on the host the partition the kernels would
+    # (the same rule), so the work items and with them every bit of the output are the same
+    oh = ea.attn_decode(*args, max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
+                        sum_kv_len=int(b.seq_lens.sum()), seq_lens_host=b.seq_lens)
+    torch.cuda.synchronize()
+    assert torch.equal(oh, out)
 
 
 def test_config3_mixed_full_size(G):
