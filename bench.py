@@ -430,6 +430,87 @@ def small_batch_bench(torch, ea, synth):
     return out
 
 
+def stack_bench(torch, ea, synth, layers=36):
+    """The attention block of every layer of ONE decode step, replayed from one HIP graph:
+    per layer the QKV projection (the library's GEMM entry point, 2880 -> 5120 with bias),
+    rotary embedding + split + KV write, paged sink-attention (even layers a 128-token
+    window, odd layers full attention, as gpt-oss alternates) and the output projection with
+    bias and residual add (4096 -> 2880).  Config 2's batch (64 sequences); every layer has
+    its own pages (one pool, disjoint page sets) and its own weights, so nothing is served
+    from a cache that a real model would not have.  Norms, MoE and sampling are not here."""
+    import numpy as np
+    dev = "cuda:0"
+    b0 = synth.config2()
+    S, H, NQKV = b0.num_seqs, 2880, (64 + 2 * 8) * 64
+    nblk = int(((b0.seq_lens.astype(np.int64) + 15) // 16).sum())
+    nb = layers * nblk
+    gfull, gwin = ea.AttnGeometry(), ea.AttnGeometry(window=128)
+    kc = torch.empty((nb, 16, 8, 64), dtype=torch.bfloat16, device=dev)
+    vc = torch.empty_like(kc)
+    synth.fill_pool_gpu(gfull, kc, vc, 21)
+    sl_h = b0.seq_lens
+    sl = torch.from_numpy(sl_h).to(dev)
+    pos = torch.from_numpy((sl_h - 1).astype(np.int32)).to(dev)
+    cos_sin = torch.from_numpy(ea.yarn_cos_sin(int(sl_h.max()) + 1)).to(dev)
+    sinks = torch.zeros(64, device=dev)
+    hidden0 = (torch.randn((S, H), device=dev) * 0.5).to(torch.bfloat16)
+    hidden = hidden0.clone()
+    qkv = torch.empty((S, NQKV), dtype=torch.bfloat16, device=dev)
+    q = torch.empty((S, 64, 64), dtype=torch.bfloat16, device=dev)
+    lay, ws = [], {}
+    for l in range(layers):
+        batch = synth.config2(num_blocks=nb, perm_offset=l * nblk)
+        bt = torch.from_numpy(batch.block_table).to(dev)
+        g = gwin if l % 2 == 0 else gfull
+        call = ea.prepare("eid_attn_decode", g, q, kc, vc, bt, sl, None, max_kv_len=b0.max_kv_len,
+                          sinks=sinks, sum_kv_len=int(sl_h.sum()), seq_lens_host=sl_h,
+                          workspace=ws.get(l % 2))
+        ws[l % 2] = call._keep[-1]
+        lay.append(dict(
+            wqkv=(torch.randn((NQKV, H), device=dev) * 0.02).to(torch.bfloat16),
+            bqkv=torch.zeros(NQKV, dtype=torch.bfloat16, device=dev),
+            wo=(torch.randn((H, 4096), device=dev) * 0.02).to(torch.bfloat16),
+            bo=torch.zeros(H, dtype=torch.bfloat16, device=dev),
+            slots=torch.from_numpy(batch.slot_mapping).to(dev), geom=g, attn=call))
+
+    def step(stream=None):
+        hidden.copy_(hidden0)
+        for L in lay:
+            ea.o_proj(hidden, L["wqkv"], L["bqkv"], out=qkv)
+            ea.rope_kv_write(L["geom"], qkv, pos, cos_sin, kc, vc, L["slots"], q_out=q)
+            L["attn"](stream=stream)
+            ea.o_proj(L["attn"].out, L["wo"], L["bo"], residual=hidden, out=hidden)
+
+    step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(side.cuda_stream)
+        side.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr, stream=side):
+            step(side.cuda_stream)
+    torch.cuda.synchronize()
+    gr.replay()
+    torch.cuda.synchronize()
+    ms = event_ms(lambda i: gr.replay(), 20, torch)
+    ms_eager = event_ms(lambda i: step(), 5, torch)
+    ok = bool(torch.isfinite(hidden.float()).all().item())
+    kv_bytes = sum(synth.algorithmic_work(synth.config2(window=0 if l % 2 else 128))["bytes"]
+                   for l in range(layers))
+    w_bytes = layers * (NQKV * H + H * 4096) * 2
+    r = {"config": f"attention_stack_{layers}_layers_config2_batch", "ms": ms, "ms_eager": ms_eager,
+         "layers": layers, "us_per_layer": ms * 1e3 / layers, "kv_bytes": kv_bytes,
+         "weight_bytes": w_bytes, "GBps": (kv_bytes + w_bytes) / ms / 1e6, "finite": ok}
+    log(f"[bench] attention stack, {layers} layers x (QKV proj, RoPE + KV write, attention, "
+        f"o_proj), 64 seqs: {ms*1e3:.0f} us per decode step from one graph "
+        f"({ms*1e3/layers:.1f} us per layer, {ms_eager*1e3:.0f} us launched eagerly); "
+        f"{(kv_bytes + w_bytes)/1e9:.2f} GB of KV + weights -> {r['GBps']:.0f} GB/s; "
+        f"{S / ms * 1e3:.0f} tokens/s bound from attention blocks alone")
+    return [r]
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -499,7 +580,7 @@ def main():
                     help="experiment: no host-side lengths for the library (desc.sum_kv_len = 0, no "
                          "seq_lens_host): the kernels size and plan the launch themselves")
     ap.add_argument("--only", default="",
-                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small "
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack "
                          "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
@@ -614,6 +695,8 @@ def main():
             extra.extend(prefill_bench(torch, ea, synth))
         if want("small"):
             extra.extend(small_batch_bench(torch, ea, synth))
+        if want("stack"):
+            extra.extend(stack_bench(torch, ea, synth))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:
         threads = min(16, os.cpu_count() or 1)

@@ -306,6 +306,7 @@ struct ClassSpans {
 ClassSpans class_spans(const eid_attn_desc *d, const int32_t *seq_lens, const int32_t *cu,
                        int32_t ws_rows, int32_t qlen_lo, int32_t qlen_hi) {
   ClassSpans c;
+  c.spans.reserve(d->num_seqs);
   for (int32_t s = 0; s < d->num_seqs; ++s) {
     const int32_t L = seq_lens[s], qlen = cu ? cu[s + 1] - cu[s] : 1;
     if (qlen < qlen_lo || qlen > qlen_hi || qlen > ws_rows || L < qlen) continue;
@@ -381,7 +382,12 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   constexpr int32_t kHostPlanMaxSeqs = 8192;  // beyond that the host pass is no longer free
   const int32_t *cu = decode ? nullptr : a->cu_seqlens_q_host;
   if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs) return cp;
-  const ClassSpans c = class_spans(d, a->seq_lens_host, cu, pl.ws_rows, qlen_lo, qlen_hi);
+  ClassSpans c;
+  try {
+    c = class_spans(d, a->seq_lens_host, cu, pl.ws_rows, qlen_lo, qlen_hi);
+  } catch (...) {  // out of host memory: nothing may cross the C ABI; the kernels plan instead
+    return cp;
+  }
   if (c.spans.empty()) {
     cp.skip = true;
     return cp;

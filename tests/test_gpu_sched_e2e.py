@@ -81,11 +81,13 @@ def test_continuous_batching_with_prefix_reuse(G):
         args = (geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens))
         if b.max_q_len == 1:
             out = ea.attn_decode(*args, max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
-                                 sum_kv_len=b.sum_kv_len)
+                                 sum_kv_len=b.sum_kv_len, seq_lens_host=b.seq_lens)
         else:
+            # the builder's host arrays go to the library as they are: it plans with them
             out = ea.attn_varlen(*args, G.dev(b.cu_seqlens_q), max_q_len=b.max_q_len,
                                  max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
-                                 sum_kv_len=b.sum_kv_len)
+                                 sum_kv_len=b.sum_kv_len, seq_lens_host=b.seq_lens,
+                                 cu_seqlens_q_host=b.cu_seqlens_q)
         torch.cuda.synchronize()
         assert_close(G.bits_host(out), ref, f"step {ids} {q_lens}")
         return b
