@@ -15,7 +15,8 @@
 //
 // Two kernels:
 //   oproj_skinny_kernel  T <= 64 (decode batches).  HBM-bound: the weight (N*K*2 bytes) is
-//                        streamed once.  One workgroup per 16 features; its 8 waves deal the
+//                        streamed once.  One workgroup per 16 features (per 32 when that
+//                        keeps the workgroups within one per CU); its 8 waves deal the
 //                        K dimension in 64-element chunks, each wave keeps a whole batch of
 //                        weight loads in flight, the partial sums meet in LDS.
 //   oproj_tiled_kernel   any T.  128 x 128 (or, for batches too small to fill the device
@@ -66,7 +67,7 @@ constexpr int kSkRowBytes = kSkSlab * 2 + 16;      // LDS row of an activation s
 }  // namespace
 
 // ---------------------------------------------------------------------------------------
-// Streaming kernel.  grid = N / 16, block = 512.  TT = number of 16-token tiles (T <= 16 TT).
+// Streaming kernel.  grid = N / (16 FT), block = 512.  TT = number of 16-token tiles (T <= 16 TT).
 // K is walked in rounds of 512 elements; in round r wave w owns chunk 8 r + w.
 //   weights      each wave loads the fragments of its chunks of 8 rounds (all of K = 4096)
 //                back to back, straight from memory: 16 KiB in flight per wave
@@ -78,7 +79,11 @@ constexpr int kSkRowBytes = kSkSlab * 2 + 16;      // LDS row of an activation s
 //                and read from there as fragments.
 // The eight K shares meet in LDS (reusing the slab tiles).  Requires K % 64 == 0.
 // ---------------------------------------------------------------------------------------
-template <int TT>
+// FT = 16-feature tiles per workgroup.  A workgroup's cost is mostly its pass over the
+// activations, whatever the number of features, and with three or four token tiles only one
+// workgroup fits a CU (LDS): when N / 16 exceeds the number of CUs, two feature tiles per
+// workgroup (N % 32 == 0) finish in one round of workgroups instead of two.
+template <int TT, int FT>
 __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
@@ -86,12 +91,13 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
   constexpr int kRows = TT * 16;
   constexpr int kLd = kRows / kSkWaves;  // slab rows per wave = loads per thread and slab
   constexpr int kTileBytes = kRows * kSkRowBytes;
-  static_assert(2 * kTileBytes >= (int)sizeof(f32x4) * kSkWaves * TT * 64, "reduction reuses the tiles");
+  static_assert(2 * kTileBytes >= (int)sizeof(f32x4) * kSkWaves * TT * FT * 64, "reduction reuses the tiles");
+  static_assert(TT * FT <= kSkWaves, "one wave per result tile in the epilogue");
   __shared__ __align__(16) uint8_t lds[2 * kTileBytes];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * FT;
   const int nchunks = K / kSkChunk;
   const int R = (nchunks + kSkWaves - 1) / kSkWaves;
 
@@ -115,29 +121,36 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
   };
   const uint32_t rd_off = (uint32_t)i16 * kSkRowBytes + wave * 128 + g * 16;
 
-  f32x4 acc[TT];
+  f32x4 acc[FT][TT];
 #pragma unroll
-  for (int tt = 0; tt < TT; ++tt) acc[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) acc[ft][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // Rounds rb .. rb + 7.  Every load is issued unconditionally (clamped): a load under a
   // branch would leave the count of loads in flight unknown where the paths join, and the
   // waits that follow would then drain all of them.
-  constexpr bool kEarlyW = TT < 4;
-  Frag8 wf[kSkRounds][2];
+  constexpr bool kEarlyW = TT < 4 && FT == 1;
+  constexpr int kR = kSkRounds / FT;  // rounds per batch: 64 VGPRs of weights on their way
+  Frag8 wf[kR][FT][2];
   auto w_fetch = [&](const int rb) {
 #pragma unroll
-    for (int j = 0; j < kSkRounds; ++j) {
+    for (int j = 0; j < kR; ++j) {
       const int c = min((rb + j) * kSkWaves + wave, nchunks - 1);
-      wf[j][0].u = ld16(wp + c * kSkChunk);
-      wf[j][1].u = ld16(wp + c * kSkChunk + 32);
+#pragma unroll
+      for (int ft = 0; ft < FT; ++ft) {
+        wf[j][ft][0].u = ld16(wp + (size_t)ft * 16 * K + c * kSkChunk);
+        wf[j][ft][1].u = ld16(wp + (size_t)ft * 16 * K + c * kSkChunk + 32);
+      }
     }
   };
   auto batch = [&](const int rb) {
     if (rb > 0 || !kEarlyW) w_fetch(rb);  // else the first batch's weights are on their way
 #pragma unroll
-    for (int j = 0; j < kSkRounds; ++j) {
-      const int par = j & 1;  // = (rb + j) % 2: rb is a multiple of 8
+    for (int j = 0; j < kR; ++j) {
+      const int par = j & 1;  // = (rb + j) % 2: rb is a multiple of kR, which is even
       const int r = rb + j;
+      if (r >= R) break;  // (the same for every wave of the workgroup)
       // LDS tile `par` holds slab r, register stage par ^ 1 slab r + 1 (in flight)
       a_fetch(par, min(r + 2, R - 1));
       if (r * kSkWaves + wave < nchunks) {  // wave-uniform
@@ -147,8 +160,11 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
           const uint8_t *src = &lds[par * kTileBytes + rd_off + tt * 16 * kSkRowBytes];
           a0.u = *(const u32x4 *)src;
           a1.u = *(const u32x4 *)(src + 64);
-          acc[tt] = mfma16x32(wf[j][0], a0, acc[tt]);
-          acc[tt] = mfma16x32(wf[j][1], a1, acc[tt]);
+#pragma unroll
+          for (int ft = 0; ft < FT; ++ft) {
+            acc[ft][tt] = mfma16x32(wf[j][ft][0], a0, acc[ft][tt]);
+            acc[ft][tt] = mfma16x32(wf[j][ft][1], a1, acc[ft][tt]);
+          }
         }
       }
       a_stash(par ^ 1, par ^ 1);
@@ -163,17 +179,19 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
   a_fetch(1, min(1, R - 1));
   a_stash(0, 0);
   __syncthreads();
-  if (R <= kSkRounds) {
+  if (R <= kR) {
     batch(0);  // straight-line code for K <= 4096
   } else {
-    for (int rb = 0; rb < R; rb += kSkRounds) batch(rb);
+    for (int rb = 0; rb < R; rb += kR) batch(rb);
   }
 
-  f32x4(*red)[TT][64] = reinterpret_cast<f32x4(*)[TT][64]>(lds);  // all tile reads are done
+  f32x4(*red)[FT * TT][64] = reinterpret_cast<f32x4(*)[FT * TT][64]>(lds);  // all tile reads are done
 #pragma unroll
-  for (int tt = 0; tt < TT; ++tt) red[wave][tt][lane] = acc[tt];
+  for (int ft = 0; ft < FT; ++ft)
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) red[wave][ft * TT + tt][lane] = acc[ft][tt];
   __syncthreads();
-  if (wave < TT) {  // wave tt sums tile tt over the eight K shares and writes it out
+  if (wave < FT * TT) {  // wave (ft, tt) sums its tile over the eight K shares and writes it out
     f32x4 s = red[0][wave][lane];
 #pragma unroll
     for (int w2 = 1; w2 < kSkWaves; ++w2) {
@@ -183,8 +201,9 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
       s[2] += x[2];
       s[3] += x[3];
     }
-    const int t = wave * 16 + i16;
-    if (t < T) oproj_store(s, bias, resid, out, (size_t)t * N, n0 + 4 * g);
+    const int ft = wave / TT, tt = wave - ft * TT;
+    const int t = tt * 16 + i16;
+    if (t < T) oproj_store(s, bias, resid, out, (size_t)t * N, n0 + ft * 16 + 4 * g);
   }
 }
 
@@ -325,15 +344,29 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
                          hipStream_t st) {
   if (T == 0) return hipSuccess;
   if (T <= 64) {
-    const dim3 grid(N / 16), block(kSkWaves * 64);
+    const dim3 block(kSkWaves * 64);
+    // one workgroup per CU (registers, LDS): no more workgroups than CUs if that can be had
+    if (N / 16 > device_cus() && N % 32 == 0) {
+      const dim3 grid(N / 32);
+      if (T <= 16)
+        oproj_skinny_kernel<1, 2><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      else if (T <= 32)
+        oproj_skinny_kernel<2, 2><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      else if (T <= 48)
+        oproj_skinny_kernel<3, 2><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      else
+        oproj_skinny_kernel<4, 2><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      return hipGetLastError();
+    }
+    const dim3 grid(N / 16);
     if (T <= 16)
-      oproj_skinny_kernel<1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      oproj_skinny_kernel<1, 1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     else if (T <= 32)
-      oproj_skinny_kernel<2><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      oproj_skinny_kernel<2, 1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     else if (T <= 48)
-      oproj_skinny_kernel<3><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      oproj_skinny_kernel<3, 1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     else
-      oproj_skinny_kernel<4><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
+      oproj_skinny_kernel<4, 1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     return hipGetLastError();
   }
   // The 128 x 128 tile once it gives most CUs a workgroup, else 64 x 64 (measured

@@ -79,6 +79,16 @@ def test_streaming_kernel_shapes(G, T, N, K, with_bias, with_res):
     _run(G, T, N, K, with_bias, with_res, seed=T + N)
 
 
+# more 16-feature tiles than CUs: two tiles per workgroup (the QKV projection's shape,
+# 2880 -> 5120, for every token-tile count), short and ragged K, and a feature count that
+# cannot be paired (257 tiles: one tile per workgroup after all)
+@pytest.mark.parametrize("T,N,K", [(1, 5120, 2880), (16, 5120, 2880), (17, 5120, 2880),
+                                   (33, 5120, 2880), (49, 5120, 2880), (64, 5120, 2880),
+                                   (64, 8192, 128), (30, 4160, 4160), (9, 4112, 576)])
+def test_streaming_kernel_wide_outputs(G, T, N, K):
+    _run(G, T, N, K, True, T % 2 == 0, seed=T + K)
+
+
 # the 64 x 64 tile (few workgroups) and the 128 x 128 tile (the last three: 276, 288 and 286
 # big tiles), with ragged token counts and feature counts that end inside a tile
 @pytest.mark.parametrize("T,N,K", [(65, 2880, 4096), (128, 128, 64), (129, 16, 128), (200, 144, 576),
