@@ -574,6 +574,35 @@ def test_host_copies_of_the_lengths_plan_the_launches(G, kv_dtype, window, parti
     assert np.array_equal(both, out)   # the sum adds nothing the arrays do not say
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_seeded_small_batches_with_long_contexts(G, seed):
+    """One to six sequences with contexts drawn log-uniformly up to 20,000 tokens: the
+    regime where the host chooses between 512-key partitions with a wave per chunk and the
+    split-KV kernel, with and without the sum and the host copies of the lengths."""
+    rng = np.random.default_rng(5000 + seed)
+    S = int(rng.integers(1, 7))
+    q_lens = rng.choice([1, 1, 1, 2, 4, 5, 6], size=S)
+    if rng.random() < 0.5:
+        q_lens[:] = 1
+    top = int(rng.choice([600, 5000, 20000]))
+    ctx = np.exp(rng.uniform(0.0, np.log(top), size=S)).astype(np.int64)
+    seq_lens = q_lens + ctx
+    window = int(rng.choice([0, 0, 0, 128, 2000]))
+    kv_dtype = KV_FP8_E4M3 if rng.random() < 0.3 else KV_BF16
+    hint, host = bool(rng.random() < 0.5), bool(rng.random() < 0.6)
+    b = make_batch(seq_lens, q_lens, window=window, kv_dtype=kv_dtype, seed=seed)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, hint=hint,
+                          host_lens=host)
+    what = f"seed {seed}: L={seq_lens.tolist()} q={q_lens.tolist()} w={window} dtype={kv_dtype}"
+    assert_close(out, ref, what)
+    assert np.allclose(lse, ref_lse, atol=3e-3), what
+
+
 # ---------------------------------------------------------------- benchmark configurations
 def _sample_check(G, b, q_d, kc_d, vc_d, sinks, out_d, seqs, what, ks=None, vs=None):
     sub, kc, vc = G.compact_to_cpu(b, kc_d, vc_d, seqs)
