@@ -624,7 +624,8 @@ def main():
         "breakdown_us": {"kv_write": r["ms_kv_write"] * 1e3, "attn_call": r["ms_attn"] * 1e3,
                          "merge": r["ms_merge"] * 1e3,
                          "step_as_two_launches": r["ms_per_step_two_launches"] * 1e3},
-        "roofline": {"bound": "hbm", "kernel": "splitkv_kernel<1,bf16,8 waves>",
+        "roofline": {"bound": "hbm", "kernel": ("splitkv_kernel<1,bf16,8 waves>" if a.no_hint or os.environ.get("EID_NO_ITEM_TABLE")
+                                else "splitkv_table_kernel<1,bf16,8 waves>"),
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
                      "traffic": TRAFFIC_BYTES_PER_LAUNCH if a.partition == 0 and not a.no_shuffle else None,

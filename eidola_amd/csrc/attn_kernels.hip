@@ -752,6 +752,34 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds);
 }
 
+// The same for a decode launch whose items the host has listed (q_len 1, row = sequence):
+// no scan, no hand-over through LDS.
+__device__ __forceinline__ WorkItem table_item(const AttnParams &p, const ItemTable &tab,
+                                               const int w, const int P) {
+  const unsigned long long e = tab.e[w];
+  WorkItem it;
+  it.seq = (int)(e & 0xffffu);
+  it.part = (int)((e >> 16) & 0xffffu);
+  it.seq_len = (int)(e >> 32);
+  it.row0 = it.seq;
+  it.qlen = 1;
+  it.nparts = num_partitions(p, it.seq_len - kv_begin(it.seq_len, 1, p.window), P);
+  return it;
+}
+
+template <int NT, bool FP8, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_table_kernel(
+    const AttnParams p, const ItemTable tab) {
+  __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kvh = blockIdx.y * WAVES + wave;
+  if ((int)blockIdx.x >= tab.n) return;
+  const int P = p.partition;
+  const WorkItem it = table_item(p, tab, blockIdx.x, P);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
+  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds);
+}
+
 // ---------------------------------------------------------------------------------------
 // Short-span kernel: one wave per 64-token chunk.  When no sequence spans more than 8 chunks
 // (sliding-window layers, short contexts) a sequence is too short to be worth partitioning
@@ -773,7 +801,7 @@ constexpr int kShortWaves = 8;
 static_assert(kShortSpanMax == kShortWaves * kChunk, "one chunk per wave");
 
 template <int NT, bool FP8>
-__global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan_kernel(const AttnParams p) {
+__device__ __forceinline__ void shortspan_body(const AttnParams &p, const ItemTable *tab) {
   constexpr int kRows = NT * 16;
   constexpr int kPartBytes = kRows * kHeadDim * 4;  // one wave's fp32 accumulators
   constexpr int kWaveBytes = kPartBytes > kWaveLdsBytes ? kPartBytes : kWaveLdsBytes;
@@ -789,11 +817,17 @@ __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan
     if (v.span <= 0) return;  // not of this class, or malformed: the whole workgroup leaves
     L = v.seq_len, qlen = v.qlen, row0 = v.row0;
   } else {
-    // partitions of kShortSpanMax keys (the host set p.partition to that): every wave looks
-    // the item up for itself, there is nothing else to do yet and no barrier to wait at
+    // partitions of kShortSpanMax keys (the host set p.partition to that): the item comes
+    // from the host's list, or every wave looks it up for itself (there is nothing else to
+    // do yet and no barrier to wait at)
     WorkItem it;
-    int P;
-    if (!find_work_item(p, blockIdx.x, P, it)) return;
+    if (tab) {
+      if ((int)blockIdx.x >= tab->n) return;
+      it = table_item(p, *tab, blockIdx.x, kShortSpanMax);
+    } else {
+      int P;
+      if (!find_work_item(p, blockIdx.x, P, it)) return;
+    }
     s = it.seq, part = it.part, nparts = it.nparts;
     L = it.seq_len, qlen = it.qlen, row0 = it.row0;
   }
@@ -877,6 +911,16 @@ __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan
     *(uint32_t *)(p.out + orow * kHeadDim + d2) = pack_bf16(o0 * inv, o1 * inv);
     if (p.lse && d2 == 0) p.lse[orow] = (M + __log2f(den)) * kLn2;
   }
+}
+
+template <int NT, bool FP8>
+__global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan_kernel(const AttnParams p) {
+  shortspan_body<NT, FP8>(p, nullptr);
+}
+template <int NT, bool FP8>
+__global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan_table_kernel(
+    const AttnParams p, const ItemTable tab) {
+  shortspan_body<NT, FP8>(p, &tab);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1548,7 +1592,14 @@ long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, in
 
 // Short-span launch: see shortspan_kernel.  The caller has checked that no sequence spans
 // more than kShortSpanMax tokens.
-hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st) {
+hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st,
+                            const ItemTable *tab) {
+  if (tab && ntiles == 1 && p.nparts_max > 1) {  // decode launch with the host's item list
+    dim3 grid((unsigned)tab->n, p.num_kv_heads);
+    if (fp8) shortspan_table_kernel<1, true><<<grid, kShortWaves * 64, 0, st>>>(p, *tab);
+    else shortspan_table_kernel<1, false><<<grid, kShortWaves * 64, 0, st>>>(p, *tab);
+    return hipGetLastError();
+  }
   const long long items = p.exact_items > 0 && p.nparts_max > 1
                               ? p.exact_items
                               : shortspan_items(p.num_seqs, p.nparts_max, p.sum_kv_len, p.window);
@@ -1578,10 +1629,19 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same
 // params so that it uses the same partition.
-hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st) {
+hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
+                          const ItemTable *tab) {
   p.target_items_lo = fill_lo(p.target_items);
   p.plan = nullptr;
   p.plan_slot = plan_slot;
+  // decode launch with the host's item list (fixed partition, eight KV heads per workgroup)
+  if (tab && ntiles == 1 && p.nparts_max > 1 && !p.dynamic_partition && !p.share_cus &&
+      waves_for(p.num_kv_heads) == 8) {
+    dim3 grid((unsigned)tab->n, p.num_kv_heads / 8);
+    if (fp8) splitkv_table_kernel<1, true, 8><<<grid, 512, 0, st>>>(p, *tab);
+    else splitkv_table_kernel<1, false, 8><<<grid, 512, 0, st>>>(p, *tab);
+    return hipGetLastError();
+  }
   if (p.nparts_max > 1 && p.exact_items == 0 && item_bound(p) > 4LL * p.target_items) {
     AttnParams q = p;
     plan_kernel<<<1, 64, 0, st>>>(q, plan_slot);

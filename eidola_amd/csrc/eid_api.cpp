@@ -12,9 +12,11 @@
 #include <vector>
 
 namespace eid {
-hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st);
+hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
+                          const ItemTable *tab = nullptr);
 int splitkv_fill(int ntiles, bool fp8, int Hkv);
-hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st);
+hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st,
+                            const ItemTable *tab = nullptr);
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
 long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
@@ -293,7 +295,7 @@ int32_t hip_fail(hipError_t e, const char *what) {
 
 // Key spans of the sequences of one q_len class, as the kernels see them (view_seq).
 struct ClassSpans {
-  std::vector<int32_t> spans;
+  std::vector<int32_t> spans, seq, len;  // span, index and length of every such sequence
   long long total = 0;
   int32_t longest = 0;
   long long items(int32_t P, int32_t nparts_max) const {
@@ -307,12 +309,16 @@ ClassSpans class_spans(const eid_attn_desc *d, const int32_t *seq_lens, const in
                        int32_t ws_rows, int32_t qlen_lo, int32_t qlen_hi) {
   ClassSpans c;
   c.spans.reserve(d->num_seqs);
+  c.seq.reserve(d->num_seqs);
+  c.len.reserve(d->num_seqs);
   for (int32_t s = 0; s < d->num_seqs; ++s) {
     const int32_t L = seq_lens[s], qlen = cu ? cu[s + 1] - cu[s] : 1;
     if (qlen < qlen_lo || qlen > qlen_hi || qlen > ws_rows || L < qlen) continue;
     const int32_t span = L - eid::kv_begin(L, qlen, d->window);
     if (span <= 0) continue;
     c.spans.push_back(span);
+    c.seq.push_back(s);
+    c.len.push_back(L);
     c.total += span;
     c.longest = std::max(c.longest, span);
   }
@@ -368,8 +374,9 @@ struct ClassPlan {
 // descriptor alone; with them, the run-time choices of the kernels are made here.
 ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan &pl,
                      eid::AttnParams &p, int ntiles, int32_t qlen_lo, int32_t qlen_hi,
-                     bool decode) {
+                     bool decode, eid::ItemTable *table = nullptr) {
   ClassPlan cp;
+  if (table) table->n = 0;
   const bool fp8 = d->kv_dtype == EID_KV_FP8_E4M3;
   p.qlen_lo = qlen_lo;
   p.qlen_hi = qlen_hi;
@@ -407,6 +414,19 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   }
   p.exact_items = c.items(p.partition, pl.nparts_max);
   cp.merge = p.exact_items > (long long)c.spans.size();
+  // Few items of a decode launch: list them for the kernels (sequence-major, as they would
+  // find them themselves)
+  static const bool no_table = getenv("EID_NO_ITEM_TABLE") != nullptr;  // for A/B measurements
+  if (table && decode && !no_table && p.exact_items <= eid::kItemTableMax) {
+    int32_t n = 0;
+    for (size_t i = 0; i < c.spans.size(); ++i) {
+      const int32_t parts = std::min((c.spans[i] + p.partition - 1) / p.partition, pl.nparts_max);
+      for (int32_t part = 0; part < parts; ++part)
+        table->e[n++] = (unsigned long long)(uint32_t)c.seq[i] | (unsigned long long)part << 16 |
+                        (unsigned long long)(uint32_t)c.len[i] << 32;
+    }
+    table->n = n;
+  }
   return cp;
 }
 
@@ -500,12 +520,14 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true);
+  eid::ItemTable table;  // (3 KiB on the stack; only `n` entries are ever read)
+  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table);
   if (cp.skip) return EID_OK;  // (every sequence empty or malformed: nothing is written)
+  const eid::ItemTable *tab = table.n > 0 ? &table : nullptr;
   // spans of at most 8 chunks, or a small batch in partitions of that size: one workgroup
   // per (sequence, partition, KV head), a chunk per wave
-  hipError_t e = cp.short_span ? eid::launch_shortspan(p, 1, fp8, st)
-                               : eid::launch_splitkv(p, 1, fp8, plan_slots, st);
+  hipError_t e = cp.short_span ? eid::launch_shortspan(p, 1, fp8, st, tab)
+                               : eid::launch_splitkv(p, 1, fp8, plan_slots, st, tab);
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (args->split_done_event) {
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);

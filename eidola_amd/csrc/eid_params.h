@@ -54,6 +54,15 @@ struct AttnParams {
   float softmax_scale;
 };
 
+// Work items of a decode launch listed by the host (it has the sequence lengths): entry =
+// seq | part << 16 | seq_len << 32.  Passed by value as a kernel argument, so a workgroup has
+// its item after one scalar load instead of a scan of seq_lens.
+constexpr int kItemTableMax = 384;
+struct ItemTable {
+  int32_t n, pad;
+  unsigned long long e[kItemTableMax];
+};
+
 // First key visible to any query row of a sequence, rounded down to a page boundary.
 __host__ __device__ inline int kv_begin(int seq_len, int q_len, int window) {
   int p0 = seq_len - q_len;
