@@ -125,6 +125,8 @@ class Workload:
                       sum_kv_len=0 if NO_HINT else int(b0.seq_lens.sum()),
                       seq_lens_host=None if NO_HINT else b0.seq_lens,
                       cu_seqlens_q_host=None if NO_HINT or kind != "varlen" else b0.cu_seqlens_q)
+            if kind == "decode" and not NO_HINT:
+                kw["block_table_host"] = bt.cpu().numpy()
             cu = self.cu if kind == "varlen" else None
             c = ea.prepare(fn, g, self.q, self.k_cache, self.v_cache, bt, self.seq_lens, cu, **kw)
             ws = c._keep[-1]

@@ -76,6 +76,7 @@ class AttnArgs(C.Structure):
         ("v_new", C.c_void_p),
         ("seq_lens_host", C.c_void_p),
         ("cu_seqlens_q_host", C.c_void_p),
+        ("block_table_host", C.c_void_p),
     ]
 
 

@@ -190,13 +190,19 @@ __device__ __forceinline__ u32x4 quantize16_fp8(const u32x4 lo, const u32x4 hi, 
 // kv_write_kernel would have used, so the step needs no separate write launch.  Key ranges
 // of different partitions are disjoint and every wave owns one KV head: exactly one lane
 // group writes each (sequence, head) row, and nobody else reads it in this launch.
+// Page ids of a work item's first chunk, when the launch carries them (else have == 0).
+struct FirstPages {
+  int have = 0;
+  int id[4] = {0, 0, 0, 0};
+};
+
 template <int NT, bool FP8>
 __device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
                                        const int t_begin, const int t_end, const int seq_len,
                                        const int pos_first, const int lo_last,
                                        const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                        uint8_t *wave_lds, float (&m)[NT], f32x4 (&lacc)[NT],
-                                       f32x4 (&acc)[NT][4]) {
+                                       f32x4 (&acc)[NT][4], const FirstPages &first = FirstPages{}) {
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
   const int Hkv = p.num_kv_heads;
@@ -223,8 +229,13 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   const int pos_new = (NT == 1 && p.k_new && seq_len - 1 >= t_begin && seq_len - 1 < t_end)
                           ? seq_len - 1 : -1;
   int blk[kPages];
+  if (first.have) {  // (wave-uniform) the launch brought the first chunk's page ids along
 #pragma unroll
-  for (int b = 0; b < kPages; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
+    for (int b = 0; b < kPages; ++b) blk[b] = first.id[b];
+  } else {
+#pragma unroll
+    for (int b = 0; b < kPages; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
+  }
 
   for (int ti = t_begin; ti < t_end; ti += kIter) {
     const int nbi = min(kPages, (t_end - ti + kBlock - 1) / kBlock);
@@ -665,7 +676,8 @@ __global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *p
 // partition it.part (P tokens) of sequence it.seq and writes the output or the partial.
 template <int NT, bool FP8>
 __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem &it, const int P,
-                                             const int kvh, const int wave, uint8_t *lds) {
+                                             const int kvh, const int wave, uint8_t *lds,
+                                             const FirstPages &first = FirstPages{}) {
   const int s = it.seq, part = it.part, nparts = it.nparts;
   const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
   const int kb = kv_begin(L, qlen, p.window);
@@ -687,7 +699,7 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
-                  lacc, acc);
+                  lacc, acc, first);
   finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lacc, acc);
 }
 
@@ -777,7 +789,11 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_table_k
   const int P = p.partition;
   const WorkItem it = table_item(p, tab, blockIdx.x, P);
   if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
-  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds);
+  FirstPages first;  // (read element by element: a pointer into the argument would make the
+  first.have = tab.has_blk;  // compiler copy the whole list into private memory)
+#pragma unroll
+  for (int b = 0; b < 4; ++b) first.id[b] = tab.blk[blockIdx.x][b];
+  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds, first);
 }
 
 // ---------------------------------------------------------------------------------------

@@ -376,7 +376,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
                      eid::AttnParams &p, int ntiles, int32_t qlen_lo, int32_t qlen_hi,
                      bool decode, eid::ItemTable *table = nullptr) {
   ClassPlan cp;
-  if (table) table->n = 0;
+  if (table) table->n = table->has_blk = 0;
   const bool fp8 = d->kv_dtype == EID_KV_FP8_E4M3;
   p.qlen_lo = qlen_lo;
   p.qlen_hi = qlen_hi;
@@ -419,13 +419,24 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   static const bool no_table = getenv("EID_NO_ITEM_TABLE") != nullptr;  // for A/B measurements
   if (table && decode && !no_table && p.exact_items <= eid::kItemTableMax) {
     int32_t n = 0;
+    const int32_t *bth = a->block_table_host;
     for (size_t i = 0; i < c.spans.size(); ++i) {
       const int32_t parts = std::min((c.spans[i] + p.partition - 1) / p.partition, pl.nparts_max);
-      for (int32_t part = 0; part < parts; ++part)
+      const int32_t L = c.len[i], kb = eid::kv_begin(L, 1, d->window);
+      for (int32_t part = 0; part < parts; ++part) {
+        if (bth) {  // the ids the kernel would fetch for the item's first chunk (see attend)
+          const int32_t t0 = kb + part * p.partition, t1 = std::min(t0 + p.partition, L);
+          const int32_t last = (t1 + eid::kBlock - 1) / eid::kBlock - 1;
+          for (int32_t b = 0; b < 4; ++b)
+            table->blk[n][b] = bth[(size_t)c.seq[i] * d->max_blocks_per_seq +
+                                   std::min(t0 / eid::kBlock + b, last)];
+        }
         table->e[n++] = (unsigned long long)(uint32_t)c.seq[i] | (unsigned long long)part << 16 |
-                        (unsigned long long)(uint32_t)c.len[i] << 32;
+                        (unsigned long long)(uint32_t)L << 32;
+      }
     }
     table->n = n;
+    table->has_blk = bth ? 1 : 0;
   }
   return cp;
 }

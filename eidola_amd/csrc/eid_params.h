@@ -59,8 +59,10 @@ struct AttnParams {
 // its item after one scalar load instead of a scan of seq_lens.
 constexpr int kItemTableMax = 384;
 struct ItemTable {
-  int32_t n, pad;
+  int32_t n;
+  int32_t has_blk;  // blk[] holds the page ids of every item's first four pages
   unsigned long long e[kItemTableMax];
+  int32_t blk[kItemTableMax][4];
 };
 
 // First key visible to any query row of a sequence, rounded down to a page boundary.

@@ -224,10 +224,24 @@ def _host_i32(a, name, n):
     return a
 
 
+def _host_bt(a, block_table):
+    """A host copy of the block table as contiguous int32 numpy of the device table's shape."""
+    if a is None:
+        return None
+    if isinstance(a, torch.Tensor):
+        if a.is_cuda:
+            raise ValueError("block_table_host must live in host memory")
+        a = a.numpy()
+    a = np.ascontiguousarray(a, dtype=np.int32)
+    if a.shape != tuple(block_table.shape):
+        raise ValueError("block_table_host must have the shape of block_table")
+    return a
+
+
 def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q,
                max_q_len, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace,
                return_lse, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None,
-               cu_seqlens_q_host=None):
+               cu_seqlens_q_host=None, block_table_host=None):
     _require(q, "q", torch.bfloat16, 3)
     k_cache = _cache_view(k_cache, geom, "k_cache")
     v_cache = _cache_view(v_cache, geom, "v_cache")
@@ -287,6 +301,8 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
     cu_h = _host_i32(cu_seqlens_q_host, "cu_seqlens_q_host", S + 1)
     args.seq_lens_host = sl_h.ctypes.data if sl_h is not None else None
     args.cu_seqlens_q_host = cu_h.ctypes.data if cu_h is not None else None
+    bt_h = _host_bt(block_table_host, block_table)
+    args.block_table_host = bt_h.ctypes.data if bt_h is not None else None
     check(getattr(lib, fn_name)(C.byref(desc), C.byref(args), _stream()))
     return (out, lse) if return_lse else out
 
@@ -312,7 +328,7 @@ class PreparedCall:
 def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, *,
             max_q_len=1, max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
             workspace=None, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None,
-            cu_seqlens_q_host=None):
+            cu_seqlens_q_host=None, block_table_host=None):
     """Build a PreparedCall for "eid_attn_decode" / "eid_attn_varlen" / "eid_lse_merge".
     `seq_lens_host` / `cu_seqlens_q_host` (host copies of the two length arrays) are copied
     and kept by the object."""
@@ -352,15 +368,19 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
     cu_h = cu_h.copy() if cu_h is not None else None
     args.seq_lens_host = sl_h.ctypes.data if sl_h is not None else None
     args.cu_seqlens_q_host = cu_h.ctypes.data if cu_h is not None else None
+    bt_h = _host_bt(block_table_host, block_table)
+    bt_h = bt_h.copy() if bt_h is not None else None
+    args.block_table_host = bt_h.ctypes.data if bt_h is not None else None
     keep = (q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, sinks, k_scale, v_scale,
-            k_new, v_new, sl_h, cu_h,
+            k_new, v_new, sl_h, cu_h, bt_h,
             workspace)  # workspace stays last: callers share it via _keep[-1]
     return PreparedCall(fn_name, desc, args, keep, out, lse)
 
 
 def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, sinks=None,
                 k_scale=None, v_scale=None, out=None, lse=None, workspace=None,
-                return_lse=False, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None):
+                return_lse=False, sum_kv_len=0, k_new=None, v_new=None, seq_lens_host=None,
+                block_table_host=None):
     """Stages K2+K4: one query row per sequence (q is [num_seqs, Hq, D]).  `sum_kv_len` is the
     optional host-side sum of seq_lens (any upper bound): it sizes the launch to the work;
     `seq_lens_host`, a host copy of seq_lens, lets the library plan the launch exactly.
@@ -368,7 +388,7 @@ def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len,
     yet in the cache) the call writes those rows into the caches itself (stage K1 fused)."""
     return _attn_call("eid_attn_decode", geom, q, k_cache, v_cache, block_table, seq_lens, None,
                       1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse,
-                      sum_kv_len, k_new, v_new, seq_lens_host)
+                      sum_kv_len, k_new, v_new, seq_lens_host, None, block_table_host)
 
 
 def attn_varlen(geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, *, max_q_len,

@@ -120,6 +120,10 @@ typedef struct eid_attn_args {
                            which kernels have work at all) instead of leaving that to every
                            workgroup of the kernels.  They must equal the device arrays;
                            results do not depend on whether they are given. */
+  const int32_t *block_table_host;  /* optional HOST copy of block_table (same shape), used by
+                           eid_attn_decode together with seq_lens_host: the page ids of every
+                           work item's first chunk then travel with the launch instead of
+                           being fetched by the workgroup before its first K/V load */
 } eid_attn_args;
 
 /*

@@ -64,6 +64,8 @@ def run_attn(batch, q, kc_d, vc_d, sinks, k_scale=None, v_scale=None, *, decode=
     if host_lens:
         kw["seq_lens_host"] = batch.seq_lens
     if decode:
+        if host_lens:
+            kw["block_table_host"] = batch.block_table
         r = ea.attn_decode(geom, bf16_dev(q), kc_d, vc_d, bt, sl, **kw)
     else:
         if host_lens:

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layout_matches_header():
     assert C.sizeof(AttnDesc) == 72
     assert AttnDesc.num_blocks.offset == 40 and AttnDesc.softmax_scale.offset == 48
-    assert C.sizeof(AttnArgs) == 18 * 8
+    assert C.sizeof(AttnArgs) == 19 * 8
 
 
 def test_workspace_and_partition_planning():

@@ -658,6 +658,11 @@ def test_config2_full_size(G, window):
                         sum_kv_len=int(b.seq_lens.sum()), seq_lens_host=b.seq_lens)
     torch.cuda.synchronize()
     assert torch.equal(oh, out)
+    # ... and with the host copy of the block table the first chunk's page ids come along
+    oh = ea.attn_decode(*args, max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
+                        seq_lens_host=b.seq_lens, block_table_host=b.block_table)
+    torch.cuda.synchronize()
+    assert torch.equal(oh, out)
 
 
 def test_config3_mixed_full_size(G):
