@@ -432,7 +432,7 @@ def small_batch_bench(torch, ea, synth):
     return out
 
 
-def stack_bench(torch, ea, synth, layers=36):
+def stack_bench(torch, ea, synth, layers=36, fused_qkv=True):
     """The attention block of every layer of ONE decode step, replayed from one HIP graph:
     per layer the QKV projection (the library's GEMM entry point, 2880 -> 5120 with bias),
     rotary embedding + split + KV write, paged sink-attention (even layers a 128-token
@@ -478,8 +478,12 @@ def stack_bench(torch, ea, synth, layers=36):
     def step(stream=None):
         hidden.copy_(hidden0)
         for L in lay:
-            ea.o_proj(hidden, L["wqkv"], L["bqkv"], out=qkv)
-            ea.rope_kv_write(L["geom"], qkv, pos, cos_sin, kc, vc, L["slots"], q_out=q)
+            if fused_qkv:
+                ea.qkv_rope_kv_write(L["geom"], hidden, L["wqkv"], L["bqkv"], pos, cos_sin, kc, vc,
+                                     L["slots"], q_out=q)
+            else:
+                ea.o_proj(hidden, L["wqkv"], L["bqkv"], out=qkv)
+                ea.rope_kv_write(L["geom"], qkv, pos, cos_sin, kc, vc, L["slots"], q_out=q)
             L["attn"](stream=stream)
             ea.o_proj(L["attn"].out, L["wo"], L["bo"], residual=hidden, out=hidden)
 
@@ -502,11 +506,13 @@ def stack_bench(torch, ea, synth, layers=36):
     kv_bytes = sum(synth.algorithmic_work(synth.config2(window=0 if l % 2 else 128))["bytes"]
                    for l in range(layers))
     w_bytes = layers * (NQKV * H + H * 4096) * 2
-    r = {"config": f"attention_stack_{layers}_layers_config2_batch", "ms": ms, "ms_eager": ms_eager,
+    r = {"config": f"attention_stack_{layers}_layers_config2_batch" + ("" if fused_qkv else "_qkv_unfused"),
+         "ms": ms, "ms_eager": ms_eager,
          "layers": layers, "us_per_layer": ms * 1e3 / layers, "kv_bytes": kv_bytes,
          "weight_bytes": w_bytes, "GBps": (kv_bytes + w_bytes) / ms / 1e6, "finite": ok}
-    log(f"[bench] attention stack, {layers} layers x (QKV proj, RoPE + KV write, attention, "
-        f"o_proj), 64 seqs: {ms*1e3:.0f} us per decode step from one graph "
+    log(f"[bench] attention stack, {layers} layers x ("
+        + ("QKV proj + RoPE + KV write in one launch" if fused_qkv else "QKV proj, RoPE + KV write")
+        + f", attention, o_proj), 64 seqs: {ms*1e3:.0f} us per decode step from one graph "
         f"({ms*1e3/layers:.1f} us per layer, {ms_eager*1e3:.0f} us launched eagerly); "
         f"{(kv_bytes + w_bytes)/1e9:.2f} GB of KV + weights -> {r['GBps']:.0f} GB/s; "
         f"{S / ms * 1e3:.0f} tokens/s bound from attention blocks alone")
@@ -699,6 +705,7 @@ def main():
         if want("small"):
             extra.extend(small_batch_bench(torch, ea, synth))
         if want("stack"):
+            extra.extend(stack_bench(torch, ea, synth, fused_qkv=False))
             extra.extend(stack_bench(torch, ea, synth))
         w = Workload(lambda off: synth.config2(perm_offset=off), 1, 7, torch, ea, synth, "decode")
     if not a.no_cpu:

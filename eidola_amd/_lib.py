@@ -100,7 +100,7 @@ class BatchInfo(C.Structure):
     ]
 
 
-EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
+EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_qkv_rope_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
            "eid_o_proj",
            "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
@@ -134,6 +134,9 @@ def load_library():
     lib.eid_rope_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, C.c_int32, P, P, P, P,
                                       C.c_int32, P, P, P]
     lib.eid_rope_kv_write.restype = C.c_int32
+    lib.eid_qkv_rope_kv_write.argtypes = [C.POINTER(AttnDesc), P, P, P, C.c_int32, P, P, C.c_int32,
+                                          P, P, P, P, C.c_int32, P, P, P]
+    lib.eid_qkv_rope_kv_write.restype = C.c_int32
     lib.eid_o_proj.argtypes = [P, P, P, P, P, C.c_int32, C.c_int32, C.c_int32, P]
     lib.eid_o_proj.restype = C.c_int32
     for name in ("eid_attn_decode", "eid_attn_varlen", "eid_lse_merge"):

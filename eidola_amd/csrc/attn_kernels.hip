@@ -151,23 +151,6 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
   }
 }
 
-// Software round-to-nearest-even onto the OCP e4m3fn grid, saturating at +-448; NaN -> 0x7F.
-__device__ __forceinline__ uint32_t fp8_e4m3_encode(float x) {
-  const uint32_t u = __float_as_uint(x);
-  const uint32_t sign = (u >> 24) & 0x80u;
-  const uint32_t a = u & 0x7fffffffu;
-  if (a > 0x7f800000u) return 0x7Fu;
-  if (a >= 0x43E00000u) return sign | 0x7Eu;  // |x| >= 448
-  if (a >= (121u << 23)) {                    // normal in e4m3: |x| >= 2^-6
-    uint32_t r = a + 0x7FFFFu + ((a >> 20) & 1u);
-    r >>= 20;  // exponent and 3 mantissa bits, carry propagated
-    return sign | (r - (120u << 3));
-  }
-  // subnormal: multiples of 2^-9; 8 rounds up into the smallest normal (0x08)
-  const float y = __uint_as_float(a) * 512.0f;
-  return sign | (uint32_t)__float2int_rn(y);
-}
-
 // 16 bf16 values -> 16 fp8-e4m3fn bytes, RNE of x / scale (the arithmetic of kv_write_kernel)
 __device__ __forceinline__ u32x4 quantize16_fp8(const u32x4 lo, const u32x4 hi, const float sc) {
   u32x4 o = {0, 0, 0, 0};

@@ -28,6 +28,8 @@ hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
                                 int64_t num_slots, int num_tokens, bool fp8, hipStream_t st);
 int device_cus();
 long long prefill_tiles_bound(int num_q_tokens, int num_seqs);
+hipError_t launch_qkv_rope(const uint16_t *a, const uint16_t *w, const uint16_t *bias, int T, int K,
+                           const RopeArgs &r, hipStream_t st);
 hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
                          const uint16_t *resid, uint16_t *out, int T, int N, int K,
                          hipStream_t st);
@@ -510,6 +512,52 @@ int32_t eid_rope_kv_write(const eid_attn_desc *desc, const void *qkv, const int3
       desc->num_kv_heads, desc->num_blocks * desc->block_size, num_tokens, fp8,
       static_cast<hipStream_t>(hip_stream));
   if (e != hipSuccess) return hip_fail(e, "rope_kv_write launch");
+  return EID_OK;
+}
+
+int32_t eid_qkv_rope_kv_write(const eid_attn_desc *desc, const void *hidden, const void *weight,
+                              const void *bias, int32_t in_features, const int32_t *positions,
+                              const float *cos_sin, int32_t max_pos, void *q_out, void *k_cache,
+                              void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
+                              const float *k_scale, const float *v_scale, void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_geometry(desc)) return rc;
+  if (num_tokens < 0) return fail(EID_ERR_INVALID_ARG, "num_tokens %d < 0", num_tokens);
+  if (num_tokens > 64)
+    return fail(EID_ERR_UNSUPPORTED, "num_tokens %d > 64: use eid_o_proj, then eid_rope_kv_write",
+                num_tokens);
+  if (max_pos <= 0) return fail(EID_ERR_INVALID_ARG, "max_pos %d must be positive", max_pos);
+  if (in_features <= 0 || in_features % 64 != 0)
+    return fail(EID_ERR_INVALID_ARG, "in_features %d must be a positive multiple of 64", in_features);
+  if (num_tokens == 0) return EID_OK;
+  if (!hidden || !weight || !positions || !cos_sin || !q_out || !k_cache || !v_cache || !slot_mapping)
+    return fail(EID_ERR_INVALID_ARG, "hidden, weight, positions, cos_sin, q_out, k_cache, v_cache, "
+                                     "slot_mapping must be non-NULL");
+  if (!aligned16(hidden) || !aligned16(weight) || !aligned16(cos_sin) || !aligned16(q_out) ||
+      !aligned16(k_cache) || !aligned16(v_cache))
+    return fail(EID_ERR_INVALID_ARG,
+                "hidden, weight, cos_sin, q_out, k_cache and v_cache must be 16-byte aligned");
+  const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  if (fp8 && (!k_scale || !v_scale)) return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
+  eid::RopeArgs r;
+  r.positions = positions;
+  r.cos_sin = cos_sin;
+  r.q_out = static_cast<uint16_t *>(q_out);
+  r.k_cache = static_cast<uint8_t *>(k_cache);
+  r.v_cache = static_cast<uint8_t *>(v_cache);
+  r.slot_mapping = slot_mapping;
+  r.k_scale = k_scale;
+  r.v_scale = v_scale;
+  r.num_slots = desc->num_blocks * desc->block_size;
+  r.max_pos = max_pos;
+  r.Hq = desc->num_q_heads;
+  r.Hkv = desc->num_kv_heads;
+  r.fp8 = fp8 ? 1 : 0;
+  hipError_t e = eid::launch_qkv_rope(static_cast<const uint16_t *>(hidden),
+                                      static_cast<const uint16_t *>(weight),
+                                      static_cast<const uint16_t *>(bias), num_tokens, in_features, r,
+                                      static_cast<hipStream_t>(hip_stream));
+  if (e != hipSuccess) return hip_fail(e, "qkv_rope_kv_write launch");
   return EID_OK;
 }
 

@@ -77,6 +77,24 @@ __device__ __forceinline__ void fp8x8_to_bf16x8(uint32_t d0, uint32_t d1, uint32
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
+// Software round-to-nearest-even onto the OCP e4m3fn grid, saturating at +-448; NaN -> 0x7F.
+__device__ __forceinline__ uint32_t fp8_e4m3_encode(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const uint32_t sign = (u >> 24) & 0x80u;
+  const uint32_t a = u & 0x7fffffffu;
+  if (a > 0x7f800000u) return 0x7Fu;
+  if (a >= 0x43E00000u) return sign | 0x7Eu;  // |x| >= 448
+  if (a >= (121u << 23)) {                    // normal in e4m3: |x| >= 2^-6
+    uint32_t r = a + 0x7FFFFu + ((a >> 20) & 1u);
+    r >>= 20;  // exponent and 3 mantissa bits, carry propagated
+    return sign | (r - (120u << 3));
+  }
+  // subnormal: multiples of 2^-9; 8 rounds up into the smallest normal (0x08)
+  const float y = __uint_as_float(a) * 512.0f;
+  return sign | (uint32_t)__float2int_rn(y);
+}
+
+
 // LDS transpose read (gfx950 ds_read_b64_tr_b16).  Within each 16-lane row, treat the
 // 16 lanes x 4 halfwords addressed by the lanes as a flat array F[lane*4 + e]; lane i
 // receives F[i], F[16+i], F[32+i], F[48+i].

@@ -65,6 +65,18 @@ struct ItemTable {
   int32_t blk[kItemTableMax][4];
 };
 
+// What the QKV projection needs to finish as rope_kv_write_kernel would (see oproj_kernels.hip).
+struct RopeArgs {
+  const int32_t *positions;
+  const float *cos_sin;
+  uint16_t *q_out;
+  uint8_t *k_cache, *v_cache;
+  const int64_t *slot_mapping;
+  const float *k_scale, *v_scale;
+  int64_t num_slots;
+  int max_pos, Hq, Hkv, fp8;
+};
+
 // First key visible to any query row of a sequence, rounded down to a page boundary.
 __host__ __device__ inline int kv_begin(int seq_len, int q_len, int window) {
   int p0 = seq_len - q_len;

@@ -26,6 +26,7 @@
 #include <stdint.h>
 
 #include "eid_device.h"
+#include "eid_params.h"
 
 namespace eid {
 
@@ -83,11 +84,22 @@ constexpr int kSkRowBytes = kSkSlab * 2 + 16;      // LDS row of an activation s
 // activations, whatever the number of features, and with three or four token tiles only one
 // workgroup fits a CU (LDS): when N / 16 exceeds the number of CUs, two feature tiles per
 // workgroup (N % 32 == 0) finish in one round of workgroups instead of two.
-template <int TT, int FT>
+//
+// ROPE (FT == 2, N = (Hq + 2 Hkv) * 64: the QKV projection of a decode step): the two feature
+// tiles of a workgroup are dims d..d+15 and d+32..d+47 of one head row, i.e. the partners of
+// the half-split rotary embedding, and the epilogue does what rope_kv_write_kernel would do
+// with the projection's bf16 output: rotate q and k rows by the token's position, store q
+// rows to q_out and k / v rows into their cache slot (bf16 copy or fp8 quantisation), with
+// the same arithmetic on the same bf16-rounded values, so the results are bit-identical to
+// the two launches and the [T, N] intermediate never exists.
+
+template <int TT, int FT, bool ROPE = false>
 __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
-    uint16_t *out, const int T, const int N, const int K) {
+    uint16_t *out, const int T, const int N, const int K, const RopeArgs rope = RopeArgs{}) {
+  static_assert(!ROPE || FT == 2, "the rotation pairs two feature tiles");
+  constexpr int kFtStride = ROPE ? 32 : 16;  // features between the workgroup's two tiles
   constexpr int kRows = TT * 16;
   constexpr int kLd = kRows / kSkWaves;  // slab rows per wave = loads per thread and slab
   constexpr int kTileBytes = kRows * kSkRowBytes;
@@ -97,7 +109,7 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16 * FT;
+  const int n0 = ROPE ? (blockIdx.x >> 1) * 64 + (blockIdx.x & 1) * 16 : blockIdx.x * 16 * FT;
   const int nchunks = K / kSkChunk;
   const int R = (nchunks + kSkWaves - 1) / kSkWaves;
 
@@ -127,6 +139,21 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) acc[ft][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
+  // ROPE: what the epilogue needs from memory (position -> cos / sin row, cache slot) is
+  // requested now by the waves that will need it, and has long arrived when the sums are done.
+  f32x4 rope_c = {1.f, 1.f, 1.f, 1.f}, rope_s = {0.f, 0.f, 0.f, 0.f};
+  int64_t rope_slot = -1;
+  if constexpr (ROPE) {
+    if (wave < TT) {
+      const int t = min(wave * 16 + i16, T - 1);
+      const int pos = min(max(rope.positions[t], 0), rope.max_pos - 1);
+      const float *cs = rope.cos_sin + (size_t)pos * 64 + (n0 & 63) + 4 * g;
+      rope_c = *(const f32x4 *)cs;
+      rope_s = *(const f32x4 *)(cs + 32);
+      rope_slot = rope.slot_mapping[t];
+    }
+  }
+
   // Rounds rb .. rb + 7.  Every load is issued unconditionally (clamped): a load under a
   // branch would leave the count of loads in flight unknown where the paths join, and the
   // waits that follow would then drain all of them.
@@ -139,8 +166,8 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
       const int c = min((rb + j) * kSkWaves + wave, nchunks - 1);
 #pragma unroll
       for (int ft = 0; ft < FT; ++ft) {
-        wf[j][ft][0].u = ld16(wp + (size_t)ft * 16 * K + c * kSkChunk);
-        wf[j][ft][1].u = ld16(wp + (size_t)ft * 16 * K + c * kSkChunk + 32);
+        wf[j][ft][0].u = ld16(wp + (size_t)ft * kFtStride * K + c * kSkChunk);
+        wf[j][ft][1].u = ld16(wp + (size_t)ft * kFtStride * K + c * kSkChunk + 32);
       }
     }
   };
@@ -191,6 +218,79 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 #pragma unroll
     for (int tt = 0; tt < TT; ++tt) red[wave][ft * TT + tt][lane] = acc[ft][tt];
   __syncthreads();
+  if constexpr (ROPE) {
+    if (wave < TT) {  // wave tt: both tiles of token tile tt, rotation, stores
+      f32x4 s1 = red[0][wave][lane], s2 = red[0][TT + wave][lane];
+#pragma unroll
+      for (int w2 = 1; w2 < kSkWaves; ++w2) {
+        const f32x4 x = red[w2][wave][lane], y = red[w2][TT + wave][lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s1[e] += x[e];
+          s2[e] += y[e];
+        }
+      }
+      const int t = wave * 16 + i16;
+      if (t >= T) return;
+      const int head = n0 >> 6, d1 = (n0 & 63) + 4 * g;  // head row of [q | k | v], dim of s1[0]
+      // the projection's output as eid_o_proj would have stored it: + bias, one bf16 rounding
+      float x1[4], x2[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v1 = s1[e], v2 = s2[e];
+        if (bias) {
+          v1 += bf16_bits_to_f32(bias[n0 + 4 * g + e]);
+          v2 += bf16_bits_to_f32(bias[n0 + 32 + 4 * g + e]);
+        }
+        x1[e] = bf16_bits_to_f32(pack_bf16(v1, 0.f) & 0xffffu);
+        x2[e] = bf16_bits_to_f32(pack_bf16(v2, 0.f) & 0xffffu);
+      }
+      const bool is_v = head >= rope.Hq + rope.Hkv;
+      float o1[4], o2[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        o1[e] = x1[e];
+        o2[e] = x2[e];
+      }
+      if (!is_v) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          o1[e] = __builtin_fmaf(-x2[e], rope_s[e], __fmul_rn(x1[e], rope_c[e]));
+          o2[e] = __builtin_fmaf(x1[e], rope_s[e], __fmul_rn(x2[e], rope_c[e]));
+        }
+      }
+      const u32x2 p1 = {pack_bf16(o1[0], o1[1]), pack_bf16(o1[2], o1[3])};
+      const u32x2 p2 = {pack_bf16(o2[0], o2[1]), pack_bf16(o2[2], o2[3])};
+      if (head < rope.Hq) {
+        uint16_t *dst = rope.q_out + ((size_t)t * rope.Hq + head) * 64 + d1;
+        *(u32x2 *)dst = p1;
+        *(u32x2 *)(dst + 32) = p2;
+        return;
+      }
+      const int64_t slot = rope_slot;
+      if (slot < 0 || slot >= rope.num_slots) return;
+      const int kh = is_v ? head - rope.Hq - rope.Hkv : head - rope.Hq;
+      uint8_t *cache = is_v ? rope.v_cache : rope.k_cache;
+      const size_t elem = ((size_t)slot * rope.Hkv + kh) * 64 + d1;
+      if (rope.fp8) {
+        const float sc = (is_v ? rope.v_scale : rope.k_scale)[kh];
+        uint32_t q1 = 0, q2 = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float r1 = bf16_bits_to_f32((p1[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+          const float r2 = bf16_bits_to_f32((p2[e >> 1] >> ((e & 1) * 16)) & 0xffffu);
+          q1 |= fp8_e4m3_encode(__fdiv_rn(r1, sc)) << (e * 8);
+          q2 |= fp8_e4m3_encode(__fdiv_rn(r2, sc)) << (e * 8);
+        }
+        *(uint32_t *)(cache + elem) = q1;
+        *(uint32_t *)(cache + elem + 32) = q2;
+      } else {
+        *(u32x2 *)(cache + elem * 2) = p1;
+        *(u32x2 *)(cache + (elem + 32) * 2) = p2;
+      }
+    }
+    return;
+  }
   if (wave < FT * TT) {  // wave (ft, tt) sums its tile over the eight K shares and writes it out
     f32x4 s = red[0][wave][lane];
 #pragma unroll
@@ -381,6 +481,23 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
     oproj_tiled_kernel<2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
                                                             tiles_m, tiles_n);
   }
+  return hipGetLastError();
+}
+
+// QKV projection + rotary embedding + split + KV write in one launch (decode batches).
+hipError_t launch_qkv_rope(const uint16_t *a, const uint16_t *w, const uint16_t *bias, int T, int K,
+                           const RopeArgs &r, hipStream_t st) {
+  if (T == 0) return hipSuccess;
+  const int N = (r.Hq + 2 * r.Hkv) * 64;
+  const dim3 grid(N / 32), block(kSkWaves * 64);
+  if (T <= 16)
+    oproj_skinny_kernel<1, 2, true><<<grid, block, 0, st>>>(a, w, bias, nullptr, nullptr, T, N, K, r);
+  else if (T <= 32)
+    oproj_skinny_kernel<2, 2, true><<<grid, block, 0, st>>>(a, w, bias, nullptr, nullptr, T, N, K, r);
+  else if (T <= 48)
+    oproj_skinny_kernel<3, 2, true><<<grid, block, 0, st>>>(a, w, bias, nullptr, nullptr, T, N, K, r);
+  else
+    oproj_skinny_kernel<4, 2, true><<<grid, block, 0, st>>>(a, w, bias, nullptr, nullptr, T, N, K, r);
   return hipGetLastError();
 }
 

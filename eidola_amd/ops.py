@@ -153,6 +153,47 @@ def rope_kv_write(geom, qkv, positions, cos_sin, k_cache, v_cache, slot_mapping,
     return q_out
 
 
+def qkv_rope_kv_write(geom, hidden, weight, bias, positions, cos_sin, k_cache, v_cache,
+                      slot_mapping, k_scale=None, v_scale=None, q_out=None):
+    """QKV projection + rope_kv_write in one launch (at most 64 tokens): hidden [T, K] bf16,
+    weight [(Hq + 2 Hkv) * D, K] bf16, bias [(Hq + 2 Hkv) * D] bf16 or None; the rest as
+    rope_kv_write.  Returns q_out [T, Hq, D] bf16; bit-identical to o_proj + rope_kv_write."""
+    _require(hidden, "hidden", torch.bfloat16, 2)
+    _require(weight, "weight", torch.bfloat16, 2)
+    _require(positions, "positions", torch.int32, 1)
+    _require(cos_sin, "cos_sin", torch.float32, 2)
+    k_cache = _cache_view(k_cache, geom, "k_cache")
+    v_cache = _cache_view(v_cache, geom, "v_cache")
+    _require(slot_mapping, "slot_mapping", torch.int64, 1)
+    T, K = hidden.shape
+    N = (geom.num_q_heads + 2 * geom.num_kv_heads) * geom.head_dim
+    if tuple(weight.shape) != (N, K):
+        raise ValueError(f"weight must be [{N}, {K}]")
+    if bias is not None:
+        _require(bias, "bias", torch.bfloat16, 1)
+        if bias.shape[0] != N:
+            raise ValueError(f"bias must be [{N}]")
+    if positions.shape[0] != T or slot_mapping.shape[0] != T:
+        raise ValueError("positions and slot_mapping must have one entry per token")
+    if cos_sin.shape[1] != geom.head_dim:
+        raise ValueError("cos_sin must be [max_pos, head_dim]")
+    if geom.kv_dtype == KV_FP8_E4M3:
+        _require(k_scale, "k_scale", torch.float32, 1)
+        _require(v_scale, "v_scale", torch.float32, 1)
+    if q_out is None:
+        q_out = torch.empty((T, geom.num_q_heads, geom.head_dim), dtype=torch.bfloat16,
+                            device=hidden.device)
+    else:
+        _require(q_out, "q_out", torch.bfloat16, 3)
+    desc = make_desc(geom, num_seqs=1, num_q_tokens=1, max_q_len=1, max_kv_len=1,
+                     max_blocks_per_seq=1, num_blocks=k_cache.shape[0])
+    check(load_library().eid_qkv_rope_kv_write(
+        C.byref(desc), _ptr(hidden), _ptr(weight), _ptr(bias), K, _ptr(positions), _ptr(cos_sin),
+        cos_sin.shape[0], _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _ptr(slot_mapping), T,
+        _ptr(k_scale), _ptr(v_scale), _stream()))
+    return q_out
+
+
 def o_proj(attn_out, weight, bias=None, residual=None, out=None):
     """Output projection after attention: attn_out [T, Hq, D] (or [T, K]) bf16, weight [N, K]
     bf16 (out_features x in_features), optional bias [N] and residual [T, N] bf16; returns

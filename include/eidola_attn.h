@@ -229,6 +229,25 @@ int32_t eid_o_proj(const void *attn_out, const void *weight, const void *bias,
                    const void *residual, void *out, int32_t num_tokens, int32_t out_features,
                    int32_t in_features, void *hip_stream);
 
+/*
+ * QKV projection and eid_rope_kv_write in ONE launch, for decode-sized batches
+ * (num_tokens <= 64; EID_ERR_UNSUPPORTED beyond: use eid_o_proj, then eid_rope_kv_write):
+ *   qkv = hidden @ weight^T + bias        hidden [num_tokens, in_features] bf16,
+ *                                         weight [(Hq + 2 Hkv) * 64, in_features] bf16,
+ *                                         bias   [(Hq + 2 Hkv) * 64] bf16 or NULL
+ * followed by exactly what eid_rope_kv_write does with that qkv (rotation of the q and k
+ * heads by positions[t], q rows to q_out, k and v rows into their cache slots), with the
+ * same arithmetic on the same bf16-rounded projection outputs: q_out and the caches come
+ * out bit-identical to the two calls, and the [num_tokens, (Hq + 2 Hkv) * 64] intermediate
+ * is never written.  in_features % 64 == 0.  Other arguments as eid_rope_kv_write.
+ * Reference counterpart: none.
+ */
+int32_t eid_qkv_rope_kv_write(const eid_attn_desc *desc, const void *hidden, const void *weight,
+                              const void *bias, int32_t in_features, const int32_t *positions,
+                              const float *cos_sin, int32_t max_pos, void *q_out, void *k_cache,
+                              void *v_cache, const int64_t *slot_mapping, int32_t num_tokens,
+                              const float *k_scale, const float *v_scale, void *hip_stream);
+
 /* Bytes of workspace eid_attn_decode / eid_attn_varlen / eid_lse_merge need for desc.
  * Returns 0 for an invalid desc. */
 size_t eid_workspace_bytes(const eid_attn_desc *desc);

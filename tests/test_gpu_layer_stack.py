@@ -97,11 +97,16 @@ def test_two_layers_of_attention_blocks_against_the_oracle_chain(G):
                                 seq_lens_host=b.seq_lens))
         slots.append(G.dev(b.slot_mapping))
 
-    def step(stream=None):
+    def step(stream=None, fused_qkv=False):
         hidden.copy_(hidden0_d)
         for l, L in enumerate(layers):
-            ea.o_proj(hidden, dev["wqkv"][l], dev["bqkv"][l], out=qkv_d)
-            ea.rope_kv_write(L["g"], qkv_d, pos_d, tab_d, L["kc_d"], L["vc_d"], slots[l], q_out=q_d)
+            if fused_qkv:   # projection, rotation and KV write in one launch: same bits
+                ea.qkv_rope_kv_write(L["g"], hidden, dev["wqkv"][l], dev["bqkv"][l], pos_d, tab_d,
+                                     L["kc_d"], L["vc_d"], slots[l], q_out=q_d)
+            else:
+                ea.o_proj(hidden, dev["wqkv"][l], dev["bqkv"][l], out=qkv_d)
+                ea.rope_kv_write(L["g"], qkv_d, pos_d, tab_d, L["kc_d"], L["vc_d"], slots[l],
+                                 q_out=q_d)
             calls[l](stream=stream)
             ea.o_proj(calls[l].out, dev["wo"][l], dev["bo"][l], residual=hidden, out=hidden)
 
@@ -117,15 +122,18 @@ def test_two_layers_of_attention_blocks_against_the_oracle_chain(G):
     for L in layers:
         kd = _f32(G.cache_host(L["kc_d"]))
         assert np.abs(kd - _f32(L["kc"])).max() <= 0.15
+    step(fused_qkv=True)
+    torch.cuda.synchronize()
+    assert torch.equal(hidden, eager)
     # the same chain from one HIP graph, twice, with eager work in between
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        step(side.cuda_stream)
+        step(side.cuda_stream, fused_qkv=True)
         side.synchronize()
         gr = torch.cuda.CUDAGraph()
         with torch.cuda.graph(gr, stream=side):
-            step(side.cuda_stream)
+            step(side.cuda_stream, fused_qkv=True)
     torch.cuda.synchronize()
     for _ in range(2):
         hidden.zero_()

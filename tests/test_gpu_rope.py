@@ -8,7 +8,7 @@ import torch
 
 import oracle
 import eidola_amd as ea
-from eidola_amd import KV_BF16, KV_FP8_E4M3, synth
+from eidola_amd import KV_BF16, KV_FP8_E4M3, _lib, synth
 
 from helpers import assert_close
 
@@ -106,3 +106,63 @@ def test_front_of_a_step_then_attention(G):
     torch.cuda.synchronize()
     assert np.array_equal(G.bits_host(q_d), q_ref)
     assert_close(G.bits_host(out), ref, "rope + write + decode")
+
+
+# ---------------------------------------------------------------- fused with the projection
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+@pytest.mark.parametrize("T,hkv,K,with_bias", [(1, 8, 2880, True), (16, 8, 2880, True),
+                                               (17, 8, 256, False), (40, 8, 2880, True),
+                                               (64, 8, 2880, True), (64, 1, 128, True),
+                                               (33, 2, 640, False)])
+def test_projection_rotation_and_write_in_one_launch(G, kv_dtype, T, hkv, K, with_bias):
+    """eid_qkv_rope_kv_write against eid_o_proj followed by eid_rope_kv_write on the same
+    inputs: q_out and both caches bit for bit (skipped slots and poison included), and the
+    two-launch path is itself bit-exact against the oracle's rotation of its projection."""
+    nb, max_pos = 24, 3000
+    g = ea.AttnGeometry(num_q_heads=8 * hkv, num_kv_heads=hkv, kv_dtype=kv_dtype)
+    N = 10 * hkv * D
+    rng = np.random.default_rng(T + K)
+    hidden = G.bf16_dev(synth.normal_bf16((T, K), 70 + T, synth.TID_Q))
+    w_bits = synth.f32_to_bf16_bits((synth.bf16_bits_to_f32(
+        synth.normal_bf16((N, K), 71 + T, synth.TID_K)) * (1.5 / np.sqrt(K))).astype(np.float32))
+    weight = G.bf16_dev(w_bits)
+    bias = G.bf16_dev(synth.normal_bf16((N,), 72 + T, synth.TID_V)) if with_bias else None
+    pos = rng.integers(0, max_pos, size=T).astype(np.int32)
+    pos[0] = max_pos + 5                                 # clamped into the table
+    slots = rng.permutation(nb * 16)[:T].astype(np.int64)
+    slots[2::5] = -1
+    table = G.dev(ea.yarn_cos_sin(max_pos))
+    if kv_dtype == KV_FP8_E4M3:
+        fill, dt = 0x5A, np.uint8
+        ks = G.dev(np.linspace(0.008, 0.02, hkv).astype(np.float32))
+        vs = G.dev(np.linspace(0.02, 0.008, hkv).astype(np.float32))
+    else:
+        fill, dt, ks, vs = 0xABCD, np.uint16, None, None
+    caches = [G.cache_dev(np.full((nb, 16, hkv, D), fill, dt)) for _ in range(4)]
+    qkv = ea.o_proj(hidden, weight, bias)
+    q_two = ea.rope_kv_write(g, qkv, G.dev(pos), table, caches[0], caches[1], G.dev(slots), ks, vs)
+    q_one = ea.qkv_rope_kv_write(g, hidden, weight, bias, G.dev(pos), table, caches[2], caches[3],
+                                 G.dev(slots), ks, vs)
+    torch.cuda.synchronize()
+    assert torch.equal(q_one, q_two)
+    assert torch.equal(caches[2], caches[0]) and torch.equal(caches[3], caches[1])
+    assert not torch.equal(caches[0], G.cache_dev(np.full((nb, 16, hkv, D), fill, dt)))
+
+
+def test_fused_projection_argument_errors(G):
+    g = ea.AttnGeometry()
+    hidden = torch.zeros((65, 128), dtype=torch.bfloat16, device=G.DEV)
+    weight = torch.zeros((5120, 128), dtype=torch.bfloat16, device=G.DEV)
+    kc = torch.zeros((4, 16, 8, 64), dtype=torch.bfloat16, device=G.DEV)
+    pos = torch.zeros(65, dtype=torch.int32, device=G.DEV)
+    slots = torch.zeros(65, dtype=torch.int64, device=G.DEV)
+    table = G.dev(ea.yarn_cos_sin(16))
+    with pytest.raises(ea.EidError) as e:                # more than 64 tokens
+        ea.qkv_rope_kv_write(g, hidden, weight, None, pos, table, kc, kc.clone(), slots)
+    assert e.value.status == _lib.EID_ERR_UNSUPPORTED
+    with pytest.raises(ea.EidError) as e:                # in_features not a multiple of 64
+        ea.qkv_rope_kv_write(g, hidden[:4, :96].contiguous(), weight[:, :96].contiguous(), None,
+                             pos[:4], table, kc, kc.clone(), slots[:4])
+    assert e.value.status == _lib.EID_ERR_INVALID_ARG
+    q = ea.qkv_rope_kv_write(g, hidden[:0], weight, None, pos[:0], table, kc, kc.clone(), slots[:0])
+    assert q.shape[0] == 0                               # empty batch: nothing launched
