@@ -173,6 +173,11 @@ __device__ __forceinline__ u32x4 quantize16_fp8(const u32x4 lo, const u32x4 hi, 
 // kv_write_kernel would have used, so the step needs no separate write launch.  Key ranges
 // of different partitions are disjoint and every wave owns one KV head: exactly one lane
 // group writes each (sequence, head) row, and nobody else reads it in this launch.
+// A page id as the kernels use it: clamped into the pool (scalar, one instruction).
+__device__ __forceinline__ int clamp_page(const int id, const int last_block) {
+  return (int)min((unsigned)id, (unsigned)last_block);
+}
+
 // Page ids of a work item's first chunk, when the launch carries them (else have == 0).
 struct FirstPages {
   int have = 0;
@@ -233,8 +238,10 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         vraw[b][e] = u32x4{0, 0, 0, 0};
       }
       if (b < nbi) {
-        const uint8_t *kp = p.k_cache + (size_t)blk[b] * page_bytes + lane_off;
-        const uint8_t *vp = p.v_cache + (size_t)blk[b] * page_bytes + lane_off;
+        // (clamped here, at its use: at the load it would make the wave wait for the id)
+        const size_t page_off = (size_t)clamp_page(blk[b], p.last_block) * page_bytes + lane_off;
+        const uint8_t *kp = p.k_cache + page_off;
+        const uint8_t *vp = p.v_cache + page_off;
 #pragma unroll
         for (int e = 0; e < kElt; ++e) {
           kraw[b][e] = ldg128(kp + 16 * e);
@@ -251,7 +258,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
       size_t dst = lane_off;
 #pragma unroll
       for (int b = 0; b < kPages; ++b)
-        if (b == b_new) dst += (size_t)blk[b] * page_bytes;
+        if (b == b_new) dst += (size_t)clamp_page(blk[b], p.last_block) * page_bytes;
 #pragma unroll
       for (int kv = 0; kv < 2; ++kv) {
         const uint16_t *from = (kv ? p.v_new : p.k_new) + src;
@@ -506,7 +513,8 @@ struct SeqView {
 __device__ __forceinline__ SeqView view_seq(const AttnParams &p, const int s) {
   SeqView v{0, 0, 0, 0};
   if (s < p.num_seqs) {
-    v.seq_len = p.seq_lens[s];
+    // (a length beyond the table row is a caller error; clamped, it cannot index past the row)
+    v.seq_len = min(p.seq_lens[s], p.max_blocks_per_seq * kBlock);
     v.row0 = s;
     v.qlen = 1;
     if (p.cu_seqlens_q) {
@@ -755,7 +763,7 @@ __device__ __forceinline__ WorkItem table_item(const AttnParams &p, const ItemTa
   WorkItem it;
   it.seq = (int)(e & 0xffffu);
   it.part = (int)((e >> 16) & 0xffffu);
-  it.seq_len = (int)(e >> 32);
+  it.seq_len = min((int)(e >> 32), p.max_blocks_per_seq * kBlock);
   it.row0 = it.seq;
   it.qlen = 1;
   it.nparts = num_partitions(p, it.seq_len - kv_begin(it.seq_len, 1, p.window), P);
@@ -959,7 +967,7 @@ __device__ __forceinline__ bool find_prefill_item(const AttnParams &p, const int
     const int s = s0 + lane;
     int n = 0, r0 = 0, ql = 0, L = 0;
     if (s < p.num_seqs) {
-      L = p.seq_lens[s];
+      L = min(p.seq_lens[s], p.max_blocks_per_seq * kBlock);
       r0 = p.cu_seqlens_q[s];
       ql = p.cu_seqlens_q[s + 1] - r0;
       if (ql >= p.qlen_lo && ql <= p.qlen_hi && L >= ql) n = (ql + kPfTok - 1) / kPfTok;
@@ -1082,7 +1090,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   auto fetch = [&](const int tc) {  // global -> registers for chunk starting at token tc
     int ids[4];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) ids[b] = bt[min(tc / kBlock + b, nblk_total - 1)];
+    for (int b = 0; b < 4; ++b)
+      ids[b] = clamp_page(bt[min(tc / kBlock + b, nblk_total - 1)], p.last_block);
     const int blk = ld_page == 0 ? ids[0] : ld_page == 1 ? ids[1] : ld_page == 2 ? ids[2] : ids[3];
 #pragma unroll
     for (int e = 0; e < kElt; ++e) {
@@ -1247,7 +1256,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
     qlen = p.cu_seqlens_q[s + 1] - row0;
   }
   if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
-  const int L = p.seq_lens[s];
+  const int L = min(p.seq_lens[s], p.max_blocks_per_seq * kBlock);  // as the split-KV kernels read it
   if (L < qlen) return;
   // run-time partition: recorded by the split-KV launch of this class; else the caller's
   const int P = p.plan_slot ? p.plan_slot[0] : p.partition;

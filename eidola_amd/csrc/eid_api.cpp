@@ -241,6 +241,7 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   p.num_q_heads = d->num_q_heads;
   p.num_kv_heads = d->num_kv_heads;
   p.max_blocks_per_seq = d->max_blocks_per_seq;
+  p.last_block = (int32_t)std::min<int64_t>(d->num_blocks - 1, 0x7fffffff);
   p.window = d->window;
   p.partition = pl.partition;
   p.dynamic_partition = pl.dynamic ? 1 : 0;
@@ -314,7 +315,8 @@ ClassSpans class_spans(const eid_attn_desc *d, const int32_t *seq_lens, const in
   c.seq.reserve(d->num_seqs);
   c.len.reserve(d->num_seqs);
   for (int32_t s = 0; s < d->num_seqs; ++s) {
-    const int32_t L = seq_lens[s], qlen = cu ? cu[s + 1] - cu[s] : 1;
+    const int32_t L = std::min<int64_t>(seq_lens[s], (int64_t)d->max_blocks_per_seq * eid::kBlock);
+    const int32_t qlen = cu ? cu[s + 1] - cu[s] : 1;
     if (qlen < qlen_lo || qlen > qlen_hi || qlen > ws_rows || L < qlen) continue;
     const int32_t span = L - eid::kv_begin(L, qlen, d->window);
     if (span <= 0) continue;

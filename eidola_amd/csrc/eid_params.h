@@ -38,6 +38,9 @@ struct AttnParams {
   int32_t target_items_lo; // workgroups at one per CU (<= target_items)
   long long sum_kv_len;  // host's upper bound on the sum of seq_lens, 0 = unknown
   int32_t num_seqs, num_q_heads, num_kv_heads, max_blocks_per_seq;
+  int32_t last_block;    // num_blocks - 1: every page id is clamped to [0, last_block] before
+                         // use, so a stale or wrong table entry reads a wrong page, never
+                         // memory outside the caches
   int32_t window, partition, nparts_max, ws_rows;
   int32_t qlen_lo, qlen_hi;  // this launch serves sequences with qlen_lo <= q_len <= qlen_hi
   int32_t dynamic_partition; // 1: kernels derive the partition from the batch (>= partition)

@@ -312,6 +312,24 @@ def test_partition_count_at_its_maximum(G):
     assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "64 partitions")
 
 
+@pytest.mark.parametrize("host_lens", [False, True])
+def test_table_entries_beyond_a_sequence_do_not_matter(G, host_lens):
+    """Entries of a block-table row past the sequence's last page are undefined: whatever
+    they hold (here negative and huge ids), the output is the same bit for bit, through the
+    short-span, split-KV and prefill kernels."""
+    b = make_batch([700, 45, 3000, 1, 130, 2000], [1, 1, 5, 1, 2, 40])
+    q, k, v, sinks = logical_tensors(b)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    clean = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=host_lens)
+    junk = np.array([-1, 0x7fffffff, -(2 ** 31), 123456789], np.int32)
+    for s_, L in enumerate(b.seq_lens):
+        n = (int(L) + 15) // 16
+        tail = b.block_table[s_, n:]
+        tail[:] = junk[np.arange(len(tail)) % 4]
+    dirty = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=host_lens)
+    assert np.array_equal(clean, dirty)
+
+
 def test_errors_surface_as_status_codes_on_the_gpu_box(G):
     b = make_batch([100], [1])
     q, k, v, sinks = logical_tensors(b)
