@@ -28,7 +28,9 @@
  *   k_new, v_new      [num_tokens,   num_kv_heads, 64] bf16
  *   k_cache, v_cache  [num_blocks, 16, num_kv_heads, 64]  bf16 or fp8-e4m3fn
  *   slot_mapping      [num_tokens] int64   slot = block*16 + offset, -1 = skip
- *   block_table       [num_seqs, max_blocks_per_seq] int32
+ *   block_table       [num_seqs, max_blocks_per_seq] int32   entries past a sequence's last page
+ *                     are never needed; ids are clamped to [0, num_blocks) and lengths to the
+ *                     row before use, so junk there cannot make a kernel leave the caches
  *   cu_seqlens_q      [num_seqs + 1] int32
  *   seq_lens          [num_seqs] int32   KV length AFTER this step's append
  *   sinks             [num_q_heads] fp32 (NULL = no sink, i.e. -inf)
