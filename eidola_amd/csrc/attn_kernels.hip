@@ -1511,8 +1511,8 @@ static int waves_for(int Hkv) { return Hkv >= 8 ? 8 : Hkv; }
 // Workgroups of the split-KV instantiation (ntiles, fp8, Hkv) the device holds at once.
 int splitkv_fill(int ntiles, bool fp8, int Hkv) {
   const int waves = waves_for(Hkv);
-  if (fp8) return ntiles == 1 ? fill_t<1, true>(waves) : fill_t<3, true>(waves);
-  return ntiles == 1 ? fill_t<1, false>(waves) : fill_t<3, false>(waves);
+  if (fp8) return ntiles == 1 ? fill_t<1, true>(waves) : ntiles == 3 ? fill_t<3, true>(waves) : fill_t<4, true>(waves);
+  return ntiles == 1 ? fill_t<1, false>(waves) : ntiles == 3 ? fill_t<3, false>(waves) : fill_t<4, false>(waves);
 }
 
 // Upper bound on the number of work items of a launch, from what the host knows.  Items
@@ -1614,10 +1614,12 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
   dim3 grid((unsigned)items, p.num_kv_heads);
   if (fp8) {
     if (ntiles == 1) shortspan_kernel<1, true><<<grid, kShortWaves * 64, 0, st>>>(p);
-    else shortspan_kernel<3, true><<<grid, kShortWaves * 64, 0, st>>>(p);
+    else if (ntiles == 3) shortspan_kernel<3, true><<<grid, kShortWaves * 64, 0, st>>>(p);
+    else shortspan_kernel<4, true><<<grid, kShortWaves * 64, 0, st>>>(p);
   } else {
     if (ntiles == 1) shortspan_kernel<1, false><<<grid, kShortWaves * 64, 0, st>>>(p);
-    else shortspan_kernel<3, false><<<grid, kShortWaves * 64, 0, st>>>(p);
+    else if (ntiles == 3) shortspan_kernel<3, false><<<grid, kShortWaves * 64, 0, st>>>(p);
+    else shortspan_kernel<4, false><<<grid, kShortWaves * 64, 0, st>>>(p);
   }
   return hipGetLastError();
 }
@@ -1626,12 +1628,14 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
 // once; beyond that the split-KV kernel's one workgroup per item with longer partitions makes
 // fewer, better filled rounds.
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
-  static const int fill[2][2] = {
+  static const int fill[3][2] = {
       {device_fill(shortspan_kernel<1, false>, kShortWaves * 64),
        device_fill(shortspan_kernel<1, true>, kShortWaves * 64)},
       {device_fill(shortspan_kernel<3, false>, kShortWaves * 64),
-       device_fill(shortspan_kernel<3, true>, kShortWaves * 64)}};
-  return num_items * Hkv <= fill[ntiles == 1 ? 0 : 1][fp8 ? 1 : 0];
+       device_fill(shortspan_kernel<3, true>, kShortWaves * 64)},
+      {device_fill(shortspan_kernel<4, false>, kShortWaves * 64),
+       device_fill(shortspan_kernel<4, true>, kShortWaves * 64)}};
+  return num_items * Hkv <= fill[ntiles == 1 ? 0 : ntiles == 3 ? 1 : 2][fp8 ? 1 : 0];
 }
 
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
@@ -1659,10 +1663,12 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   }
   if (fp8) {
     if (ntiles == 1) return launch_splitkv_t<1, true>(p, st);
-    return launch_splitkv_t<3, true>(p, st);
+    if (ntiles == 3) return launch_splitkv_t<3, true>(p, st);
+    return launch_splitkv_t<4, true>(p, st);
   }
   if (ntiles == 1) return launch_splitkv_t<1, false>(p, st);
-  return launch_splitkv_t<3, false>(p, st);
+  if (ntiles == 3) return launch_splitkv_t<3, false>(p, st);
+  return launch_splitkv_t<4, false>(p, st);
 }
 
 // Upper bound on the prefill kernel's 32-token query tiles: every sequence rounds up by at most

@@ -124,10 +124,20 @@ struct Plan {
   size_t pf_ml_bytes, pf_acc_bytes;
 };
 
+// Longest query a split-KV (verify) sequence may have in this call: 6 rows x 8 heads = three
+// 16-row tiles; 8 rows = four tiles when no sequence of the batch is longer than that (the
+// prefill kernel's 32-token tile would be three quarters empty for such a sequence, and the
+// batch is bandwidth-bound).
+int32_t short_q_max(const eid_attn_desc *d) {
+  return d->max_q_len > eid::kShortQMax && d->max_q_len <= eid::kShortQMaxWide ? eid::kShortQMaxWide
+                                                                                : eid::kShortQMax;
+}
+int verify_tiles(const eid_attn_desc *d) { return short_q_max(d) == eid::kShortQMaxWide ? 4 : 3; }
+
 // Longest key span a split-KV sequence can have (from its first visible page to its end).
 int32_t max_span(const eid_attn_desc *d) {
   if (d->window > 0) {
-    const int64_t w = (int64_t)d->window + eid::kShortQMax + eid::kBlock - 1;
+    const int64_t w = (int64_t)d->window + short_q_max(d) + eid::kBlock - 1;
     return (int32_t)(w < d->max_kv_len ? w : d->max_kv_len);
   }
   return d->max_kv_len;
@@ -154,7 +164,7 @@ Plan make_plan(const eid_attn_desc *d) {
   if (pl.dynamic) {
     const long long items = eid::shortspan_items(
         d->num_seqs, (span + eid::kShortSpanMax - 1) / eid::kShortSpanMax, d->sum_kv_len, d->window);
-    if (eid::shortspan_applies(d->max_q_len <= 2 ? 1 : 3, d->kv_dtype == EID_KV_FP8_E4M3, items,
+    if (eid::shortspan_applies(d->max_q_len <= 2 ? 1 : verify_tiles(d), d->kv_dtype == EID_KV_FP8_E4M3, items,
                                d->num_kv_heads)) {
       P = eid::kShortSpanMax;
       pl.dynamic = false;
@@ -162,7 +172,7 @@ Plan make_plan(const eid_attn_desc *d) {
   }
   pl.partition = P;
   pl.nparts_max = (span + P - 1) / P;
-  pl.ws_rows = d->max_q_len < eid::kShortQMax ? d->max_q_len : eid::kShortQMax;
+  pl.ws_rows = std::min(d->max_q_len, short_q_max(d));
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
   pl.ml_bytes = (cells * 2 * sizeof(float) + 255) / 256 * 256;
   pl.acc_bytes = (cells * eid::kHeadDim * sizeof(_Float16) + 255) / 256 * 256;
@@ -171,7 +181,7 @@ Plan make_plan(const eid_attn_desc *d) {
   // of at least 512 keys that run side by side and are merged afterwards.
   pl.pf_splits = 1;
   pl.pf_ml_bytes = pl.pf_acc_bytes = 0;
-  if (d->max_q_len > eid::kShortQMax) {
+  if (d->max_q_len > short_q_max(d)) {
     const long long wgs = eid::prefill_tiles_bound(d->num_q_tokens, d->num_seqs) * d->num_kv_heads;
     // (aim: the split that comes nearest to one fill; two fills were measured too: better for
     // one 512-token chunk behind 60k tokens, worse for a 2,048-token chunk without a prior)
@@ -616,8 +626,9 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   // has max_q_len query rows (num_q_tokens says so) the host knows the one class that is
   // populated and launches nothing for the others.
   const bool uniform = (int64_t)desc->num_seqs * desc->max_q_len == desc->num_q_tokens;
-  const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= eid::kShortQMax;
-  const bool only_prefill = uniform && desc->max_q_len > eid::kShortQMax;
+  const int32_t qmax = short_q_max(desc);
+  const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= qmax;
+  const bool only_prefill = uniform && desc->max_q_len > qmax;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   auto launch_split = [&](const ClassPlan &cp, const int ntiles, int32_t *slot) {
     if (!cp.short_span) return eid::launch_splitkv(p, ntiles, fp8, slot, st);
@@ -628,7 +639,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   // Mixed batch: the MFMA-bound prefill launch and the HBM-bound split-KV launches use
   // different halves of the machine, so they run side by side: prefill on the thread's
   // helper stream, forked from and joined back into the caller's stream.
-  const bool has_prefill = desc->max_q_len > eid::kShortQMax;
+  const bool has_prefill = desc->max_q_len > qmax;
   static const bool serial = getenv("EID_SERIAL_CLASSES") != nullptr;  // for A/B measurements
   Helper *hs = (has_prefill && !only_prefill && !serial) ? helper_stream() : nullptr;
   p.share_cus = hs ? 1 : 0;
@@ -650,7 +661,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   }
   if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
     eid::AttnParams pp = p;
-    pp.qlen_lo = eid::kShortQMax + 1;
+    pp.qlen_lo = qmax + 1;
     pp.qlen_hi = 0x7fffffff;
     e = eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream);
     if (e == hipSuccess) e = hipEventRecord(hs->join, hs->stream);
@@ -665,9 +676,10 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     if (e != hipSuccess) return hip_fail(e, "merge launch");
   }
   if (desc->max_q_len > 2 && !only_prefill) {  // q_len 3..6: three tiles
-    const ClassPlan cp3 = plan_class(desc, args, pl, p, 3, 3, eid::kShortQMax, false);
+    const int vt = verify_tiles(desc);
+    const ClassPlan cp3 = plan_class(desc, args, pl, p, vt, 3, qmax, false);
     if (!cp3.skip) {
-      e = launch_split(cp3, 3, plan_slots + 2);
+      e = launch_split(cp3, vt, plan_slots + 2);
       if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
       if (cp3.merge) {
         e = eid::launch_merge(p, st);
@@ -679,7 +691,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     e = hipStreamWaitEvent(st, hs->join, 0);
     if (e != hipSuccess) return hip_fail(e, "join of the helper stream");
   } else if (has_prefill) {  // long chunks: MFMA prefill kernel
-    p.qlen_lo = eid::kShortQMax + 1;
+    p.qlen_lo = qmax + 1;
     p.qlen_hi = 0x7fffffff;
     e = eid::launch_prefill(p, desc->num_q_tokens, fp8, st);
     if (e != hipSuccess) return hip_fail(e, "prefill launch");
@@ -693,11 +705,11 @@ int32_t eid_lse_merge(const eid_attn_desc *desc, const eid_attn_args *args, void
   if (int32_t rc = check_attn_args(desc, args, false, false)) return rc;
   const Plan pl = make_plan(desc);
   eid::AttnParams p = make_params(desc, args, pl);
-  // One class of sequences per call, as the split-KV launches are: q_len <= 2, else 3..6.
+  // One class of sequences per call, as the split-KV launches are: q_len <= 2, else 3..6 (3..8).
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   p.qlen_lo = desc->max_q_len <= 2 ? 1 : 3;
-  p.qlen_hi = desc->max_q_len <= 2 ? 2 : eid::kShortQMax;
-  p.target_items = eid::splitkv_fill(desc->max_q_len <= 2 ? 1 : 3, fp8, desc->num_kv_heads);
+  p.qlen_hi = desc->max_q_len <= 2 ? 2 : short_q_max(desc);
+  p.target_items = eid::splitkv_fill(desc->max_q_len <= 2 ? 1 : verify_tiles(desc), fp8, desc->num_kv_heads);
   // With a run-time partition the merge takes the size the split-KV launch of this class
   // recorded in the workspace header (the attention entry points do the same).
   if (pl.dynamic)

@@ -10,6 +10,7 @@ constexpr int kHeadDim = 64;
 constexpr int kBlock = 16;        // tokens per KV page
 constexpr int kGroup = 8;         // query heads per KV head
 constexpr int kShortQMax = 6;     // q_len handled by the split-KV kernel (6*8 = 48 rows = 3 tiles)
+constexpr int kShortQMaxWide = 8; // ... when no sequence of the batch has more than 8 rows: four tiles
 constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the split-KV loop
 constexpr int kDynPartitionMin = 256;   // lower bound (and workspace sizing) of the dynamic partition
 constexpr int kDynPartitionCap = 2048;  // a workgroup streams serially: keep its share bounded

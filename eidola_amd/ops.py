@@ -473,12 +473,13 @@ def workspace_layout(desc):
     o   float16 [num_seqs*ws_rows, nparts_max, Hq, 64] (partition output sum e^(s-m) v / l) at
     the byte offsets returned."""
     P = partition_size(desc)
+    qmax = 8 if 6 < desc.max_q_len <= 8 else 6   # rows of a split-KV sequence (see short_q_max)
     if desc.window > 0:
-        span = min(desc.max_kv_len, desc.window + 6 + desc.block_size - 1)
+        span = min(desc.max_kv_len, desc.window + qmax + desc.block_size - 1)
     else:
         span = desc.max_kv_len
     nparts = (span + P - 1) // P
-    ws_rows = min(desc.max_q_len, 6)
+    ws_rows = min(desc.max_q_len, qmax)
     cells = desc.num_seqs * ws_rows * desc.num_q_heads * nparts
     ml_bytes = (cells * 8 + 255) // 256 * 256
     return P, nparts, ws_rows, 256, 256 + ml_bytes

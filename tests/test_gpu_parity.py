@@ -157,6 +157,48 @@ def test_verify_five_rows(G, window, partition):
     assert np.allclose(lse, ref_lse, atol=2e-3)
 
 
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+@pytest.mark.parametrize("window,partition,seq_lens,q_lens,host_lens", [
+    (0, 0, [3000, 700, 5000, 90, 8], [8, 7, 3, 1, 8], False),        # small batch: 512-key partitions
+    (0, 256, [3000, 700, 5000, 90], [8, 7, 5, 2], False),            # the caller's partition
+    (128, 0, [3000, 700, 150, 9], [8, 7, 8, 7], True),               # windowed: short spans
+    (0, 0, [1200 + 37 * i for i in range(40)], [7, 8] * 20, True),   # split-KV kernel, host plan
+    (0, 0, [900 + 53 * i for i in range(70)], [8] * 70, False),      # one class only, run-time rule
+])
+def test_seven_and_eight_query_rows_take_four_tiles(G, kv_dtype, window, partition, seq_lens,
+                                                    q_lens, host_lens):
+    """When no sequence of the batch has more than 8 query rows, sequences of 7 and 8 rows
+    stay in the split-KV class (64 rows = four 16-row tiles per KV head) instead of going to
+    the prefill kernel.  Against the oracle, with lse, for every kernel that serves the class."""
+    b = make_batch(seq_lens, q_lens, window=window, partition=partition, kv_dtype=kv_dtype)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, host_lens=host_lens,
+                          hint=host_lens)
+    assert_close(out, ref, f"q_len 7..8 w={window} P={partition}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
+def test_eighth_row_agrees_with_the_prefill_kernel(G):
+    """The same 8-row sequences once in a batch whose longest query is 8 rows (split-KV class,
+    four tiles) and once next to a 9-row sequence (then they are prefill rows): two kernels,
+    one result within rounding."""
+    L, ql = [2500, 900, 4000], [8, 7, 8]
+    b8 = make_batch(L, ql, seed=3)
+    b9 = make_batch(L + [600], ql + [9], seed=3)
+    q, k, v, sinks = logical_tensors(b9)
+    kc_d, vc_d = G.gpu_caches(b9, k, v)
+    o9 = G.run_attn(b9, q, kc_d, vc_d, sinks)
+    b8.block_table[:, :] = b9.block_table[:3, :b8.block_table.shape[1]]
+    o8 = G.run_attn(b8, q[:23], kc_d, vc_d, sinks)
+    a = synth.bf16_bits_to_f32(o8).astype(np.float64)
+    c = synth.bf16_bits_to_f32(o9[:23]).astype(np.float64)
+    assert np.abs(a - c).max() <= 4e-3
+
+
 def test_verify_row_equals_decode_row(G):
     L = 777
     b5 = make_batch([L], [5], partition=256)
