@@ -668,7 +668,8 @@ __global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *p
 template <int NT, bool FP8>
 __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem &it, const int P,
                                              const int kvh, const int wave, uint8_t *lds,
-                                             const FirstPages &first = FirstPages{}) {
+                                             const FirstPages &first = FirstPages{},
+                                             const int tq0 = 0) {
   const int s = it.seq, part = it.part, nparts = it.nparts;
   const int row0 = it.row0, qlen = it.qlen, L = it.seq_len;
   const int kb = kv_begin(L, qlen, p.window);
@@ -679,7 +680,8 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
 
   Frag8 qf[NT][2];
   RowInfo ri;
-  load_q<NT>(p, row0, qlen, 0, kvh, pos0, qf, ri);
+  if (tq0 >= qlen) return;  // (a row group past the sequence's rows)
+  load_q<NT>(p, row0, qlen, tq0, kvh, pos0, qf, ri);
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
@@ -691,7 +693,7 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
   }
   attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
                   lacc, acc, first);
-  finish<NT, FP8>(p, s, kvh, row0, qlen, 0, nparts == 1, part, m, lacc, acc);
+  finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, nparts == 1, part, m, lacc, acc);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -700,11 +702,17 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
 // blockIdx.y*WAVES + w, so the workgroup as a whole streams whole 16-token pages (all KV
 // heads) of its partition.
 // ---------------------------------------------------------------------------------------
-template <int NT, bool FP8, int WAVES>
+//
+// RS > 1 (q_len beyond one wave's rows): RS waves share a KV head, wave w taking the query
+// tokens [8 (w % RS), +8) of the sequence; the workgroup then covers WAVES / RS KV heads and
+// the grid's y dimension grows by RS.  Both waves load the head's K/V (the second from cache).
+template <int NT, bool FP8, int WAVES, int RS = 1>
 __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(const AttnParams p) {
+  static_assert(RS == 1 || (NT == 4 && WAVES % RS == 0), "row groups are 8 tokens = four tiles");
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kvh = blockIdx.y * WAVES + wave;
+  const int kvh = blockIdx.y * (WAVES / RS) + wave / RS;
+  const int tq0 = (wave % RS) * (NT * 16 / kGroup);
   if (p.nparts_max == 1) {
     // Every sequence is a single item (short spans: sliding-window layers, short contexts):
     // workgroup w serves sequence w, found with scalar loads alone; sequences of another
@@ -718,7 +726,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
     it.row0 = v.row0;
     it.qlen = v.qlen;
     it.seq_len = v.seq_len;
-    splitkv_item<NT, FP8>(p, it, 1 << 30, kvh, wave, lds);
+    splitkv_item<NT, FP8>(p, it, 1 << 30, kvh, wave, lds, FirstPages{}, tq0);
     return;
   }
   if (planned_out(p, blockIdx.x)) return;
@@ -752,7 +760,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   it.seq_len = __builtin_amdgcn_readfirstlane(item_lds[6]);
   // the merge launch that follows reads the partition from here instead of re-deriving it
   if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
-  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds);
+  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds, FirstPages{}, tq0);
 }
 
 // The same for a decode launch whose items the host has listed (q_len 1, row = sequence):
@@ -1490,9 +1498,9 @@ int device_cus() {
   return cus;
 }
 
-template <int NT, bool FP8, int WAVES>
+template <int NT, bool FP8, int WAVES, int RS = 1>
 static int fill_of() {
-  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES>, WAVES * 64);
+  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES, RS>, WAVES * 64);
   return fill;
 }
 
@@ -1511,6 +1519,7 @@ static int waves_for(int Hkv) { return Hkv >= 8 ? 8 : Hkv; }
 // Workgroups of the split-KV instantiation (ntiles, fp8, Hkv) the device holds at once.
 int splitkv_fill(int ntiles, bool fp8, int Hkv) {
   const int waves = waves_for(Hkv);
+  if (ntiles == 8) return fp8 ? fill_of<4, true, 8, 2>() : fill_of<4, false, 8, 2>();  // two row groups
   if (fp8) return ntiles == 1 ? fill_t<1, true>(waves) : ntiles == 3 ? fill_t<3, true>(waves) : fill_t<4, true>(waves);
   return ntiles == 1 ? fill_t<1, false>(waves) : ntiles == 3 ? fill_t<3, false>(waves) : fill_t<4, false>(waves);
 }
@@ -1551,9 +1560,9 @@ static long long item_bound(const AttnParams &p) {
   return items;
 }
 
-template <int NT, bool FP8, int WAVES>
+template <int NT, bool FP8, int WAVES, int RS = 1>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
-  dim3 grid((unsigned)item_bound(p), p.num_kv_heads / WAVES);
+  dim3 grid((unsigned)item_bound(p), p.num_kv_heads / (WAVES / RS));
   // With a prefill launch beside it (mixed batch, p.share_cus): one 8-wave workgroup per CU.
   // A second resident workgroup adds little to a kernel that streams from HBM (it only
   // covers the prologues of many short items), while half of the CU's registers left free
@@ -1566,13 +1575,13 @@ static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
-      e = hipFuncSetAttribute((const void *)splitkv_kernel<NT, FP8, WAVES>,
+      e = hipFuncSetAttribute((const void *)splitkv_kernel<NT, FP8, WAVES, RS>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, kPad);
       if (e != hipSuccess) return e;
       if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
     }
   }
-  splitkv_kernel<NT, FP8, WAVES><<<grid, WAVES * 64, kPad, st>>>(p);
+  splitkv_kernel<NT, FP8, WAVES, RS><<<grid, WAVES * 64, kPad, st>>>(p);
   return hipGetLastError();
 }
 
@@ -1628,6 +1637,7 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
 // once; beyond that the split-KV kernel's one workgroup per item with longer partitions makes
 // fewer, better filled rounds.
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
+  if (ntiles == 8) return false;  // two row groups per KV head: split-KV kernel only
   static const int fill[3][2] = {
       {device_fill(shortspan_kernel<1, false>, kShortWaves * 64),
        device_fill(shortspan_kernel<1, true>, kShortWaves * 64)},
@@ -1661,6 +1671,8 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
     if (e != hipSuccess) return e;
     p.plan = plan_slot;
   }
+  if (ntiles == 8)  // 9..16 rows: two waves per KV head (the host checked num_kv_heads % 8 == 0)
+    return fp8 ? launch_splitkv_w<4, true, 8, 2>(p, st) : launch_splitkv_w<4, false, 8, 2>(p, st);
   if (fp8) {
     if (ntiles == 1) return launch_splitkv_t<1, true>(p, st);
     if (ntiles == 3) return launch_splitkv_t<3, true>(p, st);

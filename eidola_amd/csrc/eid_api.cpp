@@ -125,14 +125,26 @@ struct Plan {
 };
 
 // Longest query a split-KV (verify) sequence may have in this call: 6 rows x 8 heads = three
-// 16-row tiles; 8 rows = four tiles when no sequence of the batch is longer than that (the
-// prefill kernel's 32-token tile would be three quarters empty for such a sequence, and the
-// batch is bandwidth-bound).
+// 16-row tiles; 8 rows = four tiles, or 16 rows = two waves of four tiles per KV head, when
+// no sequence of the batch is longer than that (the prefill kernel's 32-token tile would be
+// mostly empty for such sequences, and the batch is bandwidth-bound).
 int32_t short_q_max(const eid_attn_desc *d) {
+  // 9..16 rows: two waves per KV head, 8 rows each, both loading the head's K/V.  That doubles
+  // the traffic through the CU's cache, so it pays only while the prefill kernel's workgroups
+  // (one per sequence and KV head at these lengths) would not fill the device: 8 x 16 rows
+  // behind 32k tokens 310 -> 182 us, 32 x 16 behind 8k 322 -> 194 us, 48 x 16 387 -> 300 us,
+  // but 64 x 16 414 -> 427 us (left to the prefill kernel).
+  if (d->max_q_len > eid::kShortQMaxWide && d->max_q_len <= eid::kShortQMaxRows &&
+      d->num_kv_heads % 8 == 0 && (long long)d->num_seqs * d->num_kv_heads <= eid::kRowsMaxGroups)
+    return eid::kShortQMaxRows;
   return d->max_q_len > eid::kShortQMax && d->max_q_len <= eid::kShortQMaxWide ? eid::kShortQMaxWide
                                                                                 : eid::kShortQMax;
 }
-int verify_tiles(const eid_attn_desc *d) { return short_q_max(d) == eid::kShortQMaxWide ? 4 : 3; }
+// 16-row tiles per KV head of the verify class: 3, 4, or 8 (two waves of four)
+int verify_tiles(const eid_attn_desc *d) {
+  const int32_t q = short_q_max(d);
+  return q == eid::kShortQMaxRows ? 8 : q == eid::kShortQMaxWide ? 4 : 3;
+}
 
 // Longest key span a split-KV sequence can have (from its first visible page to its end).
 int32_t max_span(const eid_attn_desc *d) {

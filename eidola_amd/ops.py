@@ -473,7 +473,11 @@ def workspace_layout(desc):
     o   float16 [num_seqs*ws_rows, nparts_max, Hq, 64] (partition output sum e^(s-m) v / l) at
     the byte offsets returned."""
     P = partition_size(desc)
-    qmax = 8 if 6 < desc.max_q_len <= 8 else 6   # rows of a split-KV sequence (see short_q_max)
+    if (8 < desc.max_q_len <= 16 and desc.num_kv_heads % 8 == 0
+            and desc.num_seqs * desc.num_kv_heads <= 448):
+        qmax = 16   # rows of a split-KV sequence (see short_q_max in eid_api.cpp)
+    else:
+        qmax = 8 if 6 < desc.max_q_len <= 8 else 6
     if desc.window > 0:
         span = min(desc.max_kv_len, desc.window + qmax + desc.block_size - 1)
     else:

@@ -164,12 +164,18 @@ def test_verify_five_rows(G, window, partition):
     (128, 0, [3000, 700, 150, 9], [8, 7, 8, 7], True),               # windowed: short spans
     (0, 0, [1200 + 37 * i for i in range(40)], [7, 8] * 20, True),   # split-KV kernel, host plan
     (0, 0, [900 + 53 * i for i in range(70)], [8] * 70, False),      # one class only, run-time rule
+    (0, 0, [3000, 700, 5000, 90, 16], [16, 9, 3, 1, 16], False),     # 9..16 rows: two waves per KV head
+    (0, 256, [3000, 700, 5000, 90], [12, 16, 5, 2], True),
+    (128, 0, [3000, 700, 150, 13], [16, 10, 8, 13], True),           # ... windowed (one partition each)
+    (0, 0, [1200 + 37 * i for i in range(40)], [16, 11] * 20, True),
+    (0, 0, [900 + 53 * i for i in range(70)], [16] * 70, False),     # too many for that: prefill kernel
 ])
 def test_seven_and_eight_query_rows_take_four_tiles(G, kv_dtype, window, partition, seq_lens,
                                                     q_lens, host_lens):
     """When no sequence of the batch has more than 8 query rows, sequences of 7 and 8 rows
     stay in the split-KV class (64 rows = four 16-row tiles per KV head) instead of going to
-    the prefill kernel.  Against the oracle, with lse, for every kernel that serves the class."""
+    the prefill kernel; up to 16 rows, two waves share a KV head (8 query tokens each).
+    Against the oracle, with lse, for every kernel that serves the class."""
     b = make_batch(seq_lens, q_lens, window=window, partition=partition, kv_dtype=kv_dtype)
     q, k, v, sinks = logical_tensors(b)
     ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
@@ -196,6 +202,23 @@ def test_eighth_row_agrees_with_the_prefill_kernel(G):
     o8 = G.run_attn(b8, q[:23], kc_d, vc_d, sinks)
     a = synth.bf16_bits_to_f32(o8).astype(np.float64)
     c = synth.bf16_bits_to_f32(o9[:23]).astype(np.float64)
+    assert np.abs(a - c).max() <= 4e-3
+
+
+def test_sixteen_rows_agree_with_the_prefill_kernel(G):
+    """9..16-row sequences through the row-split split-KV kernel, and the same sequences
+    next to a 17-row one (prefill kernel): one result within rounding."""
+    L, ql = [2500, 900, 4000, 300], [16, 9, 12, 16]
+    bs = make_batch(L, ql, seed=5)
+    bl = make_batch(L + [600], ql + [17], seed=5)
+    q, k, v, sinks = logical_tensors(bl)
+    kc_d, vc_d = G.gpu_caches(bl, k, v)
+    ol = G.run_attn(bl, q, kc_d, vc_d, sinks)
+    bs.block_table[:, :] = bl.block_table[:4, :bs.block_table.shape[1]]
+    n = sum(ql)
+    os_ = G.run_attn(bs, q[:n], kc_d, vc_d, sinks)
+    a = synth.bf16_bits_to_f32(os_).astype(np.float64)
+    c = synth.bf16_bits_to_f32(ol[:n]).astype(np.float64)
     assert np.abs(a - c).max() <= 4e-3
 
 
