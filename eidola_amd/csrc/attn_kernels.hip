@@ -1520,6 +1520,7 @@ static int waves_for(int Hkv) { return Hkv >= 8 ? 8 : Hkv; }
 int splitkv_fill(int ntiles, bool fp8, int Hkv) {
   const int waves = waves_for(Hkv);
   if (ntiles == 8) return fp8 ? fill_of<4, true, 8, 2>() : fill_of<4, false, 8, 2>();  // two row groups
+  if (ntiles == 16) return fp8 ? fill_of<4, true, 8, 4>() : fill_of<4, false, 8, 4>();  // four
   if (fp8) return ntiles == 1 ? fill_t<1, true>(waves) : ntiles == 3 ? fill_t<3, true>(waves) : fill_t<4, true>(waves);
   return ntiles == 1 ? fill_t<1, false>(waves) : ntiles == 3 ? fill_t<3, false>(waves) : fill_t<4, false>(waves);
 }
@@ -1637,7 +1638,7 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
 // once; beyond that the split-KV kernel's one workgroup per item with longer partitions makes
 // fewer, better filled rounds.
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
-  if (ntiles == 8) return false;  // two row groups per KV head: split-KV kernel only
+  if (ntiles >= 8) return false;  // several row groups per KV head: split-KV kernel only
   static const int fill[3][2] = {
       {device_fill(shortspan_kernel<1, false>, kShortWaves * 64),
        device_fill(shortspan_kernel<1, true>, kShortWaves * 64)},
@@ -1671,6 +1672,8 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
     if (e != hipSuccess) return e;
     p.plan = plan_slot;
   }
+  if (ntiles == 16)  // 17..32 rows: four waves per KV head
+    return fp8 ? launch_splitkv_w<4, true, 8, 4>(p, st) : launch_splitkv_w<4, false, 8, 4>(p, st);
   if (ntiles == 8)  // 9..16 rows: two waves per KV head (the host checked num_kv_heads % 8 == 0)
     return fp8 ? launch_splitkv_w<4, true, 8, 2>(p, st) : launch_splitkv_w<4, false, 8, 2>(p, st);
   if (fp8) {

@@ -133,7 +133,13 @@ int32_t short_q_max(const eid_attn_desc *d) {
   // the traffic through the CU's cache, so it pays only while the prefill kernel's workgroups
   // (one per sequence and KV head at these lengths) would not fill the device: 8 x 16 rows
   // behind 32k tokens 310 -> 182 us, 32 x 16 behind 8k 322 -> 194 us, 48 x 16 387 -> 300 us,
-  // but 64 x 16 414 -> 427 us (left to the prefill kernel).
+  // but 64 x 16 414 -> 427 us (left to the prefill kernel).  With four waves per KV head
+  // (17..32 rows) the balance tips earlier: 2 x 20 rows behind 60k 296 -> 141 us, 8 x 24
+  // behind 32k 330 -> 273 us, 8 x 32 358 -> 338 us, but 32 x 32 behind 8k 351 -> 360 us.
+  if (d->max_q_len > eid::kShortQMaxRows && d->max_q_len <= eid::kShortQMaxRows4 &&
+      d->num_kv_heads % 8 == 0 &&
+      (long long)d->num_seqs * d->num_kv_heads <= eid::kRows4MaxGroups)
+    return eid::kShortQMaxRows4;  // four waves per KV head: a handful of sequences only (below)
   if (d->max_q_len > eid::kShortQMaxWide && d->max_q_len <= eid::kShortQMaxRows &&
       d->num_kv_heads % 8 == 0 && (long long)d->num_seqs * d->num_kv_heads <= eid::kRowsMaxGroups)
     return eid::kShortQMaxRows;
@@ -143,7 +149,7 @@ int32_t short_q_max(const eid_attn_desc *d) {
 // 16-row tiles per KV head of the verify class: 3, 4, or 8 (two waves of four)
 int verify_tiles(const eid_attn_desc *d) {
   const int32_t q = short_q_max(d);
-  return q == eid::kShortQMaxRows ? 8 : q == eid::kShortQMaxWide ? 4 : 3;
+  return q == eid::kShortQMaxRows4 ? 16 : q == eid::kShortQMaxRows ? 8 : q == eid::kShortQMaxWide ? 4 : 3;
 }
 
 // Longest key span a split-KV sequence can have (from its first visible page to its end).

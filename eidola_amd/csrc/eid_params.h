@@ -12,6 +12,8 @@ constexpr int kGroup = 8;         // query heads per KV head
 constexpr int kShortQMax = 6;     // q_len handled by the split-KV kernel (6*8 = 48 rows = 3 tiles)
 constexpr int kShortQMaxWide = 8; // ... when no sequence of the batch has more than 8 rows: four tiles
 constexpr int kShortQMaxRows = 16; // ... or more than 16: two waves of four tiles share a KV head
+constexpr int kShortQMaxRows4 = 32; // ... or 32: four waves per KV head
+constexpr int kRows4MaxGroups = 64;  // num_seqs * Hkv up to which 17..32 rows take four waves per KV head
 constexpr int kRowsMaxGroups = 448; // ... the latter only for num_seqs * Hkv up to this (see short_q_max)
 constexpr int kChunk = 64;        // tokens a wave consumes per iteration of the split-KV loop
 constexpr int kDynPartitionMin = 256;   // lower bound (and workspace sizing) of the dynamic partition

@@ -473,7 +473,10 @@ def workspace_layout(desc):
     o   float16 [num_seqs*ws_rows, nparts_max, Hq, 64] (partition output sum e^(s-m) v / l) at
     the byte offsets returned."""
     P = partition_size(desc)
-    if (8 < desc.max_q_len <= 16 and desc.num_kv_heads % 8 == 0
+    if (16 < desc.max_q_len <= 32 and desc.num_kv_heads % 8 == 0
+            and desc.num_seqs * desc.num_kv_heads <= 64):
+        qmax = 32
+    elif (8 < desc.max_q_len <= 16 and desc.num_kv_heads % 8 == 0
             and desc.num_seqs * desc.num_kv_heads <= 448):
         qmax = 16   # rows of a split-KV sequence (see short_q_max in eid_api.cpp)
     else:

@@ -178,7 +178,8 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args,
  * verify and mixed prefill+decode batches.  Query row i of sequence s sits at absolute
  * position seq_lens[s] - q_len_s + i and sees keys 0..position (clipped by `window`).
  * Sequences with q_len <= 6 (<= 8 when desc->max_q_len <= 8; <= 16 when desc->max_q_len <= 16,
- * num_kv_heads % 8 == 0 and num_seqs * num_kv_heads <= 448) run on the bandwidth-bound split-KV kernel; longer chunks
+ * num_kv_heads % 8 == 0 and num_seqs * num_kv_heads <= 448; <= 32 when desc->max_q_len <= 32 and
+ * num_seqs * num_kv_heads <= 64) run on the bandwidth-bound split-KV kernel; longer chunks
  * run on the bf16-MFMA tile kernel.  Reference counterpart: none.
  */
 int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
@@ -188,11 +189,11 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  * Stage K4 alone — merge the split-KV partials found in args->workspace (as laid out by
  * the split-KV kernel for this desc) into args->out / args->lse.  Exposed for tests.
  * Serves one class of sequences per call, as the split-KV launches do: q_len <= 2 when
- * desc->max_q_len <= 2, otherwise q_len 3..6 (3..8 or 3..16 under the conditions above).  Sequences with a single partition are left
+ * desc->max_q_len <= 2, otherwise q_len 3..6 (3..8, 3..16 or 3..32 under the conditions above).  Sequences with a single partition are left
  * alone (the split-KV kernel writes their output itself).  With desc->partition_size == 0
  * the partition is the one the last eid_attn_decode / eid_attn_varlen call on this
  * workspace recorded in its header, so such a call must have preceded.
- * Workspace layout, with R = min(max_q_len, 6) (min(max_q_len, 8) or min(max_q_len, 16) under the conditions above) and N = partitions per sequence (max):
+ * Workspace layout, with R = min(max_q_len, 6) (min(max_q_len, 8), 16 or 32 under the conditions above) and N = partitions per sequence (max):
  *   256 bytes                         launch plan (written by the library)
  *   float ml [num_seqs*R][N][Hq][2]   m (natural-log units, -inf if empty) and
  *                                     l = sum of e^(s-m) over the partition's keys

@@ -169,6 +169,9 @@ def test_verify_five_rows(G, window, partition):
     (128, 0, [3000, 700, 150, 13], [16, 10, 8, 13], True),           # ... windowed (one partition each)
     (0, 0, [1200 + 37 * i for i in range(40)], [16, 11] * 20, True),
     (0, 0, [900 + 53 * i for i in range(70)], [16] * 70, False),     # too many for that: prefill kernel
+    (0, 0, [3000, 700, 5000, 90, 32], [32, 17, 3, 1, 32], False),    # 17..32 rows: four waves per KV head
+    (0, 256, [6000, 2100], [20, 25], True),
+    (128, 0, [3000, 700, 150, 30, 400, 77, 900, 64], [32, 20, 8, 30, 1, 17, 24, 2], True),
 ])
 def test_seven_and_eight_query_rows_take_four_tiles(G, kv_dtype, window, partition, seq_lens,
                                                     q_lens, host_lens):
