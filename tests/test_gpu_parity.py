@@ -689,6 +689,36 @@ def test_seeded_small_batches_with_long_contexts(G, seed):
     assert np.allclose(lse, ref_lse, atol=3e-3), what
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_seeded_batches_of_up_to_32_query_rows(G, seed):
+    """Query lengths drawn from 1..8, 1..16 or 1..32 in batches of a few to a few dozen
+    sequences: the classes that stay on the split-KV kernels with four tiles per wave and
+    two or four waves per KV head, or go to the prefill kernel, depending on the batch."""
+    rng = np.random.default_rng(9000 + seed)
+    S = int(rng.integers(1, int(rng.choice([4, 9, 60]))))
+    qmax = int(rng.choice([8, 16, 32]))
+    q_lens = rng.integers(1, qmax + 1, size=S)
+    top = int(rng.choice([300, 3000, 9000]))
+    ctx = np.exp(rng.uniform(0.0, np.log(top), size=S)).astype(np.int64)
+    seq_lens = q_lens + ctx
+    window = int(rng.choice([0, 0, 0, 128, 1000]))
+    partition = int(rng.choice([0, 0, 0, 64, 256, 1024]))
+    kv_dtype = KV_FP8_E4M3 if rng.random() < 0.3 else KV_BF16
+    hint, host = bool(rng.random() < 0.5), bool(rng.random() < 0.5)
+    b = make_batch(seq_lens, q_lens, window=window, partition=partition, kv_dtype=kv_dtype,
+                   seed=seed)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v) if kv_dtype == KV_FP8_E4M3 else (None, None)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, hint=hint,
+                          host_lens=host)
+    what = f"seed {seed}: S={S} q<={qmax} w={window} P={partition} dtype={kv_dtype}"
+    assert_close(out, ref, what)
+    assert np.allclose(lse, ref_lse, atol=3e-3), what
+
+
 # ---------------------------------------------------------------- benchmark configurations
 def _sample_check(G, b, q_d, kc_d, vc_d, sinks, out_d, seqs, what, ks=None, vs=None):
     sub, kc, vc = G.compact_to_cpu(b, kc_d, vc_d, seqs)
