@@ -54,7 +54,12 @@ struct RowInfo {
 // and whose V tile sits in LDS (four 16-token pages of kVRowBytes-padded rows; `v_rd` is
 // the lane's transpose-read base).  The V^T operands are fetched once and reused by all NT
 // row tiles.
-template <int NT, int VROW = kVRowBytes>
+//
+// PRE: the Q operands already carry the factor c2 (load_q<NT, true>), so the MFMA result is
+// the score in log2 units, and the reference maximum enters as the accumulator's initial
+// value: the matrix pipe delivers S * c2 - m and the softmax needs one v_exp_f32 per score,
+// no FMA.  A row that has seen no key yet (m == kNegBig) starts from 0 instead.
+template <int NT, int VROW = kVRowBytes, bool PRE = false>
 __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
                                            const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                            const int tc, const bool need_mask, const float c2,
@@ -80,10 +85,13 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
     // S^T = K Q^T (raw scores, fp32); the prefill kernel raises its priority around MFMA
     // clusters so that the matrix pipe is fed first when both of a SIMD's waves are ready
     f32x4 S[4];
+    const bool fresh = PRE && m[nt] == kNegBig;
+    const float base = fresh ? 0.f : m[nt];
     if (NT == 4) __builtin_amdgcn_s_setprio(2);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      if (PRE) z = f32x4{-base, -base, -base, -base};
       z = mfma16x32(kf[b][0], qf[nt][0], z);
       S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
     }
@@ -108,27 +116,54 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
     mloc = max3(mloc, S[2][3], S[3][0]);
     mloc = max3(mloc, S[3][1], S[3][2]);
     mloc = max2(mloc, S[3][3]);
-    mloc = rowgroup_max(mloc) * c2;
     // Lazy rescaling: the reference maximum m only moves when the running maximum has
     // outgrown it by more than kLazyLog2 (in log2 units), so exp2(s - m) stays <= 2^kLazyLog2
     // (exact in the end: numerator and denominator share m) and the accumulators are
     // rescaled on few chunks only.
-    if (__any(mloc > m[nt] + kLazyLog2)) {
-      const float m_new = mloc > m[nt] + kLazyLog2 ? mloc : m[nt];
-      const float alpha = fast_exp2(m[nt] - m_new);
-      m[nt] = m_new;
+    if constexpr (PRE) {
+      // S holds s - base.  A fresh row moves to its first finite maximum (a fully masked
+      // chunk, maximum -inf, leaves it fresh); the others when the excess passes the slack.
+      mloc = rowgroup_max(mloc);
+      const bool up = mloc > (fresh ? kNegBig : kLazyLog2);
+      if (__any(up)) {
+        const float shift = up ? mloc : 0.f;
+        const float m_new = up ? base + mloc : m[nt];
+        const float alpha = fast_exp2(m[nt] - m_new);
+        m[nt] = m_new;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
+        for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+          for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) S[b][r] -= shift;
+      }
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(S[b][r]);
+    } else {
+      mloc = rowgroup_max(mloc) * c2;
+      if (__any(mloc > m[nt] + kLazyLog2)) {
+        const float m_new = mloc > m[nt] + kLazyLog2 ? mloc : m[nt];
+        const float alpha = fast_exp2(m[nt] - m_new);
+        m[nt] = m_new;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+      }
+      const float m_ref = m[nt];
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_ref));
     }
-    const float m_ref = m[nt];
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) S[b][r] = fast_exp2(__builtin_fmaf(S[b][r], c2, -m_ref));
     // P^T as B operands: pair 0 = pages 0,1; pair 1 = pages 2,3
     Frag8 pf[2];
 #pragma unroll
@@ -419,10 +454,12 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
   }
 }
 
-template <int NT>
+// PRE: the operands are multiplied by `c2` (fp32 product, rounded to bf16 once) for
+// chunk_step<.., PRE = true>.
+template <int NT, bool PRE = false>
 __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, const int qlen,
                                        const int tq0, const int kvh, const int pos0,
-                                       Frag8 (&qf)[NT][2], RowInfo &ri) {
+                                       Frag8 (&qf)[NT][2], RowInfo &ri, const float c2 = 1.0f) {
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
 #pragma unroll
@@ -435,6 +472,16 @@ __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, cons
         p.q + ((size_t)(row0 + tt) * p.num_q_heads + kvh * kGroup + (r & 7)) * kHeadDim + g * 16;
     qf[nt][0].u = valid ? *(const u32x4 *)qp : u32x4{0, 0, 0, 0};
     qf[nt][1].u = valid ? *(const u32x4 *)(qp + 8) : u32x4{0, 0, 0, 0};
+    if constexpr (PRE) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t x = qf[nt][h].w[w];
+          qf[nt][h].w[w] = pack_bf16(bf16_bits_to_f32(x & 0xffffu) * c2,
+                                     __uint_as_float(x & 0xffff0000u) * c2);
+        }
+    }
   }
   ri.t_lane = tq0 + (i16 >> 3);
   ri.tq0 = tq0;
@@ -1010,7 +1057,10 @@ __device__ __forceinline__ bool find_prefill_item(const AttnParams &p, const int
   return false;
 }
 
-template <bool FP8>
+// PRE (taken when the caller asks for no lse): the softmax factor c2 is folded into the Q
+// operands, which costs one more bf16 rounding of Q (lse would be off by up to ~5e-3, the
+// outputs stay within a bf16 ulp of the unfolded path) and saves the FMA per score.
+template <bool FP8, bool PRE>
 __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnParams p) {
   constexpr int NT = 4;
   constexpr int kElt = FP8 ? 1 : 2;
@@ -1070,7 +1120,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
 
   Frag8 qf[NT][2];
   RowInfo ri;
-  load_q<NT>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri);
+  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
+  load_q<NT, PRE>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri, c2);
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
@@ -1080,7 +1131,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
 
   // cooperative loader: thread -> (row of the 64-token chunk, 32-byte segment of the head row)
   const int ld_row = tid >> 2, ld_seg = tid & 3;
@@ -1163,7 +1213,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
         kf[b][1].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes) + 16);
       }
       const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
-      chunk_step<NT, kPfVRowBytes>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
+      chunk_step<NT, kPfVRowBytes, PRE>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
     }
     if (has_next) stash(tc + kChunk, cur ^ 1);
     __syncthreads();
@@ -1695,10 +1745,14 @@ long long prefill_tiles_bound(int num_q_tokens, int num_seqs) {
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st) {
   const long long items = prefill_tiles_bound(num_q_tokens, p.num_seqs) * max(1, p.pf_splits);
   dim3 grid((unsigned)(items * p.num_kv_heads));
-  if (fp8)
-    prefill_kernel<true><<<grid, kPfWaves * 64, 0, st>>>(p);
-  else
-    prefill_kernel<false><<<grid, kPfWaves * 64, 0, st>>>(p);
+  const bool pre = p.lse == nullptr;  // an exact lse needs the unfolded softmax factor
+  if (fp8) {
+    if (pre) prefill_kernel<true, true><<<grid, kPfWaves * 64, 0, st>>>(p);
+    else prefill_kernel<true, false><<<grid, kPfWaves * 64, 0, st>>>(p);
+  } else {
+    if (pre) prefill_kernel<false, true><<<grid, kPfWaves * 64, 0, st>>>(p);
+    else prefill_kernel<false, false><<<grid, kPfWaves * 64, 0, st>>>(p);
+  }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.pf_splits <= 1) return e;
   dim3 mgrid(p.num_q_heads / 4, num_q_tokens);
