@@ -35,7 +35,10 @@
  *   seq_lens          [num_seqs] int32   KV length AFTER this step's append
  *   sinks             [num_q_heads] fp32 (NULL = no sink, i.e. -inf)
  *   k_scale, v_scale  [num_kv_heads] fp32 (fp8 only)
- *   lse               [num_q_tokens, num_q_heads] fp32 (optional) = m + ln(denominator)
+ *   lse               [num_q_tokens, num_q_heads] fp32 (optional) = m + ln(denominator).
+ *                     Asking for it selects the prefill kernel that keeps the softmax factor
+ *                     out of its bf16 Q operands (a few per cent slower; `out` differs from
+ *                     the call without lse by at most a bf16 ulp on prefill rows).
  */
 #ifndef EIDOLA_ATTN_H
 #define EIDOLA_ATTN_H
