@@ -59,7 +59,13 @@ struct RowInfo {
 // the score in log2 units, and the reference maximum enters as the accumulator's initial
 // value: the matrix pipe delivers S * c2 - m and the softmax needs one v_exp_f32 per score,
 // no FMA.  A row that has seen no key yet (m == kNegBig) starts from 0 instead.
-template <int NT, int VROW = kVRowBytes, bool PRE = false>
+//
+// PAIR (decode rows of an fp8 cache, NT == 1): the wave serves two neighbouring KV heads at
+// once.  Its 64 key slots are 32 tokens x 2 heads, slot = 2 * token + head inside each block
+// of 16 slots (exactly what a lane group reads from a token row of the cache: full 128-byte
+// lines), and its 16 rows are the 16 query heads of the pair, row r belonging to head r / 8.
+// A row only attends to the slots of its own head: the others are masked on every chunk.
+template <int NT, int VROW = kVRowBytes, bool PRE = false, bool PAIR = false>
 __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
                                            const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                            const int tc, const bool need_mask, const float c2,
@@ -96,7 +102,25 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
       S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
     }
     if (NT == 4) __builtin_amdgcn_s_setprio(0);
-    if (need_mask) {
+    if constexpr (PAIR) {
+      const bool hi = (threadIdx.x & 8) != 0;  // the row's KV head within the pair
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (((r & 1) != 0) != hi) S[b][r] = -INFINITY;
+      if (need_mask) {
+        int pos, lo;
+        ri.bounds(nt, pos, lo);
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int j = tc + b * (kBlock / 2) + 2 * g + (r >> 1);
+            if (j < lo || j > pos) S[b][r] = -INFINITY;
+          }
+      }
+    } else if (need_mask) {
       int pos, lo;
       ri.bounds(nt, pos, lo);
 #pragma unroll
@@ -219,7 +243,7 @@ struct FirstPages {
   int id[4] = {0, 0, 0, 0};
 };
 
-template <int NT, bool FP8>
+template <int NT, bool FP8, bool PAIR = false>
 __device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
                                        const int t_begin, const int t_end, const int seq_len,
                                        const int pos_first, const int lo_last,
@@ -232,13 +256,20 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   constexpr int kElt = FP8 ? 1 : 2;
   const uint32_t row_bytes = (uint32_t)Hkv * kHeadDim * kElt;
   const size_t page_bytes = (size_t)kBlock * row_bytes;
-  const uint32_t lane_off = (uint32_t)i16 * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
-                            (uint32_t)g * (16 * kElt);
+  static_assert(!PAIR || (FP8 && NT == 1), "head pairs: decode rows of an fp8 cache");
+  // PAIR: a block of 16 slots is 8 token rows x 2 heads (lane i16 = 2 * token + head), two
+  // blocks per page; `kvh` is the first head of the pair.
+  const uint32_t lane_off =
+      PAIR ? (uint32_t)(i16 >> 1) * row_bytes + (uint32_t)(kvh + (i16 & 1)) * (kHeadDim * kElt) +
+                 (uint32_t)g * (16 * kElt)
+           : (uint32_t)i16 * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) + (uint32_t)g * (16 * kElt);
+  constexpr int kBlkTok = PAIR ? kBlock / 2 : kBlock;  // tokens per block of 16 slots
+  const int tok_lane = PAIR ? (i16 >> 1) : i16;        // the lane's token inside its block
   const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
   const int nblk_total = (t_end + kBlock - 1) / kBlock;
   // scores enter the softmax as exp2(S * c2 - m): scale, log2(e) and the fp8 K scale in one
   // factor (> 0: softmax_scale is validated, quantisation scales are magnitudes)
-  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
+  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[PAIR ? kvh + (i16 >> 3) : kvh] : 1.0f);
 
   uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
   const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
@@ -246,8 +277,10 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
   // Page ids travel through scalar registers: the table row and the index are wave-uniform,
   // so these are scalar loads that never share a wait counter with the K/V vector loads.
   // The ids of iteration i+1 are fetched while iteration i is in flight.
-  constexpr int kPages = 4;
-  constexpr int kIter = kChunk;
+  constexpr int kPages = PAIR ? 2 : 4;
+  constexpr int kIter = PAIR ? kChunk / 2 : kChunk;
+  constexpr int kBlocks = 4;                 // blocks of 16 slots per iteration
+  constexpr int kBpp = kBlocks / kPages;     // blocks per page
   // position of the token this launch writes itself, if it lies in [t_begin, t_end); else -1
   const int pos_new = (NT == 1 && p.k_new && seq_len - 1 >= t_begin && seq_len - 1 < t_end)
                           ? seq_len - 1 : -1;
@@ -264,17 +297,18 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
     const int nbi = min(kPages, (t_end - ti + kBlock - 1) / kBlock);
 
     // ---- global loads: each lane takes 32 B (bf16) / 16 B (fp8) of one token row ----
-    u32x4 kraw[kPages][kElt], vraw[kPages][kElt];
+    u32x4 kraw[kBlocks][kElt], vraw[kBlocks][kElt];
 #pragma unroll
-    for (int b = 0; b < kPages; ++b) {
+    for (int b = 0; b < kBlocks; ++b) {
 #pragma unroll
       for (int e = 0; e < kElt; ++e) {
         kraw[b][e] = u32x4{0, 0, 0, 0};
         vraw[b][e] = u32x4{0, 0, 0, 0};
       }
-      if (b < nbi) {
+      if (b / kBpp < nbi) {
         // (clamped here, at its use: at the load it would make the wave wait for the id)
-        const size_t page_off = (size_t)clamp_page(blk[b], p.last_block) * page_bytes + lane_off;
+        const size_t page_off = (size_t)clamp_page(blk[b / kBpp], p.last_block) * page_bytes +
+                                lane_off + (uint32_t)(b % kBpp) * kBlkTok * row_bytes;
         const uint8_t *kp = p.k_cache + page_off;
         const uint8_t *vp = p.v_cache + page_off;
 #pragma unroll
@@ -287,24 +321,26 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
     if (NT == 1 && pos_new >= ti && pos_new < ti + kIter) {  // wave-uniform, once per sequence
       // One 16-byte piece at a time (K then V), so that the rare path adds few live registers
       // to a loop that runs at the register limit of two workgroups per CU.
-      const int b_new = (pos_new - ti) >> 4;
-      const bool mine = i16 == (pos_new & 15);
-      const size_t src = ((size_t)s * Hkv + kvh) * kHeadDim + g * 16;
+      const int b_new = (pos_new - ti) / kBlkTok;
+      const bool mine = tok_lane == (pos_new & (kBlkTok - 1));
+      const size_t src = ((size_t)s * Hkv + (PAIR ? kvh + (i16 & 1) : kvh)) * kHeadDim + g * 16;
       size_t dst = lane_off;
 #pragma unroll
-      for (int b = 0; b < kPages; ++b)
-        if (b == b_new) dst += (size_t)clamp_page(blk[b], p.last_block) * page_bytes;
+      for (int b = 0; b < kBlocks; ++b)
+        if (b == b_new)
+          dst += (size_t)clamp_page(blk[b / kBpp], p.last_block) * page_bytes +
+                 (size_t)(b % kBpp) * kBlkTok * row_bytes;
 #pragma unroll
       for (int kv = 0; kv < 2; ++kv) {
         const uint16_t *from = (kv ? p.v_new : p.k_new) + src;
         uint8_t *to = const_cast<uint8_t *>(kv ? p.v_cache : p.k_cache) + dst;
         if constexpr (FP8) {
-          const float sc = (kv ? p.v_scale : p.k_scale)[kvh];
+          const float sc = (kv ? p.v_scale : p.k_scale)[PAIR ? kvh + (i16 & 1) : kvh];
           const u32x4 x = quantize16_fp8(*(const u32x4 *)from, *(const u32x4 *)(from + 8), sc);
           if (mine) {
             *(u32x4 *)to = x;
 #pragma unroll
-            for (int b = 0; b < kPages; ++b)
+            for (int b = 0; b < kBlocks; ++b)
               if (b == b_new) (kv ? vraw[b][0] : kraw[b][0]) = x;
           }
           asm volatile("" ::: "memory");
@@ -315,7 +351,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
             if (mine) {
               *(u32x4 *)(to + 16 * e) = x;
 #pragma unroll
-              for (int b = 0; b < kPages; ++b)
+              for (int b = 0; b < kBlocks; ++b)
                 if (b == b_new) (kv ? vraw[b][e * (kElt - 1)] : kraw[b][e * (kElt - 1)]) = x;
             }
             asm volatile("" ::: "memory");
@@ -333,7 +369,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
     constexpr int sub = 0;
 
     // ---- V: zero rows past the sequence end, widen fp8, stage in LDS ----
-    const bool tail = tc + kChunk > seq_len;
+    const bool tail = tc + kIter > seq_len;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       u32x4 v0, v1;
@@ -349,7 +385,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
       }
       if (tail) {  // last chunk of the sequence only (kept a real branch, not 8 selects)
         asm volatile("" ::: "memory");
-        if (tc + b * kBlock + i16 >= seq_len) {
+        if (tc + b * kBlkTok + tok_lane >= seq_len) {
           v0 = u32x4{0, 0, 0, 0};
           v1 = u32x4{0, 0, 0, 0};
         }
@@ -370,15 +406,15 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         kf[b][1].u = kraw[4 * sub + b][kElt - 1];
       }
     }
-    const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
-    chunk_step<NT>(kf, lds_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
+    const bool need_mask = (tc < lo_last) || (tc + kIter > pos_first + 1);
+    chunk_step<NT, kVRowBytes, false, PAIR>(kf, lds_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
     }  // sub
   }
 }
 
 // Finish a row tile: either normalise with the sink and store bf16 output (+lse), or store
 // the partition's partial (m, l, acc) for the merge kernel.
-template <int NT, bool FP8>
+template <int NT, bool FP8, bool PAIR = false>
 __device__ __forceinline__ void finish(const AttnParams &p, const int s, const int kvh,
                                        const int row0, const int qlen, const int tq0,
                                        const bool direct, const int part, float (&m)[NT],
@@ -386,13 +422,14 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
   const int Hq = p.num_q_heads;
-  const float vs = FP8 ? p.v_scale[kvh] : 1.0f;
+  const float vs = FP8 ? p.v_scale[PAIR ? kvh + (i16 >> 3) : kvh] : 1.0f;
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const float l = lacc[nt][0];  // every lane of the row holds the full sum
     const int r = nt * 16 + i16;
-    const int t = tq0 + (r >> 3);
-    const int head = kvh * kGroup + (r & 7);
+    // (PAIR: one query token, the 16 rows are the 16 query heads of the two KV heads)
+    const int t = PAIR ? tq0 : tq0 + (r >> 3);
+    const int head = PAIR ? kvh * kGroup + r : kvh * kGroup + (r & 7);
     const bool valid = t < qlen;
     if (direct) {
       if (!valid) continue;
@@ -456,7 +493,7 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
 
 // PRE: the operands are multiplied by `c2` (fp32 product, rounded to bf16 once) for
 // chunk_step<.., PRE = true>.
-template <int NT, bool PRE = false>
+template <int NT, bool PRE = false, bool PAIR = false>
 __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, const int qlen,
                                        const int tq0, const int kvh, const int pos0,
                                        Frag8 (&qf)[NT][2], RowInfo &ri, const float c2 = 1.0f) {
@@ -465,11 +502,11 @@ __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, cons
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     const int r = nt * 16 + i16;
-    const int t = tq0 + (r >> 3);
+    const int t = PAIR ? tq0 : tq0 + (r >> 3);
     const bool valid = t < qlen;
     const int tt = valid ? t : tq0;
-    const uint16_t *qp =
-        p.q + ((size_t)(row0 + tt) * p.num_q_heads + kvh * kGroup + (r & 7)) * kHeadDim + g * 16;
+    const uint16_t *qp = p.q + ((size_t)(row0 + tt) * p.num_q_heads + kvh * kGroup +
+                                (PAIR ? r : (r & 7))) * kHeadDim + g * 16;
     qf[nt][0].u = valid ? *(const u32x4 *)qp : u32x4{0, 0, 0, 0};
     qf[nt][1].u = valid ? *(const u32x4 *)(qp + 8) : u32x4{0, 0, 0, 0};
     if constexpr (PRE) {
@@ -483,7 +520,7 @@ __device__ __forceinline__ void load_q(const AttnParams &p, const int row0, cons
         }
     }
   }
-  ri.t_lane = tq0 + (i16 >> 3);
+  ri.t_lane = PAIR ? tq0 : tq0 + (i16 >> 3);
   ri.tq0 = tq0;
   ri.qlen = qlen;
   ri.pos0 = pos0;
@@ -712,7 +749,7 @@ __global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *p
 
 // One work item: wave `wave` of the workgroup attends the rows of KV head `kvh` over
 // partition it.part (P tokens) of sequence it.seq and writes the output or the partial.
-template <int NT, bool FP8>
+template <int NT, bool FP8, bool PAIR = false>
 __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem &it, const int P,
                                              const int kvh, const int wave, uint8_t *lds,
                                              const FirstPages &first = FirstPages{},
@@ -728,7 +765,7 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
   Frag8 qf[NT][2];
   RowInfo ri;
   if (tq0 >= qlen) return;  // (a row group past the sequence's rows)
-  load_q<NT>(p, row0, qlen, tq0, kvh, pos0, qf, ri);
+  load_q<NT, false, PAIR>(p, row0, qlen, tq0, kvh, pos0, qf, ri);
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
@@ -738,9 +775,9 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  attend<NT, FP8>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes, m,
-                  lacc, acc, first);
-  finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, nparts == 1, part, m, lacc, acc);
+  attend<NT, FP8, PAIR>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes,
+                        m, lacc, acc, first);
+  finish<NT, FP8, PAIR>(p, s, kvh, row0, qlen, tq0, nparts == 1, part, m, lacc, acc);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -753,12 +790,15 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
 // RS > 1 (q_len beyond one wave's rows): RS waves share a KV head, wave w taking the query
 // tokens [8 (w % RS), +8) of the sequence; the workgroup then covers WAVES / RS KV heads and
 // the grid's y dimension grows by RS.  Both waves load the head's K/V (the second from cache).
-template <int NT, bool FP8, int WAVES, int RS = 1>
+//
+// PAIR (fp8 decode rows): every wave owns two neighbouring KV heads, see chunk_step.
+template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
 __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(const AttnParams p) {
   static_assert(RS == 1 || (NT == 4 && WAVES % RS == 0), "row groups are 8 tokens = four tiles");
+  static_assert(!PAIR || RS == 1, "head pairs have one row group");
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kvh = blockIdx.y * (WAVES / RS) + wave / RS;
+  const int kvh = (blockIdx.y * (WAVES / RS) + wave / RS) * (PAIR ? 2 : 1);
   const int tq0 = (wave % RS) * (NT * 16 / kGroup);
   if (p.nparts_max == 1) {
     // Every sequence is a single item (short spans: sliding-window layers, short contexts):
@@ -773,7 +813,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
     it.row0 = v.row0;
     it.qlen = v.qlen;
     it.seq_len = v.seq_len;
-    splitkv_item<NT, FP8>(p, it, 1 << 30, kvh, wave, lds, FirstPages{}, tq0);
+    splitkv_item<NT, FP8, PAIR>(p, it, 1 << 30, kvh, wave, lds, FirstPages{}, tq0);
     return;
   }
   if (planned_out(p, blockIdx.x)) return;
@@ -807,7 +847,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   it.seq_len = __builtin_amdgcn_readfirstlane(item_lds[6]);
   // the merge launch that follows reads the partition from here instead of re-deriving it
   if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
-  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds, FirstPages{}, tq0);
+  splitkv_item<NT, FP8, PAIR>(p, it, P, kvh, wave, lds, FirstPages{}, tq0);
 }
 
 // The same for a decode launch whose items the host has listed (q_len 1, row = sequence):
@@ -825,12 +865,12 @@ __device__ __forceinline__ WorkItem table_item(const AttnParams &p, const ItemTa
   return it;
 }
 
-template <int NT, bool FP8, int WAVES>
+template <int NT, bool FP8, int WAVES, bool PAIR = false>
 __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_table_kernel(
     const AttnParams p, const ItemTable tab) {
   __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int kvh = blockIdx.y * WAVES + wave;
+  const int kvh = (blockIdx.y * WAVES + wave) * (PAIR ? 2 : 1);
   if ((int)blockIdx.x >= tab.n) return;
   const int P = p.partition;
   const WorkItem it = table_item(p, tab, blockIdx.x, P);
@@ -839,7 +879,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_table_k
   first.have = tab.has_blk;  // compiler copy the whole list into private memory)
 #pragma unroll
   for (int b = 0; b < 4; ++b) first.id[b] = tab.blk[blockIdx.x][b];
-  splitkv_item<NT, FP8>(p, it, P, kvh, wave, lds, first);
+  splitkv_item<NT, FP8, PAIR>(p, it, P, kvh, wave, lds, first);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1548,9 +1588,9 @@ int device_cus() {
   return cus;
 }
 
-template <int NT, bool FP8, int WAVES, int RS = 1>
+template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
 static int fill_of() {
-  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES, RS>, WAVES * 64);
+  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES, RS, PAIR>, WAVES * 64);
   return fill;
 }
 
@@ -1567,7 +1607,8 @@ static int fill_t(int waves) {
 static int waves_for(int Hkv) { return Hkv >= 8 ? 8 : Hkv; }
 
 // Workgroups of the split-KV instantiation (ntiles, fp8, Hkv) the device holds at once.
-int splitkv_fill(int ntiles, bool fp8, int Hkv) {
+int splitkv_fill(int ntiles, bool fp8, int Hkv, bool pair) {
+  if (pair && fp8 && ntiles == 1) return fill_of<1, true, 4, 1, true>();  // two KV heads per wave
   const int waves = waves_for(Hkv);
   if (ntiles == 8) return fp8 ? fill_of<4, true, 8, 2>() : fill_of<4, false, 8, 2>();  // two row groups
   if (ntiles == 16) return fp8 ? fill_of<4, true, 8, 4>() : fill_of<4, false, 8, 4>();  // four
@@ -1611,9 +1652,9 @@ static long long item_bound(const AttnParams &p) {
   return items;
 }
 
-template <int NT, bool FP8, int WAVES, int RS = 1>
+template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
-  dim3 grid((unsigned)item_bound(p), p.num_kv_heads / (WAVES / RS));
+  dim3 grid((unsigned)item_bound(p), p.num_kv_heads / (WAVES / RS) / (PAIR ? 2 : 1));
   // With a prefill launch beside it (mixed batch, p.share_cus): one 8-wave workgroup per CU.
   // A second resident workgroup adds little to a kernel that streams from HBM (it only
   // covers the prologues of many short items), while half of the CU's registers left free
@@ -1626,13 +1667,13 @@ static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return e;
     if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
-      e = hipFuncSetAttribute((const void *)splitkv_kernel<NT, FP8, WAVES, RS>,
+      e = hipFuncSetAttribute((const void *)splitkv_kernel<NT, FP8, WAVES, RS, PAIR>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, kPad);
       if (e != hipSuccess) return e;
       if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
     }
   }
-  splitkv_kernel<NT, FP8, WAVES, RS><<<grid, WAVES * 64, kPad, st>>>(p);
+  splitkv_kernel<NT, FP8, WAVES, RS, PAIR><<<grid, WAVES * 64, kPad, st>>>(p);
   return hipGetLastError();
 }
 
@@ -1711,7 +1752,8 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   if (tab && ntiles == 1 && p.nparts_max > 1 && !p.dynamic_partition && !p.share_cus &&
       waves_for(p.num_kv_heads) == 8) {
     dim3 grid((unsigned)tab->n, p.num_kv_heads / 8);
-    if (fp8) splitkv_table_kernel<1, true, 8><<<grid, 512, 0, st>>>(p, *tab);
+    if (fp8 && p.fp8_pair) splitkv_table_kernel<1, true, 4, true><<<grid, 256, 0, st>>>(p, *tab);
+    else if (fp8) splitkv_table_kernel<1, true, 8><<<grid, 512, 0, st>>>(p, *tab);
     else splitkv_table_kernel<1, false, 8><<<grid, 512, 0, st>>>(p, *tab);
     return hipGetLastError();
   }
@@ -1727,6 +1769,8 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   if (ntiles == 8)  // 9..16 rows: two waves per KV head (the host checked num_kv_heads % 8 == 0)
     return fp8 ? launch_splitkv_w<4, true, 8, 2>(p, st) : launch_splitkv_w<4, false, 8, 2>(p, st);
   if (fp8) {
+    // decode rows only, eight KV heads: four waves per workgroup, two KV heads per wave
+    if (ntiles == 1 && p.fp8_pair) return launch_splitkv_w<1, true, 4, 1, true>(p, st);
     if (ntiles == 1) return launch_splitkv_t<1, true>(p, st);
     if (ntiles == 3) return launch_splitkv_t<3, true>(p, st);
     return launch_splitkv_t<4, true>(p, st);

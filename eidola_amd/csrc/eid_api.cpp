@@ -14,7 +14,7 @@
 namespace eid {
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
                           const ItemTable *tab = nullptr);
-int splitkv_fill(int ntiles, bool fp8, int Hkv);
+int splitkv_fill(int ntiles, bool fp8, int Hkv, bool pair = false);
 hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st,
                             const ItemTable *tab = nullptr);
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
@@ -415,7 +415,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   p.partition = pl.partition;
   p.dynamic_partition = pl.dynamic ? 1 : 0;
   p.exact_items = 0;
-  p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads);
+  p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0);
   cp.short_span = use_shortspan(d, pl, ntiles);
   cp.merge = pl.nparts_max > 1;
   constexpr int32_t kHostPlanMaxSeqs = 8192;  // beyond that the host pass is no longer free
@@ -591,6 +591,15 @@ int32_t eid_qkv_rope_kv_write(const eid_attn_desc *desc, const void *hidden, con
   return EID_OK;
 }
 
+// Decode rows over an fp8 cache: a wave of the split-KV kernel takes two neighbouring KV
+// heads, so that its loads cover whole 128-byte lines of a token row (one head's 64 fp8
+// bytes are half a line).  Needs one query row per sequence (the 16 rows of a wave's tile
+// are then the 16 query heads of the pair) and KV heads in groups of eight.
+static bool fp8_pair_applies(const eid_attn_desc *d) {
+  static const bool off = getenv("EID_NO_FP8_PAIR") != nullptr;  // for A/B measurements
+  return !off && d->kv_dtype == EID_KV_FP8_E4M3 && d->max_q_len == 1 && d->num_kv_heads % 8 == 0;
+}
+
 int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {
   g_err[0] = 0;
   if (int32_t rc = check_attn_desc(desc)) return rc;
@@ -608,6 +617,7 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   p.v_new = static_cast<const uint16_t *>(args->v_new);
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   eid::ItemTable table;  // (3 KiB on the stack; only `n` entries are ever read)
   const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table);
@@ -661,6 +671,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   static const bool serial = getenv("EID_SERIAL_CLASSES") != nullptr;  // for A/B measurements
   Helper *hs = (has_prefill && !only_prefill && !serial) ? helper_stream() : nullptr;
   p.share_cus = hs ? 1 : 0;
+  p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
   if (hs) {
     e = hipEventRecord(hs->fork, st);
     if (e == hipSuccess) e = hipStreamWaitEvent(hs->stream, hs->fork, 0);

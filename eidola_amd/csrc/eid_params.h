@@ -55,6 +55,8 @@ struct AttnParams {
   float *pf_ml;              // [num_q_tokens][pf_splits][Hq][2]   (m natural-log units, l)
   _Float16 *pf_acc;          // [num_q_tokens][pf_splits][Hq][64]  part output, normalised
   int32_t num_q_tokens;
+  int32_t fp8_pair;          // host-side launch flag: 1 = every sequence has one query row, fp8 cache,
+                             // eight KV heads: the split-KV launch may give each wave two KV heads
   int32_t share_cus;         // host-side launch flag: 1 = hold the split-KV kernel to one
                              // workgroup per CU (a prefill launch runs beside it)
   long long exact_items;     // host-side: the launch's exact number of work items when the host

@@ -96,6 +96,19 @@ def test_large_batch_with_launch_hint(G):
     _run(G, list(rng.integers(1, 400, size=70)), seed=9, kv_dtype=KV_FP8_E4M3)
 
 
+@pytest.mark.parametrize("hkv,window,partition,hint", [
+    (8, 0, 0, False), (8, 0, 0, True), (8, 0, 256, False), (8, 300, 0, True), (16, 0, 0, True),
+])
+def test_fp8_head_pairs_beyond_one_device_fill(G, hkv, window, partition, hint):
+    """fp8 decode batches too large for the short-span kernel: the split-KV kernel gives every
+    wave two KV heads (32 tokens x 2 heads per step).  Newest tokens at every offset of such a
+    step, sequence ends inside a step, 8 and 16 KV heads."""
+    rng = np.random.default_rng(31)
+    lens = list(rng.integers(1500, 2600, size=30)) + list(range(1100, 1134))
+    _run(G, lens, kv_dtype=KV_FP8_E4M3, hkv=hkv, window=window, partition=partition, seed=12,
+         hint=hint)
+
+
 def test_varlen_entry_rejects_the_fused_arguments(G):
     batch = make_batch([40, 50], [2, 1])
     q, k, v, sinks = logical_tensors(batch)

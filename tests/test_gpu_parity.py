@@ -111,6 +111,30 @@ def test_decode_without_sinks_and_with_extreme_sinks(G):
         assert_close(out, ref, f"sinks={None if sk is None else sk[0]}")
 
 
+@pytest.mark.parametrize("hkv", [8, 16])
+@pytest.mark.parametrize("window,partition,host_lens", [(0, 0, False), (0, 0, True), (0, 128, True),
+                                                        (200, 0, False)])
+def test_fp8_decode_two_kv_heads_per_wave(G, hkv, window, partition, host_lens):
+    """One query row per sequence over an fp8 cache with KV heads in groups of eight: a wave of
+    the split-KV kernel serves two neighbouring KV heads (per-head scales, sinks and outputs
+    must land on the right 16 query heads).  Long and short sequences, ends at every offset of
+    a 32-token step, with lse; also through the host's item list."""
+    seq_lens = [2100 + i for i in range(33)] + [5000, 64, 1, 31, 32, 33, 700, 9000]
+    b = make_batch(seq_lens, [1] * len(seq_lens), window=window, partition=partition,
+                   kv_dtype=KV_FP8_E4M3, num_kv_heads=hkv, seed=77)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v)
+    ks = (ks * np.linspace(0.5, 2.0, hkv)).astype(np.float32)   # clearly different per head
+    vs = (vs * np.linspace(2.0, 0.5, hkv)).astype(np.float32)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, host_lens=host_lens,
+                          hint=host_lens, decode=True)
+    assert_close(out, ref, f"fp8 head pairs Hkv={hkv} w={window} P={partition}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
 def test_decode_two_kv_heads(G):
     b = make_batch([200, 33], [1, 1], num_kv_heads=2, partition=64)
     q, k, v, sinks = logical_tensors(b)
