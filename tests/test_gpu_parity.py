@@ -292,6 +292,41 @@ def test_prefill_chunks_and_decodes_mixed(G, window):
     assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, f"prefill mixed w={window}, no lse")
 
 
+@pytest.mark.parametrize("shape", ["rising", "falling", "deep"])
+@pytest.mark.parametrize("window", [0, 100])
+def test_prefill_scores_far_from_zero(G, shape, window):
+    """Scores that climb by tens of log2 units per 64-key chunk (the reference maximum of the
+    lazy softmax moves on every chunk), fall as fast (later chunks underflow against it), or sit
+    some 70 log2 units below zero throughout (a row's first maximum is far from the value its
+    accumulator starts at).  Prefill rows and a few decode / verify rows, with lse (unfolded
+    softmax factor) and without (factor folded into the Q operands)."""
+    seq_lens, q_lens = [600, 333, 64, 700, 90], [64, 333, 64, 5, 1]
+    b = make_batch(seq_lens, q_lens, window=window, seed=61)
+    q, k, v, sinks = logical_tensors(b)
+    qf = synth.bf16_bits_to_f32(q) * np.float32(0.5)
+    kf = synth.bf16_bits_to_f32(k) * np.float32(0.5)
+    # a common offset on all 64 dims: q.k grows by 64 * (q offset) * (k offset), times 1/8
+    pos = np.concatenate([np.arange(L, dtype=np.float32) for L in seq_lens])[:, None, None]
+    if shape == "rising":        # + 0.5 nats per key position: 32 nats = 46 log2 units per chunk
+        qf += 1
+        kf += pos / 16
+    elif shape == "falling":
+        qf += 1
+        kf -= pos / 16
+    else:                        # about -50 nats everywhere
+        qf -= 1
+        kf += np.float32(6.25)
+    q, k = synth.f32_to_bf16_bits(qf), synth.f32_to_bf16_bits(kf)
+    sinks = None if shape == "deep" else sinks
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+    assert_close(out, ref, f"{shape} w={window}")
+    assert np.allclose(lse, ref_lse, atol=2e-3, rtol=1e-5)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, f"{shape} w={window}, no lse")
+
+
 def test_varlen_at_qlen1_equals_decode_entry_point(G):
     b = make_batch([100, 1000, 17], [1, 1, 1], partition=128)
     q, k, v, sinks = logical_tensors(b)
