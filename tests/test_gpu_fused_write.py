@@ -27,7 +27,8 @@ def G():
     return gpu_helpers
 
 
-def _run(G, seq_lens, *, kv_dtype=KV_BF16, window=0, hkv=8, partition=0, seed=3, hint=False):
+def _run(G, seq_lens, *, kv_dtype=KV_BF16, window=0, hkv=8, partition=0, seed=3, hint=False,
+         host=False):
     batch = make_batch(seq_lens, [1] * len(seq_lens), seed=seed, window=window, kv_dtype=kv_dtype,
                        num_kv_heads=hkv, partition=partition)
     g = batch.geom
@@ -48,6 +49,8 @@ def _run(G, seq_lens, *, kv_dtype=KV_BF16, window=0, hkv=8, partition=0, seed=3,
     kn_d, vn_d = G.bf16_dev(k[ends]), G.bf16_dev(v[ends])
     kw = dict(max_kv_len=batch.max_kv_len, sinks=G.dev(sinks), k_scale=G.dev(ks), v_scale=G.dev(vs),
               sum_kv_len=int(batch.seq_lens.sum()) if hint else 0)
+    if host:  # the host's item list (and first page ids) instead of the device-side lookup
+        kw.update(seq_lens_host=batch.seq_lens, block_table_host=batch.block_table)
     bt, sl, q_d = G.dev(batch.block_table), G.dev(batch.seq_lens), G.bf16_dev(q)
     # A: two launches
     ea.kv_write(g, kn_d, vn_d, kc_a, vc_a, G.dev(new_slots), G.dev(ks), G.dev(vs))
@@ -96,17 +99,27 @@ def test_large_batch_with_launch_hint(G):
     _run(G, list(rng.integers(1, 400, size=70)), seed=9, kv_dtype=KV_FP8_E4M3)
 
 
-@pytest.mark.parametrize("hkv,window,partition,hint", [
-    (8, 0, 0, False), (8, 0, 0, True), (8, 0, 256, False), (8, 300, 0, True), (16, 0, 0, True),
+@pytest.mark.parametrize("hkv,window,partition,hint,host", [
+    (8, 0, 0, False, False), (8, 0, 0, True, False), (8, 0, 256, False, False),
+    (8, 300, 0, True, False), (16, 0, 0, True, False), (8, 0, 0, True, True), (16, 0, 1024, True, True),
 ])
-def test_fp8_head_pairs_beyond_one_device_fill(G, hkv, window, partition, hint):
+def test_fp8_head_pairs_beyond_one_device_fill(G, hkv, window, partition, hint, host):
     """fp8 decode batches too large for the short-span kernel: the split-KV kernel gives every
     wave two KV heads (32 tokens x 2 heads per step).  Newest tokens at every offset of such a
     step, sequence ends inside a step, 8 and 16 KV heads."""
     rng = np.random.default_rng(31)
     lens = list(rng.integers(1500, 2600, size=30)) + list(range(1100, 1134))
     _run(G, lens, kv_dtype=KV_FP8_E4M3, hkv=hkv, window=window, partition=partition, seed=12,
-         hint=hint)
+         hint=hint, host=host)
+
+
+@pytest.mark.parametrize("kv_dtype", [KV_BF16, KV_FP8_E4M3])
+def test_fused_write_with_the_hosts_item_list(G, kv_dtype):
+    """A batch whose items fit the list a launch can carry: the split-KV kernel takes its
+    items (and their first page ids) from the kernel arguments and still writes the newest
+    tokens on its way."""
+    rng = np.random.default_rng(41)
+    _run(G, list(rng.integers(1, 8192, size=64)), kv_dtype=kv_dtype, seed=13, hint=True, host=True)
 
 
 def test_varlen_entry_rejects_the_fused_arguments(G):
