@@ -16,6 +16,7 @@ EID_ERR_UNSUPPORTED = -2
 EID_ERR_WORKSPACE = -3
 EID_ERR_HIP = -4
 EID_ERR_NO_BLOCKS = -5
+STATIC_WORKSPACE_BYTES = 32 << 20   # EID_STATIC_WORKSPACE_BYTES of the header
 
 _STATUS_NAMES = {
     EID_ERR_INVALID_ARG: "EID_ERR_INVALID_ARG",
@@ -100,8 +101,8 @@ class BatchInfo(C.Structure):
     ]
 
 
-EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_qkv_rope_kv_write", "eid_attn_decode", "eid_attn_varlen", "eid_lse_merge",
-           "eid_o_proj",
+EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_qkv_rope_kv_write", "eid_attn_decode",
+           "eid_attn_decode_noalloc", "eid_attn_varlen", "eid_lse_merge", "eid_o_proj",
            "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
                  "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
@@ -139,7 +140,7 @@ def load_library():
     lib.eid_qkv_rope_kv_write.restype = C.c_int32
     lib.eid_o_proj.argtypes = [P, P, P, P, P, C.c_int32, C.c_int32, C.c_int32, P]
     lib.eid_o_proj.restype = C.c_int32
-    for name in ("eid_attn_decode", "eid_attn_varlen", "eid_lse_merge"):
+    for name in ("eid_attn_decode", "eid_attn_decode_noalloc", "eid_attn_varlen", "eid_lse_merge"):
         fn = getattr(lib, name)
         fn.argtypes = [C.POINTER(AttnDesc), C.POINTER(AttnArgs), P]
         fn.restype = C.c_int32

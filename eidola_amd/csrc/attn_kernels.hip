@@ -1833,6 +1833,35 @@ hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------
+// Split-KV workspace owned by the library, for the decode entry point that allocates nothing:
+// a file-scope device array, one copy per GPU the library runs on, held until the process
+// ends.  Its name is a host-side stand-in here, not a device address: host code asks the
+// runtime for the address once per device (with that device current) and from then on only
+// ever uses that pointer, for kernel arguments as for anything else.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
+
+hipError_t static_scratch(uint8_t **ptr) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<uint8_t *> addr[kMaxDevices];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  uint8_t *p = addr[dev].load(std::memory_order_acquire);
+  if (!p) {  // first call on this device (threads racing here obtain the same address)
+    void *sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!sym) return hipErrorInvalidSymbol;
+    p = static_cast<uint8_t *>(sym);
+    addr[dev].store(p, std::memory_order_release);
+  }
+  *ptr = p;
+  return hipSuccess;
+}
+
 hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t *k_cache,
                            uint8_t *v_cache, const int64_t *slot_mapping, const float *k_scale,
                            const float *v_scale, int Hkv, int64_t num_slots, int num_tokens,

@@ -27,6 +27,7 @@ hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
                                 const float *k_scale, const float *v_scale, int Hq, int Hkv,
                                 int64_t num_slots, int num_tokens, bool fp8, hipStream_t st);
 int device_cus();
+hipError_t static_scratch(uint8_t **ptr);
 long long prefill_tiles_bound(int num_q_tokens, int num_seqs);
 hipError_t launch_qkv_rope(const uint16_t *a, const uint16_t *w, const uint16_t *bias, int T, int K,
                            const RopeArgs &r, hipStream_t st);
@@ -38,6 +39,9 @@ hipError_t launch_kv_write(const uint16_t *k_new, const uint16_t *v_new, uint8_t
                            const float *v_scale, int Hkv, int64_t num_slots, int num_tokens,
                            bool fp8, hipStream_t st);
 }  // namespace eid
+
+static_assert(EID_STATIC_WORKSPACE_BYTES == eid::kStaticScratchBytes,
+              "the header states the size of the static workspace");
 
 namespace {
 thread_local char g_err[512] = "";
@@ -217,7 +221,7 @@ Plan make_plan(const eid_attn_desc *d) {
 }
 
 int32_t check_attn_args(const eid_attn_desc *d, const eid_attn_args *a, bool need_q,
-                        bool need_cu) {
+                        bool need_cu, bool need_ws = true) {
   if (!a) return fail(EID_ERR_INVALID_ARG, "args is NULL");
   if (need_q && (!a->q || !a->k_cache || !a->v_cache || !a->block_table))
     return fail(EID_ERR_INVALID_ARG, "q, k_cache, v_cache and block_table must be non-NULL");
@@ -227,6 +231,7 @@ int32_t check_attn_args(const eid_attn_desc *d, const eid_attn_args *a, bool nee
     return fail(EID_ERR_INVALID_ARG, "q, out, k_cache and v_cache must be 16-byte aligned");
   if (d->kv_dtype == EID_KV_FP8_E4M3 && need_q && (!a->k_scale || !a->v_scale))
     return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
+  if (!need_ws) return EID_OK;
   const Plan pl = make_plan(d);
   const size_t need =
       eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
@@ -324,33 +329,36 @@ int32_t hip_fail(hipError_t e, const char *what) {
 
 // ---- launch planning from the caller's host copies of seq_lens / cu_seqlens_q ----------
 
-// Key spans of the sequences of one q_len class, as the kernels see them (view_seq).
+// Key spans of the sequences of one q_len class, as the kernels see them (view_seq).  The
+// three arrays live in storage the caller provides (num_seqs entries each).
 struct ClassSpans {
-  std::vector<int32_t> spans, seq, len;  // span, index and length of every such sequence
+  int32_t *spans = nullptr, *seq = nullptr, *len = nullptr;  // span, index, length per sequence
+  size_t n = 0;
   long long total = 0;
   int32_t longest = 0;
   long long items(int32_t P, int32_t nparts_max) const {
-    long long n = 0;
-    for (const int32_t sp : spans) n += std::min((sp + P - 1) / P, nparts_max);
-    return n;
+    long long c = 0;
+    for (size_t i = 0; i < n; ++i) c += std::min((spans[i] + P - 1) / P, nparts_max);
+    return c;
   }
 };
 
 ClassSpans class_spans(const eid_attn_desc *d, const int32_t *seq_lens, const int32_t *cu,
-                       int32_t ws_rows, int32_t qlen_lo, int32_t qlen_hi) {
+                       int32_t ws_rows, int32_t qlen_lo, int32_t qlen_hi, int32_t *storage) {
   ClassSpans c;
-  c.spans.reserve(d->num_seqs);
-  c.seq.reserve(d->num_seqs);
-  c.len.reserve(d->num_seqs);
+  c.spans = storage;
+  c.seq = storage + d->num_seqs;
+  c.len = storage + 2 * (size_t)d->num_seqs;
   for (int32_t s = 0; s < d->num_seqs; ++s) {
     const int32_t L = std::min<int64_t>(seq_lens[s], (int64_t)d->max_blocks_per_seq * eid::kBlock);
     const int32_t qlen = cu ? cu[s + 1] - cu[s] : 1;
     if (qlen < qlen_lo || qlen > qlen_hi || qlen > ws_rows || L < qlen) continue;
     const int32_t span = L - eid::kv_begin(L, qlen, d->window);
     if (span <= 0) continue;
-    c.spans.push_back(span);
-    c.seq.push_back(s);
-    c.len.push_back(L);
+    c.spans[c.n] = span;
+    c.seq[c.n] = s;
+    c.len[c.n] = L;
+    ++c.n;
     c.total += span;
     c.longest = std::max(c.longest, span);
   }
@@ -362,7 +370,7 @@ ClassSpans class_spans(const eid_attn_desc *d, const int32_t *seq_lens, const in
 // uniform batches, about three fills), computed once here instead of by every workgroup.
 int32_t host_partition(const ClassSpans &c, long long T, long long Tlo, int32_t Pmin,
                        int32_t nparts_max) {
-  const long long active = (long long)c.spans.size(), cap = eid::kDynPartitionCap;
+  const long long active = (long long)c.n, cap = eid::kDynPartitionCap;
   auto up64 = [](long long v) { return (v + 63) / 64 * 64; };
   auto single_fill = [&](const long long Tx) -> int32_t {
     if (active > Tx) return 0;
@@ -404,9 +412,11 @@ struct ClassPlan {
 // Sets p.partition / p.dynamic_partition / p.exact_items for the class [qlen_lo, qlen_hi] and
 // says which kernel serves it.  Without host lengths this is the plan made from the
 // descriptor alone; with them, the run-time choices of the kernels are made here.
+// `no_heap`: the call must not allocate (host memory included): batches beyond the stack
+// storage are then left to the kernels' own planning.
 ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan &pl,
                      eid::AttnParams &p, int ntiles, int32_t qlen_lo, int32_t qlen_hi,
-                     bool decode, eid::ItemTable *table = nullptr) {
+                     bool decode, eid::ItemTable *table = nullptr, bool no_heap = false) {
   ClassPlan cp;
   if (table) table->n = table->has_blk = 0;
   const bool fp8 = d->kv_dtype == EID_KV_FP8_E4M3;
@@ -421,13 +431,20 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   constexpr int32_t kHostPlanMaxSeqs = 8192;  // beyond that the host pass is no longer free
   const int32_t *cu = decode ? nullptr : a->cu_seqlens_q_host;
   if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs) return cp;
-  ClassSpans c;
-  try {
-    c = class_spans(d, a->seq_lens_host, cu, pl.ws_rows, qlen_lo, qlen_hi);
-  } catch (...) {  // out of host memory: nothing may cross the C ABI; the kernels plan instead
-    return cp;
+  int32_t stack_store[3 * eid::kStackPlanSeqs];  // 12 KiB: most batches need no heap at all
+  std::vector<int32_t> heap_store;
+  int32_t *store = stack_store;
+  if (d->num_seqs > eid::kStackPlanSeqs) {
+    if (no_heap) return cp;
+    try {
+      heap_store.resize(3 * (size_t)d->num_seqs);
+    } catch (...) {  // out of host memory: nothing may cross the C ABI; the kernels plan instead
+      return cp;
+    }
+    store = heap_store.data();
   }
-  if (c.spans.empty()) {
+  const ClassSpans c = class_spans(d, a->seq_lens_host, cu, pl.ws_rows, qlen_lo, qlen_hi, store);
+  if (c.n == 0) {
     cp.skip = true;
     return cp;
   }
@@ -445,14 +462,14 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
     p.dynamic_partition = 0;
   }
   p.exact_items = c.items(p.partition, pl.nparts_max);
-  cp.merge = p.exact_items > (long long)c.spans.size();
+  cp.merge = p.exact_items > (long long)c.n;
   // Few items of a decode launch: list them for the kernels (sequence-major, as they would
   // find them themselves)
   static const bool no_table = getenv("EID_NO_ITEM_TABLE") != nullptr;  // for A/B measurements
   if (table && decode && !no_table && p.exact_items <= eid::kItemTableMax) {
     int32_t n = 0;
     const int32_t *bth = a->block_table_host;
-    for (size_t i = 0; i < c.spans.size(); ++i) {
+    for (size_t i = 0; i < c.n; ++i) {
       const int32_t parts = std::min((c.spans[i] + p.partition - 1) / p.partition, pl.nparts_max);
       const int32_t L = c.len[i], kb = eid::kv_begin(L, 1, d->window);
       for (int32_t part = 0; part < parts; ++part) {
@@ -600,12 +617,10 @@ static bool fp8_pair_applies(const eid_attn_desc *d) {
   return !off && d->kv_dtype == EID_KV_FP8_E4M3 && d->max_q_len == 1 && d->num_kv_heads % 8 == 0;
 }
 
-int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {
-  g_err[0] = 0;
-  if (int32_t rc = check_attn_desc(desc)) return rc;
-  if (desc->max_q_len != 1 || desc->num_q_tokens != desc->num_seqs)
-    return fail(EID_ERR_INVALID_ARG, "decode needs max_q_len == 1 and num_q_tokens == num_seqs");
-  if (int32_t rc = check_attn_args(desc, args, true, false)) return rc;
+// Decode call on validated arguments whose workspace is in place (the caller's, or the
+// library's own static array).
+static int32_t decode_launch(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream,
+                             bool no_heap) {
   const Plan pl = make_plan(desc);
   eid::AttnParams p = make_params(desc, args, pl);
   p.cu_seqlens_q = nullptr;  // one row per sequence by contract
@@ -619,8 +634,8 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
-  eid::ItemTable table;  // (3 KiB on the stack; only `n` entries are ever read)
-  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table);
+  eid::ItemTable table;  // (8 KiB on the stack; only `n` entries are ever read)
+  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table, no_heap);
   if (cp.skip) return EID_OK;  // (every sequence empty or malformed: nothing is written)
   const eid::ItemTable *tab = table.n > 0 ? &table : nullptr;
   // spans of at most 8 chunks, or a small batch in partitions of that size: one workgroup
@@ -637,6 +652,38 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, vo
     if (e != hipSuccess) return hip_fail(e, "merge launch");
   }
   return EID_OK;
+}
+
+int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_attn_desc(desc)) return rc;
+  if (desc->max_q_len != 1 || desc->num_q_tokens != desc->num_seqs)
+    return fail(EID_ERR_INVALID_ARG, "decode needs max_q_len == 1 and num_q_tokens == num_seqs");
+  if (int32_t rc = check_attn_args(desc, args, true, false)) return rc;
+  return decode_launch(desc, args, hip_stream, false);
+}
+
+int32_t eid_attn_decode_noalloc(const eid_attn_desc *desc, const eid_attn_args *args,
+                                void *hip_stream) {
+  g_err[0] = 0;
+  if (int32_t rc = check_attn_desc(desc)) return rc;
+  if (desc->max_q_len != 1 || desc->num_q_tokens != desc->num_seqs)
+    return fail(EID_ERR_INVALID_ARG, "decode needs max_q_len == 1 and num_q_tokens == num_seqs");
+  if (int32_t rc = check_attn_args(desc, args, true, false, false)) return rc;
+  const Plan pl = make_plan(desc);
+  const size_t need = eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes;
+  if (need > eid::kStaticScratchBytes)
+    return fail(EID_ERR_WORKSPACE,
+                "this batch needs %zu bytes of split-KV workspace; the library's static array holds "
+                "%zu: use eid_attn_decode with a workspace of the caller's",
+                need, (size_t)eid::kStaticScratchBytes);
+  uint8_t *ws = nullptr;
+  const hipError_t e = eid::static_scratch(&ws);
+  if (e != hipSuccess) return hip_fail(e, "address of the static workspace");
+  eid_attn_args own = *args;
+  own.workspace = ws;
+  own.workspace_bytes = eid::kStaticScratchBytes;
+  return decode_launch(desc, &own, hip_stream, true);
 }
 
 int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {

@@ -21,6 +21,10 @@ constexpr int kDynPartitionCap = 2048;  // a workgroup streams serially: keep it
 constexpr int kDynPartitionFloor = 512; // smallest partition when the batch needs several fills
 constexpr int kShortSpanMax = 512;      // keys one workgroup of the short-span kernel covers
 constexpr int kPlanBytes = 256;         // head of the workspace: two {partition, items} slots
+// Size of the library's own split-KV workspace (a static device array, one copy per GPU),
+// which the decode entry point that allocates nothing uses in place of a caller's workspace.
+constexpr size_t kStaticScratchBytes = 32u << 20;
+constexpr int kStackPlanSeqs = 1024;    // sequences the host plans for without heap storage
 
 struct AttnParams {
   const uint16_t *q;

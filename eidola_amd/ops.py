@@ -316,7 +316,8 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
     need = lib.eid_workspace_bytes(C.byref(desc))
     if need == 0:
         check(getattr(lib, fn_name)(C.byref(desc), C.byref(AttnArgs()), None))
-    if workspace is None:
+    own_ws = fn_name == "eid_attn_decode_noalloc"   # the library's static array serves it
+    if workspace is None and not own_ws:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     args = AttnArgs()
     args.q = q.data_ptr()
@@ -330,8 +331,9 @@ def _attn_call(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seq
     args.sinks = sinks.data_ptr() if sinks is not None else None
     args.k_scale = k_scale.data_ptr() if k_scale is not None else None
     args.v_scale = v_scale.data_ptr() if v_scale is not None else None
-    args.workspace = workspace.data_ptr()
-    args.workspace_bytes = workspace.numel() * workspace.element_size()
+    if not own_ws:
+        args.workspace = workspace.data_ptr()
+        args.workspace_bytes = workspace.numel() * workspace.element_size()
     for name, t in (("k_new", k_new), ("v_new", v_new)):
         if t is not None:
             _require(t, name, torch.bfloat16, 3)
@@ -387,7 +389,8 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
         check(getattr(load_library(), fn_name)(C.byref(desc), C.byref(AttnArgs()), None))
     if out is None:
         out = torch.empty_like(q)
-    if workspace is None:
+    own_ws = fn_name == "eid_attn_decode_noalloc"   # the library's static array serves it
+    if workspace is None and not own_ws:
         workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
     args = AttnArgs()
     args.q, args.out = q.data_ptr(), out.data_ptr()
@@ -398,8 +401,9 @@ def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlen
     args.sinks = sinks.data_ptr() if sinks is not None else None
     args.k_scale = k_scale.data_ptr() if k_scale is not None else None
     args.v_scale = v_scale.data_ptr() if v_scale is not None else None
-    args.workspace = workspace.data_ptr()
-    args.workspace_bytes = workspace.numel()
+    if not own_ws:
+        args.workspace = workspace.data_ptr()
+        args.workspace_bytes = workspace.numel()
     args.k_new = k_new.data_ptr() if k_new is not None else None
     args.v_new = v_new.data_ptr() if v_new is not None else None
     S = seq_lens.shape[0]
@@ -430,6 +434,20 @@ def attn_decode(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len,
     return _attn_call("eid_attn_decode", geom, q, k_cache, v_cache, block_table, seq_lens, None,
                       1, max_kv_len, sinks, k_scale, v_scale, out, lse, workspace, return_lse,
                       sum_kv_len, k_new, v_new, seq_lens_host, None, block_table_host)
+
+
+def attn_decode_noalloc(geom, q, k_cache, v_cache, block_table, seq_lens, *, max_kv_len, out,
+                        sinks=None, k_scale=None, v_scale=None, lse=None, sum_kv_len=0,
+                        k_new=None, v_new=None, seq_lens_host=None, block_table_host=None):
+    """attn_decode through the entry point that allocates nothing: the split-KV partials go
+    to the library's static device array (batches whose workspace would exceed
+    STATIC_WORKSPACE_BYTES raise EID_ERR_WORKSPACE), and `out` must be given.  Calls on one
+    GPU share that array and must not overlap in time."""
+    if out is None:
+        raise ValueError("out must be given: this call allocates nothing")
+    return _attn_call("eid_attn_decode_noalloc", geom, q, k_cache, v_cache, block_table,
+                      seq_lens, None, 1, max_kv_len, sinks, k_scale, v_scale, out, lse, None,
+                      False, sum_kv_len, k_new, v_new, seq_lens_host, None, block_table_host)
 
 
 def attn_varlen(geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q, *, max_q_len,

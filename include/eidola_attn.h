@@ -177,6 +177,27 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args,
                         void *hip_stream);
 
 /*
+ * eid_attn_decode for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has NO counterpart in
+ * the reference (nor does anything else here) and exists for those callers only.
+ * Same arguments, same kernels and bit-identical results as eid_attn_decode, except that
+ * args->workspace / args->workspace_bytes are ignored: the split-KV partials go to a static
+ * device array of EID_STATIC_WORKSPACE_BYTES that the library holds on every GPU it runs on
+ * until the process ends.  The call allocates nothing, on the device or on the host (no
+ * hipMalloc / hipFree, no allocating library routine); the first call on a device looks the
+ * array's address up once.  A batch with eid_workspace_bytes(desc) above that size is
+ * rejected with EID_ERR_WORKSPACE (use eid_attn_decode with a workspace of your own); for
+ * batches of more than 1,024 sequences the host copies of the lengths are not used for
+ * planning.  All calls on one GPU share the one array: calls that overlap in time on the
+ * same GPU (two streams, two threads, two graphs in flight) race on it; serialise them, or
+ * give the others eid_attn_decode with their own workspace.  Nothing in the array has to
+ * start from a particular value, so it is never cleared.
+ */
+#define EID_STATIC_WORKSPACE_BYTES (32u << 20)
+int32_t eid_attn_decode_noalloc(const eid_attn_desc *desc, const eid_attn_args *args,
+                                void *hip_stream);
+
+/*
  * Stages K2/K3+K4 — ragged attention in cu_seqlens layout: chunked prefill, speculative
  * verify and mixed prefill+decode batches.  Query row i of sequence s sits at absolute
  * position seq_lens[s] - q_len_s + i and sees keys 0..position (clipped by `window`).

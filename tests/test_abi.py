@@ -127,6 +127,27 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     assert b"scale" in lib.eid_last_error()
 
 
+def test_noalloc_decode_validates_and_bounds_its_static_workspace_without_a_gpu():
+    lib = ea.load_library()
+    header = open(os.path.join(ROOT, "include", "eidola_attn.h")).read()
+    m = re.search(r"#define EID_STATIC_WORKSPACE_BYTES \((\d+)u << (\d+)\)", header)
+    assert int(m.group(1)) << int(m.group(2)) == ea.STATIC_WORKSPACE_BYTES
+    a = AttnArgs()
+    d = good_desc()
+    assert lib.eid_attn_decode_noalloc(C.byref(d), None, None) == _lib.EID_ERR_INVALID_ARG
+    assert lib.eid_attn_decode_noalloc(C.byref(d), C.byref(a), None) == _lib.EID_ERR_INVALID_ARG
+    for f in ("q", "out", "k_cache", "v_cache", "block_table", "seq_lens"):
+        setattr(a, f, 0x1000)
+    # a batch whose partials cannot fit the static array is turned away before any launch
+    big = ea.make_desc(ea.AttnGeometry(partition_size=128), num_seqs=512, num_q_tokens=512,
+                       max_q_len=1, max_kv_len=8192, max_blocks_per_seq=512, num_blocks=300000)
+    assert ea.workspace_bytes(big) > ea.STATIC_WORKSPACE_BYTES
+    assert lib.eid_attn_decode_noalloc(C.byref(big), C.byref(a), None) == _lib.EID_ERR_WORKSPACE
+    assert b"static" in lib.eid_last_error()
+    d5 = good_desc(num_q_tokens=20, max_q_len=5)
+    assert lib.eid_attn_decode_noalloc(C.byref(d5), C.byref(a), None) == _lib.EID_ERR_INVALID_ARG
+
+
 def test_kv_write_validation_without_a_gpu():
     lib = ea.load_library()
     d = good_desc()
