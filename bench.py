@@ -519,6 +519,54 @@ def stack_bench(torch, ea, synth, layers=36, fused_qkv=True):
     return [r]
 
 
+def overlap_bench(torch):
+    """How far matrix and vector instructions overlap on a gfx950 SIMD: the register-only
+    probe kernels of eidola_amd/csrc/probe_overlap.hip (one iteration = the 18 MFMAs and the
+    softmax vector work of one 16-row tile stage of the prefill kernel), one workgroup per CU.
+    Per mode and waves per SIMD: ns per iteration (HIP events), core cycles per iteration and
+    the core clock the waves saw (s_memtime against the 100 MHz s_memrealtime)."""
+    import ctypes as C
+    path = os.path.join(ROOT, "eidola_amd", "csrc", "libeid_probe.so")
+    lib = C.CDLL(path)
+    lib.eid_probe_overlap.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
+                                      C.c_void_p]
+    lib.eid_probe_overlap.restype = C.c_int
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    rounds = 8                      # workgroups per CU, resident one at a time (LDS-limited)
+    wgs = cus * rounds
+    out = torch.empty(wgs * 512, dtype=torch.float32, device="cuda:0")
+    clk = torch.zeros(wgs * 8 * 2, dtype=torch.int64, device="cuda:0")
+    iters = 4000
+    names = {0: "mfma_only", 1: "valu_only", 2: "phases", 3: "interleaved", 4: "role_split",
+             5: "mfma_only_32x32x16", 6: "interleaved_32x32x16"}
+    res = []
+    st = torch.cuda.current_stream().cuda_stream
+    for mode in (0, 1, 2, 3, 4, 5, 6):
+        for wps in ((2,) if mode == 4 else (1, 2)):
+            def run(i):
+                rc = lib.eid_probe_overlap(mode, wps, wgs, iters, out.data_ptr(), clk.data_ptr(), st)
+                assert rc == 0, rc
+            run(0)
+            ms = event_ms(run, 3, torch)
+            waves = wgs * (8 if (mode == 4 or wps == 2) else 4)
+            c = clk[:2 * waves].view(-1, 2).double()
+            cyc = c[:, 0].mean().item() / iters
+            mhz = (c[:, 0] / c[:, 1]).mean().item() * 100.0
+            r = {"config": f"overlap_probe_{names[mode]}_{wps}wps", "mode": names[mode],
+                 "waves_per_simd": wps, "ns_per_iter": ms * 1e6 / (iters * rounds), "cycles_per_iter": cyc,
+                 "core_mhz": mhz}
+            if mode == 4:
+                cm = clk[:2 * waves].view(wgs, 8, 2).double()
+                r["cycles_per_iter_mfma_waves"] = cm[:, :4, 0].mean().item() / iters
+                r["cycles_per_iter_valu_waves"] = cm[:, 4:, 0].mean().item() / iters
+            log(f"[bench] overlap probe {names[mode]:>22s}, {wps} wave(s)/SIMD: {r['ns_per_iter']:7.1f} ns "
+                f"= {cyc:7.1f} cycles per iteration at {mhz:6.0f} MHz"
+                + (f" (MFMA waves {r['cycles_per_iter_mfma_waves']:.1f}, vector waves "
+                   f"{r['cycles_per_iter_valu_waves']:.1f} cycles)" if mode == 4 else ""))
+            res.append(r)
+    return res
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -588,7 +636,7 @@ def main():
                     help="experiment: no host-side lengths for the library (desc.sum_kv_len = 0, no "
                          "seq_lens_host): the kernels size and plan the launch themselves")
     ap.add_argument("--only", default="",
-                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack "
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack,overlap "
                          "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
@@ -704,6 +752,8 @@ def main():
             extra.extend(prefill_bench(torch, ea, synth))
         if want("small"):
             extra.extend(small_batch_bench(torch, ea, synth))
+        if want("overlap"):
+            extra.extend(overlap_bench(torch))
         if want("stack"):
             extra.extend(stack_bench(torch, ea, synth, fused_qkv=False))
             extra.extend(stack_bench(torch, ea, synth))

@@ -18,6 +18,8 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <type_traits>
+#include <utility>
 
 namespace eid {
 
@@ -65,12 +67,15 @@ struct RowInfo {
 // of 16 slots (exactly what a lane group reads from a token row of the cache: full 128-byte
 // lines), and its 16 rows are the 16 query heads of the pair, row r belonging to head r / 8.
 // A row only attends to the slots of its own head: the others are masked on every chunk.
-template <int NT, int VROW = kVRowBytes, bool PRE = false, bool PAIR = false>
+//
+// QLDS (the prefill kernel without lse): the Q operands of row tile nt are read from the wave's
+// LDS copy (q_rd, see chunk_pipe) when the tile's turn comes, instead of being held in `qf`.
+template <int NT, int VROW = kVRowBytes, bool PRE = false, bool PAIR = false, bool QLDS = false>
 __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
-                                           const Frag8 (&qf)[NT][2], const RowInfo &ri,
+                                           const Frag8 (&qf_regs)[NT][2], const RowInfo &ri,
                                            const int tc, const bool need_mask, const float c2,
                                            float (&m)[NT], f32x4 (&lacc)[NT],
-                                           f32x4 (&acc)[NT][4]) {
+                                           f32x4 (&acc)[NT][4], const uint8_t *q_rd = nullptr) {
   const int g = (threadIdx.x & 63) >> 4;
   Frag8 ones;  // bf16 1.0 in every slot: a row of ones in place of V^T yields row sums of P
   ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
@@ -88,6 +93,14 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
     }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
+    Frag8 qf_nt[2];
+    if constexpr (QLDS) {
+      qf_nt[0].u = *(const u32x4 *)(q_rd + (2 * nt) * 1024);
+      qf_nt[1].u = *(const u32x4 *)(q_rd + (2 * nt + 1) * 1024);
+    } else {
+      qf_nt[0] = qf_regs[nt][0];
+      qf_nt[1] = qf_regs[nt][1];
+    }
     // S^T = K Q^T (raw scores, fp32); the prefill kernel raises its priority around MFMA
     // clusters so that the matrix pipe is fed first when both of a SIMD's waves are ready
     f32x4 S[4];
@@ -98,8 +111,8 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
     for (int b = 0; b < 4; ++b) {
       f32x4 z = {0.f, 0.f, 0.f, 0.f};
       if (PRE) z = f32x4{-base, -base, -base, -base};
-      z = mfma16x32(kf[b][0], qf[nt][0], z);
-      S[b] = mfma16x32(kf[b][1], qf[nt][1], z);
+      z = mfma16x32(kf[b][0], qf_nt[0], z);
+      S[b] = mfma16x32(kf[b][1], qf_nt[1], z);
     }
     if (NT == 4) __builtin_amdgcn_s_setprio(0);
     if constexpr (PAIR) {
@@ -208,6 +221,225 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
       for (int pr = 0; pr < 2; ++pr) acc[nt][mt] = mfma16x32(vf[mt][pr], pf[pr], acc[nt][mt]);
     if (NT == 4) __builtin_amdgcn_s_setprio(0);
   }
+}
+
+// Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(<N - 1>).
+template <int... Is, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+// ---------------------------------------------------------------------------------------
+// Software-pipelined form of chunk_step<4, VROW, PRE = true> for the chunks of the prefill
+// kernel that need no masking (all but the one or two at the diagonal and at a window's lower
+// edge).  Same arithmetic, same results bit for bit; what changes is the ORDER of the
+// instruction stream.
+//
+// A gfx950 SIMD issues matrix and vector instructions through one port: a wave's MFMA takes
+// one issue slot (4 cycles) and then keeps the matrix pipe busy for 16, during which three
+// more slots are free for vector instructions, but only if they come NEXT in some wave's
+// stream and do not depend on that MFMA.  Compiler-scheduled attention code runs the two
+// kinds of work one after the other (score MFMAs, then the softmax's vector instructions,
+// then the output MFMAs), and a second wave of the SIMD that happens to be in its vector
+// phase gets the port only while the first is not trying to issue an MFMA.  So the overlap
+// is written into the stream here.  With the four 16-row tiles nt = 0..3 of the wave:
+//   A(nt)  8 MFMAs   S(nt) = K Q(nt)^T - reference maximum (the accumulator's initial value)
+//   B(nt)  vector    lane-local maximum, exp2, conversion to bf16: P(nt)
+//   C(nt)  10 MFMAs  row sums and O(nt) += V^T P(nt)^T
+// the stream is  A(0) | B(0) + A(1) | B(1) + C(0), A(2) | B(2) + C(1), A(3) | B(3) + C(2) | C(3)
+// where "+" means: one MFMA, then the next few vector instructions, a scheduling barrier,
+// and so on, the vector work spread evenly over the stage's MFMAs.  A full stage has 18
+// MFMAs (288 cycles of the matrix pipe) and 8 max3 + 16 exp2 (two slots each) + 8 converts +
+// 4 moves = 52 slots of vector work on top of the MFMAs' own 18: both pipes are busy.
+//
+// The rescaling decision uses the lane's own 16 scores: the row maximum (four lanes) exceeds
+// the slack iff some lane's maximum does, so the two cross-lane exchanges per tile are only
+// executed on the few chunks where the reference maximum moves (and on a wave's first
+// pipelined chunk, `maybe_fresh`, where rows may not have a reference yet).
+//
+// The Q operands come from the wave's own LDS copy (q_rd: fragment (nt, half) at
+// (2 nt + half) * 1024 + lane * 16), read at the start of the stage that issues their MFMAs:
+// keeping all eight fragments in registers as well as two tiles' scores would not fit 256 VGPRs.
+// ---------------------------------------------------------------------------------------
+constexpr int kQFragBytes = 64 * 16;  // one Q fragment of a wave in LDS: 16 bytes per lane
+
+template <int I>
+using IC = std::integral_constant<int, I>;
+
+// Vector work of stage nt, in order: [Q read and accumulator seed of tile nt + 1] (PRE ops),
+// max3 tree (8), rescale check (1), then (exp2, exp2, convert) x 8.  Issue cycles: 4; exp2 8.
+// One mask op (skipped by a wave-uniform branch on most chunks) precedes the max tree.
+constexpr int pipe_op_cost(const int op, const int pre, const int nmask) {
+  if (op >= pre && op < pre + nmask) return 0;
+  const int e = op - (pre + nmask + 9);
+  return (e >= 0 && e % 3 != 2) ? 8 : 4;
+}
+constexpr int pipe_cost_before(const int op, const int pre, const int nmask) {
+  int c = 0;
+  for (int i = 0; i < op; ++i) c += pipe_op_cost(i, pre, nmask);
+  return c;
+}
+
+//
+// need_mask (wave-uniform): the chunk holds keys that some row must not see (the diagonal, a
+// window's lower edge, the end of the sequence): every score is compared with its row's
+// bounds before the maximum, as in chunk_step, and rows may stay without a reference maximum.
+template <int VROW>
+__device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile_stride,
+                                           const uint8_t *v_rd, const uint8_t *q_rd,
+                                           bool &maybe_fresh, float (&m)[4], f32x4 (&lacc)[4],
+                                           f32x4 (&acc)[4][4], const RowInfo &ri, const int tc,
+                                           const bool need_mask) {
+#define EID_SB() __builtin_amdgcn_sched_barrier(0)
+  Frag8 ones;
+  ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+  asm volatile("" : "+v"(ones.u));  // kept in registers (else rebuilt from constants at every use)
+  Frag8 kf[4][2], vf[4][2], qf[2][2];
+  f32x4 S[2][4], z[2];
+  Frag8 P[2][2];
+  auto read_q = [&](auto t_c) {
+    constexpr int t = t_c;
+    qf[t & 1][0].u = *(const u32x4 *)(q_rd + (2 * t) * kQFragBytes);
+    qf[t & 1][1].u = *(const u32x4 *)(q_rd + (2 * t + 1) * kQFragBytes);
+  };
+  auto build_z = [&](auto t_c) {  // -(reference maximum) of tile t; 0 for a row without one
+    constexpr int t = t_c;
+    const float nb = m[t] == kNegBig ? 0.f : -m[t];
+    z[t & 1] = f32x4{nb, nb, nb, nb};
+  };
+  // ---- operands of the chunk: K first (the first MFMAs wait for them), Q(0), Q(1), V^T ----
+#pragma unroll
+  for (int b = 0; b < 4; ++b) kf[b][0].u = *(const u32x4 *)(k_rd + b * k_tile_stride);
+  read_q(IC<0>{});
+#pragma unroll
+  for (int b = 0; b < 4; ++b) kf[b][1].u = *(const u32x4 *)(k_rd + b * k_tile_stride + 16);
+  read_q(IC<1>{});
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      const u32x2 a = lds_read_tr16(v_rd + (2 * pr) * (kBlock * VROW) + 32 * mt);
+      const u32x2 b2 = lds_read_tr16(v_rd + (2 * pr + 1) * (kBlock * VROW) + 32 * mt);
+      vf[mt][pr].w[0] = a[0];
+      vf[mt][pr].w[1] = a[1];
+      vf[mt][pr].w[2] = b2[0];
+      vf[mt][pr].w[3] = b2[1];
+    }
+  build_z(IC<0>{});
+  build_z(IC<1>{});
+  EID_SB();
+  // MFMA j of A(t): first the four token tiles' first halves, then their second halves
+  auto mfma_a = [&](auto t_c, auto j_c) {
+    constexpr int t = t_c, j = j_c, b = j & 3;
+    if constexpr (j < 4) S[t & 1][b] = mfma16x32(kf[b][0], qf[t & 1][0], z[t & 1]);
+    else S[t & 1][b] = mfma16x32(kf[b][1], qf[t & 1][1], S[t & 1][b]);
+  };
+  // MFMA j of C(t): row sums, then the four dim tiles, for token pair 0, then for pair 1
+  auto mfma_c = [&](auto t_c, auto j_c) {
+    constexpr int t = t_c, j = j_c, pr = j / 5, i = j % 5;
+    if constexpr (i == 0) lacc[t] = mfma16x32(ones, P[t & 1][pr], lacc[t]);
+    else acc[t][i - 1] = mfma16x32(vf[i - 1][pr], P[t & 1][pr], acc[t][i - 1]);
+  };
+  __builtin_amdgcn_s_setprio(1);
+  static_for<8>([&](auto j) {
+    mfma_a(IC<0>{}, j);
+    EID_SB();
+  });
+  // ---- stages ----
+  static_for<4>([&](auto nt_c) {
+    constexpr int nt = nt_c;
+    constexpr bool has_c = nt > 0, has_a = nt < 3;
+    constexpr int NM = (has_c ? 10 : 0) + (has_a ? 8 : 0);
+    constexpr int kPre = (nt == 1 || nt == 2) ? 2 : 0;  // read_q(nt + 1) and build_z(nt + 1)
+    constexpr int kMask = 1;
+    constexpr int NV = kPre + kMask + 9 + 24;
+    constexpr int total = pipe_cost_before(NV, kPre, kMask);
+    float mloc = 0.f;
+    f32x4(&Sx)[4] = S[nt & 1];
+    auto vop = [&](auto op_c) {
+      constexpr int op = op_c, o = op - kPre - kMask;
+      if constexpr (op < kPre) {
+        constexpr int t1 = nt + 1 < 4 ? nt + 1 : 0;  // (never reached for nt == 3)
+        if constexpr (op == 0) read_q(IC<t1>{});
+        else build_z(IC<t1>{});
+      } else if constexpr (op < kPre + kMask) {  // keys of the lane against the row's bounds
+        if (need_mask) {
+          int pos, lo;
+          ri.bounds(nt, pos, lo);
+          const int j0 = tc + 4 * ((threadIdx.x & 63) >> 4);
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int j = j0 + b * kBlock + r;
+              if (j < lo || j > pos) Sx[b][r] = -INFINITY;
+            }
+        }
+      } else if constexpr (o < 8) {  // max3 tree over the lane's 16 scores
+        if constexpr (o == 0) mloc = max3(Sx[0][0], Sx[0][1], Sx[0][2]);
+        else if constexpr (o == 7) mloc = max2(mloc, Sx[3][3]);
+        else mloc = max3(mloc, Sx[(2 * o + 1) >> 2][(2 * o + 1) & 3], Sx[(2 * o + 2) >> 2][(2 * o + 2) & 3]);
+      } else if constexpr (o == 8) {
+        // (rare) the reference maximum of some row has to move, exactly as in chunk_step
+        if (maybe_fresh || __any(mloc > kLazyLog2)) {
+          const bool fresh = m[nt] == kNegBig;
+          const float base = fresh ? 0.f : m[nt];
+          const float mrow = rowgroup_max(mloc);
+          const bool up = mrow > (fresh ? kNegBig : kLazyLog2);
+          if (__any(up)) {
+            const float shift = up ? mrow : 0.f;
+            const float m_new = up ? base + mrow : m[nt];
+            const float alpha = fast_exp2(m[nt] - m_new);
+            m[nt] = m_new;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) Sx[b][r] -= shift;
+          }
+        }
+      } else {
+        constexpr int e = o - 9, k = e / 3;  // convert k packs exp2 2k and 2k + 1
+        if constexpr (e % 3 != 2) {
+          constexpr int i = 2 * k + e % 3;
+          Sx[i >> 2][i & 3] = fast_exp2(Sx[i >> 2][i & 3]);
+        } else {
+          uint32_t w = pack_bf16(Sx[(2 * k) >> 2][(2 * k) & 3], Sx[(2 * k + 1) >> 2][(2 * k + 1) & 3]);
+          // (pinned here: the optimiser would otherwise sink the exponentials and the conversion
+          // to where P is used, behind the next stage's branch)
+          asm volatile("" : "+v"(w));
+          P[nt & 1][k >> 2].w[k & 3] = w;
+        }
+      }
+    };
+    // vector op `op` goes behind MFMA number (cycles of the ops before it) * NM / (all cycles)
+    static_for<NM>([&](auto s_c) {
+      constexpr int s = s_c;
+      if constexpr (has_c && s < 10) mfma_c(IC<nt - 1>{}, s_c);
+      else mfma_a(IC<nt + 1>{}, IC<(has_c ? s - 10 : s)>{});
+      static_for<NV>([&](auto op_c) {
+        constexpr int op = op_c;
+        if constexpr (pipe_cost_before(op, kPre, kMask) * NM / total == s) vop(op_c);
+      });
+      EID_SB();
+    });
+  });
+  static_for<10>([&](auto j) {
+    mfma_c(IC<3>{}, j);
+    EID_SB();
+  });
+  __builtin_amdgcn_s_setprio(0);
+  if (!need_mask) maybe_fresh = false;  // every row has seen 64 finite scores
+#undef EID_SB
 }
 
 // 16 bf16 values -> 16 fp8-e4m3fn bytes, RNE of x / scale (the arithmetic of kv_write_kernel)
@@ -1106,6 +1338,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   constexpr int kElt = FP8 ? 1 : 2;
   __shared__ __align__(16) uint8_t lds_k[2][kPfKTileBytes];  // double-buffered K tile
   __shared__ __align__(16) uint8_t lds_v[2][kPfVTileBytes];  // double-buffered V tile
+  // PRE: every wave's eight Q fragments, in fragment order (see chunk_pipe)
+  __shared__ __align__(16) uint8_t lds_q[PRE ? kPfWaves * 8 * kQFragBytes : 16];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
@@ -1162,6 +1396,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   RowInfo ri;
   const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
   load_q<NT, PRE>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri, c2);
+  uint8_t *q_lds = &lds_q[0] + (PRE ? wave * (8 * kQFragBytes) + lane * 16 : 0);
+  if constexpr (PRE) {  // (wave-private: no barrier, the reads wait for the wave's own stores)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) *(u32x4 *)(q_lds + (2 * nt + h) * kQFragBytes) = qf[nt][h].u;
+  }
+  bool maybe_fresh = true;
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
 #pragma unroll
@@ -1173,8 +1415,9 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   }
 
   // cooperative loader: thread -> (row of the 64-token chunk, 32-byte segment of the head row)
+  // (a wave loads one page of the chunk: its id is wave-uniform and travels in a scalar register)
   const int ld_row = tid >> 2, ld_seg = tid & 3;
-  const int ld_page = ld_row >> 4;
+  const int ld_page = wave;
   const uint32_t row_bytes = (uint32_t)Hkv * kHeadDim * kElt;
   const size_t page_bytes = (size_t)kBlock * row_bytes;
   const uint32_t gl_off = (uint32_t)(ld_row & 15) * row_bytes + (uint32_t)kvh * (kHeadDim * kElt) +
@@ -1186,11 +1429,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
 
   u32x4 kr[kElt], vr[kElt];
   auto fetch = [&](const int tc) {  // global -> registers for chunk starting at token tc
-    int ids[4];
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-      ids[b] = clamp_page(bt[min(tc / kBlock + b, nblk_total - 1)], p.last_block);
-    const int blk = ld_page == 0 ? ids[0] : ld_page == 1 ? ids[1] : ld_page == 2 ? ids[2] : ids[3];
+    const int blk = clamp_page(bt[min(tc / kBlock + ld_page, nblk_total - 1)], p.last_block);
 #pragma unroll
     for (int e = 0; e < kElt; ++e) {
       kr[e] = u32x4{0, 0, 0, 0};
@@ -1246,14 +1485,19 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     if (wave_active && tc <= pos_last && tc + kChunk > lo_first) {
       const uint8_t *kt = &lds_k[cur][0] + i16 * kPfKRowBytes + g * 32;
       const uint8_t *v_rd = &lds_v[cur][0] + (4 * g + (i16 >> 2)) * kPfVRowBytes + 8 * (i16 & 3);
-      Frag8 kf[4][2];
-#pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        kf[b][0].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes));
-        kf[b][1].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes) + 16);
-      }
       const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
-      chunk_step<NT, kPfVRowBytes, PRE>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
+      if constexpr (PRE) {
+        chunk_pipe<kPfVRowBytes>(kt, kBlock * kPfKRowBytes, v_rd, q_lds, maybe_fresh, m, lacc, acc, ri, tc,
+                                 need_mask);
+      } else {
+        Frag8 kf[4][2];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          kf[b][0].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes));
+          kf[b][1].u = *(const u32x4 *)(kt + b * (kBlock * kPfKRowBytes) + 16);
+        }
+        chunk_step<NT, kPfVRowBytes, false>(kf, v_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
+      }
     }
     if (has_next) stash(tc + kChunk, cur ^ 1);
     __syncthreads();
