@@ -538,10 +538,13 @@ def overlap_bench(torch):
     clk = torch.zeros(wgs * 8 * 2, dtype=torch.int64, device="cuda:0")
     iters = 4000
     names = {0: "mfma_only", 1: "valu_only", 2: "phases", 3: "interleaved", 4: "role_split",
-             5: "mfma_only_32x32x16", 6: "interleaved_32x32x16"}
+             5: "mfma_only_32x32x16", 6: "interleaved_32x32x16", 7: "tile_stage_32x32x16",
+             8: "tile_stage_branches", 9: "tile_stage_branches_lds", 10: "tile_stage_no_score_chain",
+             11: "tile_stage_scores_not_to_valu", 12: "tile_stage_p_not_to_mfma",
+             13: "tile_stage_scores_early", 14: "tile_stage_chain_3_apart", 15: "tile_stage_chain_first"}
     res = []
     st = torch.cuda.current_stream().cuda_stream
-    for mode in (0, 1, 2, 3, 4, 5, 6):
+    for mode in (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15):
         for wps in ((2,) if mode == 4 else (1, 2)):
             def run(i):
                 rc = lib.eid_probe_overlap(mode, wps, wgs, iters, out.data_ptr(), clk.data_ptr(), st)
