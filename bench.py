@@ -21,11 +21,15 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
-# HBM bytes per launch of the split-KV decode kernel on this exact seeded batch, from two
-# rocprofv3 --pmc passes over this script (FETCH_SIZE 241,250 KiB x 2.0, WRITE_SIZE 2,080 KiB
-# x 1.0; the factors are what the same counters read for a plain 1 GiB device copy run with
-# --calibrate-copy).  See profiles/splitkv_decode_config2.md.
-TRAFFIC_BYTES_PER_LAUNCH = int((241_250 * 2.0 + 2_080 * 1.0) * 1024)
+# HBM bytes per launch of the dominant kernel on the seeded configs[1] batch, by kernel name,
+# from two rocprofv3 --pmc passes over this script (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB; the
+# factors are what the same counters read for a plain 1 GiB device copy run with
+# --calibrate-copy).  See profiles/splitkv_decode_config2.md.  A kernel that is not listed
+# (or a non-default batch) reports traffic as null rather than another kernel's figure.
+TRAFFIC_BYTES_PER_LAUNCH = {
+    "splitkv_table_kernel<1,bf16,8 waves>": None,   # set from the profile of this tree, see below
+    "splitkv_kernel<1,bf16,8 waves>": int((241_250 * 2.0 + 2_080 * 1.0) * 1024),
+}
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "paged sink-attn decode HBM GB/s (% peak) + ragged-batch tokens/s, 1 GPU"
 
@@ -83,7 +87,7 @@ UNFUSED = False  # --unfused: decode steps as two launches (eid_kv_write, eid_at
 class Workload:
     """One configuration materialised on the GPU with `nsets` disjoint page sets."""
 
-    def __init__(self, make_batch, nsets, pool_seed, torch, ea, synth, kind):
+    def __init__(self, make_batch, nsets, pool_seed, torch, ea, synth, kind, pool=None):
         self.kind = kind  # "decode" or "varlen"
         dev = "cuda:0"
         b0 = make_batch(0)
@@ -91,14 +95,19 @@ class Workload:
         self.batches = [b0] + [make_batch(r * nblk) for r in range(1, nsets)]
         g = b0.geom
         self.geom = g
-        dt = torch.uint8 if g.kv_dtype == ea.KV_FP8_E4M3 else torch.bfloat16
-        self.k_cache = torch.empty((b0.num_blocks, 16, g.num_kv_heads, 64), dtype=dt, device=dev)
-        self.v_cache = torch.empty_like(self.k_cache)
-        t0 = time.time()
-        self.k_scale, self.v_scale = synth.fill_pool_gpu(g, self.k_cache, self.v_cache, pool_seed)
-        torch.cuda.synchronize()
-        log(f"[bench] {b0.name}: pool of {b0.num_blocks} blocks filled in {time.time()-t0:.1f}s, "
-            f"{nsets} page sets of {nblk} blocks")
+        if pool is not None:   # another workload's pool of the same dtype and size
+            self.k_cache, self.v_cache, self.k_scale, self.v_scale = pool
+            assert self.k_cache.shape[0] == b0.num_blocks
+        else:
+            dt = torch.uint8 if g.kv_dtype == ea.KV_FP8_E4M3 else torch.bfloat16
+            self.k_cache = torch.empty((b0.num_blocks, 16, g.num_kv_heads, 64), dtype=dt, device=dev)
+            self.v_cache = torch.empty_like(self.k_cache)
+            t0 = time.time()
+            self.k_scale, self.v_scale = synth.fill_pool_gpu(g, self.k_cache, self.v_cache, pool_seed)
+            torch.cuda.synchronize()
+            log(f"[bench] {b0.name}: pool of {b0.num_blocks} blocks filled in {time.time()-t0:.1f}s, "
+                f"{nsets} page sets of {nblk} blocks")
+        self.pool = (self.k_cache, self.v_cache, self.k_scale, self.v_scale)
         T = b0.num_q_tokens
 
         def bf16(bits):
@@ -228,6 +237,162 @@ def measure(w, steps, warmup, torch, synth, label):
         f"{100*r['attn_GBps']/HBM_PEAK_GBS:.1f}% HBM, {r['attn_TFLOPs']:.1f} TFLOP/s; "
         f"partition {r['partition']}")
     return r
+
+
+def subset(batch, idx, name, synth):
+    """The sequences `idx` of a batch as a batch of their own (same pages, same geometry)."""
+    import numpy as np
+    idx = np.asarray(idx)
+    return synth.Batch(name, batch.geom, batch.seq_lens[idx], batch.q_lens[idx],
+                       batch.block_table[idx], batch.num_blocks, batch.seed)
+
+
+def compact_pass(w, steps, warmup, torch):
+    """(ms per step, ms per attention call) of a workload: HIP events around `steps`
+    back-to-back steps / calls, page sets rotated."""
+    for i in range(warmup):
+        w.step(i)
+    ms_step = event_ms(w.step, steps, torch)
+    ms_attn = event_ms(lambda i: w.attn[i % w.n](), steps, torch)
+    return ms_step, ms_attn
+
+
+def parity_sample(w, seqs, torch, synth, what):
+    """Checker of the cpu_baseline leg: the attention output of page set 0 for the sequences
+    `seqs` against the CPU restatement's fp64 path on a compacted copy of their pages;
+    returns (max abs, mean abs) error."""
+    import numpy as np
+    import oracle
+    import eidola_amd as ea
+    b = w.batches[0]
+    seqs = [int(x) for x in seqs]
+    nblk = (b.seq_lens[seqs].astype(np.int64) + 15) // 16
+    pages = np.concatenate([b.block_table[s, :n] for s, n in zip(seqs, nblk)])
+    idx = torch.from_numpy(pages.astype(np.int64)).to("cuda:0")
+
+    def host(t):
+        t = t[idx].cpu().contiguous()
+        return t.numpy() if t.dtype == torch.uint8 else t.view(torch.int16).numpy().view(np.uint16)
+
+    kc, vc = host(w.k_cache), host(w.v_cache)
+    bt = np.zeros((len(seqs), int(nblk.max())), np.int32)
+    off = 0
+    for i, n in enumerate(nblk):
+        bt[i, :n] = np.arange(off, off + n)
+        off += int(n)
+    sub = synth.Batch(b.name + "_sample", b.geom, b.seq_lens[seqs], b.q_lens[seqs], bt, len(pages), b.seed)
+    d = ea.make_desc(sub.geom, num_seqs=sub.num_seqs, num_q_tokens=sub.num_q_tokens,
+                     max_q_len=sub.max_q_len, max_kv_len=sub.max_kv_len,
+                     max_blocks_per_seq=bt.shape[1], num_blocks=len(pages))
+    cu = b.cu_seqlens_q
+    rows = np.concatenate([np.arange(cu[s], cu[s + 1]) for s in seqs])
+    q = w.q.cpu().view(torch.int16).numpy().view(np.uint16)[rows]
+    ks = w.k_scale.cpu().numpy() if w.k_scale is not None else None
+    vs = w.v_scale.cpu().numpy() if w.v_scale is not None else None
+    ref, _ = oracle.attn_f64(d, q, kc, vc, bt, sub.seq_lens, sub.cu_seqlens_q, w.sinks.cpu().numpy(), ks, vs)
+    out = w.attn[0]()
+    torch.cuda.synchronize()
+    got = synth.bf16_bits_to_f32(out.cpu().view(torch.int16).numpy().view(np.uint16)[rows]).astype(np.float64)
+    err = np.abs(got - ref)
+    log(f"[bench] {what}: {len(seqs)} sampled sequences ({len(rows)} rows) vs the fp64 CPU restatement: "
+        f"max abs {err.max():.2e}, mean abs {err.mean():.2e}")
+    return {"max_abs": float(err.max()), "mean_abs": float(err.mean()), "rows": int(len(rows)),
+            "sequences": seqs}
+
+
+def other_configs(a, torch, ea, synth, pool2, check):
+    """Compact passes over the other BASELINE configurations: per (config, variant) the time of
+    the attention call, the algorithmic work and the roofline fraction it gives; with `check`,
+    sampled sequences against the CPU restatement (part of the cpu_baseline leg)."""
+    import numpy as np
+    steps, warm = max(10, a.steps // 8), max(3, a.warmup // 4)
+    out = {}
+
+    def hbm(work, ms, kernel, extra=None):
+        gbs = work["bytes"] / ms / 1e6
+        r = {"ms_call": ms, "alg_bytes": work["bytes"], "q_tokens": work["q_tokens"],
+             "roofline": {"bound": "hbm", "kernel": kernel, "achieved": gbs, "peak": HBM_PEAK_GBS,
+                          "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                          "how": "HIP events around back-to-back eid_attn_* calls (every launch of the "
+                                 "call), page sets rotated"}}
+        r.update(extra or {})
+        return r
+
+    # ---- 2b: decode, 128-token window (latency-bound: 17 MB of KV) ----
+    w = Workload(lambda off: synth.config2(window=128, perm_offset=off), a.sets, 7, torch, ea, synth,
+                 "decode", pool=pool2)
+    ms_step, ms_attn = compact_pass(w, steps * 2, warm, torch)
+    out["2b_window"] = hbm(synth.algorithmic_work(w.batches[0]), ms_attn, "shortspan_kernel<1,bf16>",
+                           {"ms_per_step": ms_step, "tokens_per_s": 64 / ms_step * 1e3,
+                            "note": "latency-bound: 17 MB of KV per call"})
+    if check:
+        order = np.argsort(w.batches[0].seq_lens)
+        out["2b_window"]["parity"] = parity_sample(w, [order[0], order[31], order[-1], 0, 1], torch, synth, "2b_window")
+    # ---- 3: mixed chunked prefill + decode; the two populations also on their own ----
+    full = lambda off: synth.config3(perm_offset=off)
+    w3 = Workload(full, 4, 8, torch, ea, synth, "varlen", pool=pool2)
+    ms_step, ms_attn = compact_pass(w3, steps, warm, torch)
+    b3 = w3.batches[0]
+    lw, sw = synth.algorithmic_work(b3, rows="long"), synth.algorithmic_work(b3, rows="short")
+    out["3_mixed"] = {"ms_call": ms_attn, "ms_per_step": ms_step, "q_tokens": b3.num_q_tokens,
+                      "tokens_per_s": b3.num_q_tokens / ms_step * 1e3,
+                      "prefill_TFLOPs_of_the_call": lw["flops"] / ms_attn / 1e9,
+                      "decode_GBps_of_the_call": sw["bytes"] / ms_attn / 1e6,
+                      "note": "prefill and split-KV launches run side by side (two streams)"}
+    if check:
+        lens8 = np.argsort(b3.seq_lens[:8])
+        out["3_mixed"]["parity"] = parity_sample(w3, [lens8[0], lens8[-1], 8, 9, 60, 127], torch, synth, "3_mixed")
+    wp = Workload(lambda off: subset(full(off), np.arange(8), "config3_prefill_rows", synth), 4, 8,
+                  torch, ea, synth, "varlen", pool=pool2)
+    _, ms_p = compact_pass(wp, steps, warm, torch)
+    tf = lw["flops"] / ms_p / 1e9
+    out["3_prefill"] = {"ms_call": ms_p, "alg_flops": lw["flops"], "q_tokens": lw["q_tokens"],
+                        "roofline": {"bound": "mfma", "kernel": "prefill_kernel<bf16, folded softmax factor>",
+                                     "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                                     "frac": tf / MFMA_BF16_PEAK_TFLOPS,
+                                     "how": "HIP events around back-to-back eid_attn_varlen calls on the 8 "
+                                            "prefill sequences alone"}}
+    wd = Workload(lambda off: subset(full(off), np.arange(8, 128), "config3_decode_rows", synth), 4, 8,
+                  torch, ea, synth, "varlen", pool=pool2)
+    _, ms_d = compact_pass(wd, steps, warm, torch)
+    out["3_decode"] = hbm(sw, ms_d, "splitkv_kernel<1,bf16,8 waves>")
+    w = w3 = wp = wd = None
+    # ---- 4: fp8 KV decode ----
+    w4 = Workload(lambda off: synth.config4(num_blocks=300_000, perm_offset=off), 3, 9, torch, ea,
+                  synth, "decode")
+    ms_step, ms_attn = compact_pass(w4, steps, warm, torch)
+    out["4_fp8"] = hbm(synth.algorithmic_work(w4.batches[0]), ms_attn,
+                       "splitkv_kernel<1,fp8,4 waves,head pairs>",
+                       {"ms_per_step": ms_step, "tokens_per_s": 256 / ms_step * 1e3})
+    if check:
+        order = np.argsort(w4.batches[0].seq_lens)
+        out["4_fp8"]["parity"] = parity_sample(w4, [order[0], order[127], order[-1], 0, 1], torch, synth, "4_fp8")
+    w4 = None
+    torch.cuda.empty_cache()
+    # ---- 5: speculative verify, 512-token partitions; layer 0 full, layer 1 windowed ----
+    pool5, t5 = None, 0.0
+    for layer, key in ((0, "5_full"), (1, "5_window")):
+        w5 = Workload(lambda off: synth.config5(layer=layer, num_blocks=900_000, perm_offset=off), 3,
+                      10, torch, ea, synth, "varlen", pool=pool5)
+        pool5 = w5.pool
+        ms_step, ms_attn = compact_pass(w5, max(5, steps // 2), warm, torch)
+        t5 += ms_step
+        out[key] = hbm(synth.algorithmic_work(w5.batches[0]), ms_attn,
+                       "splitkv_kernel<3,bf16,8 waves>" if layer == 0 else "shortspan_kernel<3,bf16>",
+                       {"ms_per_step": ms_step, "partition_size": 512})
+        if check:
+            order = np.argsort(w5.batches[0].seq_lens)
+            out[key]["parity"] = parity_sample(w5, [order[0], order[64], order[-1]], torch, synth, key)
+        w5 = None
+    out["5_full"]["tokens_per_s_both_layers"] = 640 / t5 * 1e3
+    for k, v in out.items():
+        rf = v.get("roofline")
+        if rf:
+            log(f"[bench] {k}: call {v['ms_call']*1e3:.1f} us, {rf['achieved']:.0f} {rf['unit']} = "
+                f"{100*rf['frac']:.1f}% of the {rf['bound']} peak")
+        else:
+            log(f"[bench] {k}: call {v['ms_call']*1e3:.1f} us, step {v['ms_per_step']*1e3:.1f} us")
+    return out
 
 
 def sched_bench(synth, ea, steps=200):
@@ -612,7 +777,17 @@ def cpu_baseline(w, torch, synth, threads):
     err = np.abs(synth.bf16_bits_to_f32(gpu).astype(np.float64)
                  - synth.bf16_bits_to_f32(out).astype(np.float64))
     work = synth.algorithmic_work(b)
+    model = ""
+    try:
+        for ln in open("/proc/cpuinfo"):
+            if ln.startswith("model name"):
+                model = ln.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
     return {"value": work["bytes"] / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "nproc": os.cpu_count(), "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
+            "cpu_model": model,
             "sample": f"{reps} full passes of the same 64-sequence decode batch "
                       f"({work['ctx_tokens']} context tokens), {dt:.3f} s each, {reps*dt:.1f} s in all; "
                       "CPU restatement of this repo (no reference CPU path exists)",
@@ -628,7 +803,10 @@ def main():
     ap.add_argument("--sets", type=int, default=8, help="disjoint page sets rotated between steps")
     ap.add_argument("--all", action="store_true", help="also measure the other configurations")
     ap.add_argument("--report", default=os.path.join(ROOT, "gpurun_out", "bench_all.jsonl"))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-cpu", action="store_true",
+                    help="skip the cpu_baseline leg (CPU timing and the sampled checks against it)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="measure configs[1] (full attention) only, not the other configurations")
     ap.add_argument("--partition", type=int, default=0)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run plain 1 GiB device copies (a kernel of known traffic, for "
@@ -664,6 +842,8 @@ def main():
     r = measure(w, a.steps, a.warmup, torch, synth, "config2_decode_full")
     split_ms = r["ms_split"]
     achieved = r["alg_bytes"] / split_ms / 1e6
+    kernel_name = ("splitkv_kernel<1,bf16,8 waves>" if a.no_hint or os.environ.get("EID_NO_ITEM_TABLE")
+                   else "splitkv_table_kernel<1,bf16,8 waves>")
     line = {
         "metric": METRIC, "value": r["step_GBps"], "unit": "GB/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"],
@@ -683,16 +863,18 @@ def main():
         "breakdown_us": {"kv_write": r["ms_kv_write"] * 1e3, "attn_call": r["ms_attn"] * 1e3,
                          "merge": r["ms_merge"] * 1e3,
                          "step_as_two_launches": r["ms_per_step_two_launches"] * 1e3},
-        "roofline": {"bound": "hbm", "kernel": ("splitkv_kernel<1,bf16,8 waves>" if a.no_hint or os.environ.get("EID_NO_ITEM_TABLE")
-                                else "splitkv_table_kernel<1,bf16,8 waves>"),
+        "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": TRAFFIC_BYTES_PER_LAUNCH if a.partition == 0 and not a.no_shuffle else None,
+                     "traffic": (TRAFFIC_BYTES_PER_LAUNCH.get(kernel_name)
+                                 if a.partition == 0 and not a.no_shuffle and not a.unfused else None),
                      "alg_bytes_per_launch": r["alg_bytes"], "launch_us": split_ms * 1e3,
                      "how": "HIP events inside full steps: before the eid_attn_decode call -> the "
                             "library's split_done_event (kernel plus the launch gap before it)"},
     }
     extra = [r]
+    if not a.headline_only:
+        line["configs"] = other_configs(a, torch, ea, synth, w.pool, check=not a.no_cpu)
     if a.calibrate_copy:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 255)
         dst = torch.empty_like(src)
