@@ -1037,6 +1037,8 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
     // workgroup w serves sequence w, found with scalar loads alone; sequences of another
     // q_len class leave at once.
     const SeqView v = view_seq(p, blockIdx.x);
+    // (every sequence one partition: a merge called by itself afterwards finds nothing to do)
+    if (p.plan_slot && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = 1 << 30;
     if (v.span <= 0) return;
     WorkItem it;
     it.seq = blockIdx.x;
@@ -1148,6 +1150,7 @@ __device__ __forceinline__ void shortspan_body(const AttnParams &p, const ItemTa
   int s = blockIdx.x, part = 0, nparts = 1, L, qlen, row0;
   if (p.nparts_max == 1) {
     const SeqView v = view_seq(p, s);
+    if (p.plan_slot && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) p.plan_slot[0] = 1 << 30;
     if (v.span <= 0) return;  // not of this class, or malformed: the whole workgroup leaves
     L = v.seq_len, qlen = v.qlen, row0 = v.row0;
   } else {
@@ -1164,6 +1167,8 @@ __device__ __forceinline__ void shortspan_body(const AttnParams &p, const ItemTa
     }
     s = it.seq, part = it.part, nparts = it.nparts;
     L = it.seq_len, qlen = it.qlen, row0 = it.row0;
+    // the partition this launch ran with, for a merge that is called by itself afterwards
+    if (p.plan_slot && blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) p.plan_slot[0] = kShortSpanMax;
   }
   const int pos0 = L - qlen;
   const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
@@ -1602,6 +1607,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (L < qlen) return;
   // run-time partition: recorded by the split-KV launch of this class; else the caller's
   const int P = p.plan_slot ? p.plan_slot[0] : p.partition;
+  if (P < 64 || (P & 63) != 0) return;  // (a slot no split-KV launch has written: nothing to merge)
   const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
   if (nparts <= 1) return;
 

@@ -294,6 +294,28 @@ struct Helper {
   hipStream_t stream = nullptr;
   hipEvent_t fork = nullptr, join = nullptr;
   bool tried = false, ok = false;
+  ~Helper() {  // the owning thread ends: give the stream and the events back
+    if (fork) (void)hipEventDestroy(fork);
+    if (join) (void)hipEventDestroy(join);
+    if (stream) (void)hipStreamDestroy(stream);
+  }
+};
+
+// Joins the helper stream back into the caller's stream when it goes out of scope, on error
+// returns as on success, so that no launch stays behind on the helper stream that the caller's
+// stream never waits for (under capture: no unjoined fork).
+struct HelperJoin {
+  Helper *hs = nullptr;
+  hipStream_t st = nullptr;
+  bool forked = false;
+  hipError_t join() {
+    if (!forked) return hipSuccess;
+    forked = false;
+    hipError_t e = hipEventRecord(hs->join, hs->stream);
+    if (e == hipSuccess) e = hipStreamWaitEvent(st, hs->join, 0);
+    return e;
+  }
+  ~HelperJoin() { (void)join(); }
 };
 Helper *helper_stream() {
   constexpr int kMaxDevices = 64;
@@ -325,6 +347,81 @@ bool use_shortspan(const eid_attn_desc *d, const Plan &pl, int ntiles) {
 
 int32_t hip_fail(hipError_t e, const char *what) {
   return fail(EID_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+// Whether work enqueued on `st` right now is being recorded into a HIP graph.  A plan made
+// from the caller's HOST copies of the lengths (exact grids, the partition size, the item
+// list passed by value) would be frozen into the graph and silently go stale when the device
+// arrays change between replays, so under capture the host copies are ignored and the
+// kernels plan from the device arrays, as they do without them.
+bool stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
+// ---- opt-in checks of what the library otherwise has to take on trust (EID_DEBUG=1) -----
+// The host copies of the length arrays and of the block table must equal the device arrays,
+// and desc.sum_kv_len must not be below the true sum: a mismatch makes the kernels drop or
+// misplace work without any error.  With EID_DEBUG set in the environment the attention entry
+// points copy the device arrays back (after waiting for the stream) and compare.  Slow, and
+// not possible on a capturing stream; meant for bring-up of an engine's scheduler.
+bool debug_checks_on() {
+  static const bool on = getenv("EID_DEBUG") != nullptr;
+  return on;
+}
+
+int32_t debug_check_host_copies(const eid_attn_desc *d, const eid_attn_args *a, bool decode,
+                                hipStream_t st) {
+  hipError_t e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return hip_fail(e, "EID_DEBUG: stream synchronize");
+  try {
+    const size_t S = (size_t)d->num_seqs;
+    std::vector<int32_t> lens(S);
+    e = hipMemcpy(lens.data(), a->seq_lens, S * sizeof(int32_t), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(e, "EID_DEBUG: copy of seq_lens");
+    long long sum = 0;
+    for (size_t s = 0; s < S; ++s) {
+      sum += lens[s];
+      if (lens[s] > d->max_kv_len)
+        return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: seq_lens[%zu] = %d exceeds desc.max_kv_len %d", s,
+                    lens[s], d->max_kv_len);
+      if (a->seq_lens_host && a->seq_lens_host[s] != lens[s])
+        return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: seq_lens_host[%zu] = %d, device holds %d", s,
+                    a->seq_lens_host[s], lens[s]);
+    }
+    if (d->sum_kv_len != 0 && d->sum_kv_len < sum)
+      return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: desc.sum_kv_len %lld is below the sum of seq_lens %lld",
+                  (long long)d->sum_kv_len, sum);
+    if (!decode && a->cu_seqlens_q_host) {
+      std::vector<int32_t> cu(S + 1);
+      e = hipMemcpy(cu.data(), a->cu_seqlens_q, (S + 1) * sizeof(int32_t), hipMemcpyDeviceToHost);
+      if (e != hipSuccess) return hip_fail(e, "EID_DEBUG: copy of cu_seqlens_q");
+      for (size_t s = 0; s <= S; ++s)
+        if (a->cu_seqlens_q_host[s] != cu[s])
+          return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: cu_seqlens_q_host[%zu] = %d, device holds %d", s,
+                      a->cu_seqlens_q_host[s], cu[s]);
+    }
+    if (decode && a->block_table_host) {
+      const size_t mb = (size_t)d->max_blocks_per_seq;
+      std::vector<int32_t> bt(S * mb);
+      e = hipMemcpy(bt.data(), a->block_table, S * mb * sizeof(int32_t), hipMemcpyDeviceToHost);
+      if (e != hipSuccess) return hip_fail(e, "EID_DEBUG: copy of block_table");
+      for (size_t s = 0; s < S; ++s) {
+        const size_t used = ((size_t)std::max(lens[s], 0) + eid::kBlock - 1) / eid::kBlock;
+        for (size_t j = 0; j < used && j < mb; ++j)
+          if (a->block_table_host[s * mb + j] != bt[s * mb + j])
+            return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: block_table_host[%zu][%zu] = %d, device holds %d",
+                        s, j, a->block_table_host[s * mb + j], bt[s * mb + j]);
+      }
+    }
+  } catch (...) {
+    return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: out of host memory");
+  }
+  return EID_OK;
 }
 
 // ---- launch planning from the caller's host copies of seq_lens / cu_seqlens_q ----------
@@ -416,7 +513,8 @@ struct ClassPlan {
 // storage are then left to the kernels' own planning.
 ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan &pl,
                      eid::AttnParams &p, int ntiles, int32_t qlen_lo, int32_t qlen_hi,
-                     bool decode, eid::ItemTable *table = nullptr, bool no_heap = false) {
+                     bool decode, eid::ItemTable *table = nullptr, bool no_heap = false,
+                     bool capturing = false) {
   ClassPlan cp;
   if (table) table->n = table->has_blk = 0;
   const bool fp8 = d->kv_dtype == EID_KV_FP8_E4M3;
@@ -430,7 +528,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   cp.merge = pl.nparts_max > 1;
   constexpr int32_t kHostPlanMaxSeqs = 8192;  // beyond that the host pass is no longer free
   const int32_t *cu = decode ? nullptr : a->cu_seqlens_q_host;
-  if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs) return cp;
+  if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) return cp;
   int32_t stack_store[3 * eid::kStackPlanSeqs];  // 12 KiB: most batches need no heap at all
   std::vector<int32_t> heap_store;
   int32_t *store = stack_store;
@@ -523,6 +621,23 @@ int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v
     return fail(EID_ERR_INVALID_ARG, "k_new, v_new, k_cache and v_cache must be 16-byte aligned");
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
   if (fp8 && (!k_scale || !v_scale)) return fail(EID_ERR_INVALID_ARG, "fp8 KV needs k_scale and v_scale");
+  if (debug_checks_on() && !stream_is_capturing(static_cast<hipStream_t>(hip_stream))) {
+    // duplicate slots in one call are undefined behaviour (two rows race for one cache row)
+    hipError_t de = hipStreamSynchronize(static_cast<hipStream_t>(hip_stream));
+    if (de != hipSuccess) return hip_fail(de, "EID_DEBUG: stream synchronize");
+    try {
+      std::vector<int64_t> slots((size_t)num_tokens);
+      de = hipMemcpy(slots.data(), slot_mapping, slots.size() * sizeof(int64_t), hipMemcpyDeviceToHost);
+      if (de != hipSuccess) return hip_fail(de, "EID_DEBUG: copy of slot_mapping");
+      std::sort(slots.begin(), slots.end());
+      for (size_t i = 1; i < slots.size(); ++i)
+        if (slots[i] >= 0 && slots[i] == slots[i - 1])
+          return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: slot %lld appears more than once in slot_mapping",
+                      (long long)slots[i]);
+    } catch (...) {
+      return fail(EID_ERR_INVALID_ARG, "EID_DEBUG: out of host memory");
+    }
+  }
   hipError_t e = eid::launch_kv_write(
       static_cast<const uint16_t *>(k_new), static_cast<const uint16_t *>(v_new),
       static_cast<uint8_t *>(k_cache), static_cast<uint8_t *>(v_cache), slot_mapping, k_scale,
@@ -632,16 +747,21 @@ static int32_t decode_launch(const eid_attn_desc *desc, const eid_attn_args *arg
   p.v_new = static_cast<const uint16_t *>(args->v_new);
   hipStream_t st = static_cast<hipStream_t>(hip_stream);
   const bool fp8 = desc->kv_dtype == EID_KV_FP8_E4M3;
+  const bool capturing = stream_is_capturing(st);
+  if (debug_checks_on() && !capturing && !no_heap)
+    if (int32_t rc = debug_check_host_copies(desc, args, true, st)) return rc;
   p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   eid::ItemTable table;  // (8 KiB on the stack; only `n` entries are ever read)
-  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table, no_heap);
+  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table, no_heap, capturing);
   if (cp.skip) return EID_OK;  // (every sequence empty or malformed: nothing is written)
   const eid::ItemTable *tab = table.n > 0 ? &table : nullptr;
   // spans of at most 8 chunks, or a small batch in partitions of that size: one workgroup
   // per (sequence, partition, KV head), a chunk per wave
+  if (cp.short_span) p.plan_slot = plan_slots;  // (the kernel records its partition there)
   hipError_t e = cp.short_span ? eid::launch_shortspan(p, 1, fp8, st, tab)
                                : eid::launch_splitkv(p, 1, fp8, plan_slots, st, tab);
+  if (cp.short_span) p.plan_slot = nullptr;     // (the merge of this call takes p.partition)
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (args->split_done_event) {
     e = hipEventRecord(static_cast<hipEvent_t>(args->split_done_event), st);
@@ -701,6 +821,9 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   // has max_q_len query rows (num_q_tokens says so) the host knows the one class that is
   // populated and launches nothing for the others.
   const bool uniform = (int64_t)desc->num_seqs * desc->max_q_len == desc->num_q_tokens;
+  const bool capturing = stream_is_capturing(st);
+  if (debug_checks_on() && !capturing)
+    if (int32_t rc = debug_check_host_copies(desc, args, false, st)) return rc;
   const int32_t qmax = short_q_max(desc);
   const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= qmax;
   const bool only_prefill = uniform && desc->max_q_len > qmax;
@@ -708,8 +831,10 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   auto launch_split = [&](const ClassPlan &cp, const int ntiles, int32_t *slot) {
     if (!cp.short_span) return eid::launch_splitkv(p, ntiles, fp8, slot, st);
     p.plan = nullptr;  // the short-span kernel works with the host's partition
-    p.plan_slot = nullptr;
-    return eid::launch_shortspan(p, ntiles, fp8, st);
+    p.plan_slot = slot;  // ... and records it for a merge called by itself afterwards
+    const hipError_t es = eid::launch_shortspan(p, ntiles, fp8, st);
+    p.plan_slot = nullptr;  // (the merge of this call takes p.partition)
+    return es;
   };
   // Mixed batch: the MFMA-bound prefill launch and the HBM-bound split-KV launches use
   // different halves of the machine, so they run side by side: prefill on the thread's
@@ -719,17 +844,21 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   Helper *hs = (has_prefill && !only_prefill && !serial) ? helper_stream() : nullptr;
   p.share_cus = hs ? 1 : 0;
   p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
+  HelperJoin joiner;
   if (hs) {
     e = hipEventRecord(hs->fork, st);
     if (e == hipSuccess) e = hipStreamWaitEvent(hs->stream, hs->fork, 0);
     if (e != hipSuccess) return hip_fail(e, "fork to the helper stream");
+    joiner.hs = hs;
+    joiner.st = st;
+    joiner.forked = true;
   }
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
   ClassPlan cp1;
   cp1.skip = true;
   if (!only_verify && !only_prefill) {
-    cp1 = plan_class(desc, args, pl, p, 1, 1, 2, false);
+    cp1 = plan_class(desc, args, pl, p, 1, 1, 2, false, nullptr, false, capturing);
     if (!cp1.skip) {
       e = launch_split(cp1, 1, plan_slots);
       if (e != hipSuccess) return hip_fail(e, "split-KV launch");
@@ -740,7 +869,6 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     pp.qlen_lo = qmax + 1;
     pp.qlen_hi = 0x7fffffff;
     e = eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream);
-    if (e == hipSuccess) e = hipEventRecord(hs->join, hs->stream);
     if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
   }
   if (args->split_done_event) {
@@ -753,7 +881,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   }
   if (desc->max_q_len > 2 && !only_prefill) {  // q_len 3..6: three tiles
     const int vt = verify_tiles(desc);
-    const ClassPlan cp3 = plan_class(desc, args, pl, p, vt, 3, qmax, false);
+    const ClassPlan cp3 = plan_class(desc, args, pl, p, vt, 3, qmax, false, nullptr, false, capturing);
     if (!cp3.skip) {
       e = launch_split(cp3, vt, plan_slots + 2);
       if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");
@@ -764,7 +892,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     }
   }
   if (hs) {
-    e = hipStreamWaitEvent(st, hs->join, 0);
+    e = joiner.join();
     if (e != hipSuccess) return hip_fail(e, "join of the helper stream");
   } else if (has_prefill) {  // long chunks: MFMA prefill kernel
     p.qlen_lo = qmax + 1;

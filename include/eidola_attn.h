@@ -11,14 +11,25 @@
  * bind it.
  *
  * Conventions
- *  - All tensor pointers are DEVICE pointers owned by the caller.  The library
- *    allocates nothing and keeps no global mutable state except a thread-local
- *    error string.
+ *  - All tensor pointers are DEVICE pointers owned by the caller; the library allocates
+ *    no device memory.  State it keeps: a thread-local error string; per process, cached
+ *    read-only facts about the device (CU count, the kernels' register and LDS footprints),
+ *    queried on first use; per calling thread and device, one helper stream and two events,
+ *    created by the thread's first mixed prefill + decode call of eid_attn_varlen and
+ *    destroyed when the thread ends; per device, the static workspace of
+ *    eid_attn_decode_noalloc.
  *  - All work is enqueued asynchronously on the caller's `hipStream_t`
  *    (passed as `void *`; NULL = the default stream).
  *  - Every function returns an `eid_status` (0 = OK, negative = error) and never
- *    throws or aborts.  Argument validation runs before the first HIP call, so
- *    invalid-argument paths can be exercised on a host without a GPU.
+ *    throws or aborts.  Argument validation needs no GPU: invalid-argument paths can be
+ *    exercised on a host without one.  Planning (eid_workspace_bytes, eid_partition_size)
+ *    asks the runtime for the device's CU count; without a device it assumes 256, the
+ *    MI355X's, so the sizes computed on a GPU-less host are the ones the GPU box uses.
+ *  - HIP graphs: every entry point may be called on a capturing stream (kernels and event
+ *    nodes only).  A captured call serves later replays with other device-side seq_lens /
+ *    block_table contents as long as the descriptor's max_kv_len and sum_kv_len bound them.
+ *    The optional HOST copies of those arrays are ignored while the stream is capturing: a
+ *    plan made from them would be frozen into the graph.
  *
  * Geometry supported by this version: head_dim 64, block_size 16,
  * num_q_heads = 8 * num_kv_heads (GQA 8:1), bf16 Q/out, bf16 or fp8-e4m3fn KV.
@@ -123,8 +134,10 @@ typedef struct eid_attn_args {
                            scheduler builds these arrays on the host anyway; with them the
                            library plans the launches itself (partition size, exact grids,
                            which kernels have work at all) instead of leaving that to every
-                           workgroup of the kernels.  They must equal the device arrays;
-                           results do not depend on whether they are given. */
+                           workgroup of the kernels.  They must equal the device arrays
+                           (EID_DEBUG=1 in the environment makes the call verify that, with a
+                           device synchronisation); results do not depend on whether they are
+                           given.  Ignored on a capturing stream (see "HIP graphs" above). */
   const int32_t *block_table_host;  /* optional HOST copy of block_table (same shape), used by
                            eid_attn_decode together with seq_lens_host: the page ids of every
                            work item's first chunk then travel with the launch instead of
