@@ -872,8 +872,55 @@ def test_config3_mixed_full_size(G):
                         sinks=G.dev(sinks), sum_kv_len=int(b.seq_lens.sum()))
     torch.cuda.synchronize()
     assert torch.equal(oh, out)
-    pre = int(np.argmin(b.seq_lens[:8]))
-    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [pre, 8, 9, 60, 127], "config3")
+    # all eight prefill chunks (the longest walks 70 chunks of keys) and ten decode rows,
+    # among them the shortest and the longest context
+    dec = 8 + np.argsort(b.seq_lens[8:])
+    seqs = list(range(8)) + [int(dec[0]), int(dec[-1]), int(dec[60])] + [8, 9, 33, 60, 90, 111, 127]
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, sorted(set(seqs)), "config3")
+    # with the scheduler's host copies of the lengths (the way bench.py calls it): same plan
+    # for the prefill rows, host-planned launches for the decode rows
+    oh = ea.attn_varlen(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                        G.dev(b.cu_seqlens_q), max_q_len=512, max_kv_len=b.max_kv_len,
+                        sinks=G.dev(sinks), sum_kv_len=int(b.seq_lens.sum()),
+                        seq_lens_host=b.seq_lens, cu_seqlens_q_host=b.cu_seqlens_q)
+    torch.cuda.synchronize()
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, oh, [0, 7, int(dec[-1]), 8, 127], "config3, host lengths")
+
+
+def test_config2_as_bench_times_it(G):
+    """Exactly the call bench.py's headline times, at full size: ONE eid_attn_decode that is
+    handed the 64 new K/V rows (fused write), the host copies of seq_lens and the block table
+    and their sum, on a page set other than the first of the 300k-block pool.  Sampled
+    sequences against the fp64 oracle, and every written cache row bit for bit."""
+    b0 = synth.config2()
+    nblk = int(((b0.seq_lens.astype(np.int64) + 15) // 16).sum())
+    b = synth.config2(perm_offset=3 * nblk)              # page set 3
+    assert not np.array_equal(b.block_table, b0.block_table)
+    q_d, kc_d, vc_d, sinks, _, _ = _gpu_inputs(G, b)
+    k_new = synth.normal_bf16((64, 8, 64), b.seed, synth.TID_K)
+    v_new = synth.normal_bf16((64, 8, 64), b.seed, synth.TID_V)
+    flat_k, flat_v = kc_d.view(-1, 8, 64), vc_d.view(-1, 8, 64)
+    slots = torch.from_numpy(b.slot_mapping).to(G.DEV)
+    flat_k[slots] = float("nan")                          # the call has to write these itself
+    flat_v[slots] = float("nan")
+    out = ea.attn_decode(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                         max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
+                         sum_kv_len=int(b.seq_lens.sum()), k_new=G.bf16_dev(k_new),
+                         v_new=G.bf16_dev(v_new), seq_lens_host=b.seq_lens,
+                         block_table_host=b.block_table)
+    torch.cuda.synchronize()
+    assert np.array_equal(G.bits_host(flat_k[slots]), k_new)
+    assert np.array_equal(G.bits_host(flat_v[slots]), v_new)
+    order = np.argsort(b.seq_lens)
+    seqs = sorted(set([int(order[0]), int(order[1]), int(order[31]), int(order[-1]), int(order[-2])]
+                      + list(range(0, 64, 9))))
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, seqs, "config2 as bench.py times it")
+    # the same call as two launches gives the same bits
+    out2 = ea.attn_decode(b.geom, q_d, kc_d, vc_d, G.dev(b.block_table), G.dev(b.seq_lens),
+                          max_kv_len=b.max_kv_len, sinks=G.dev(sinks))
+    torch.cuda.synchronize()
+    assert np.abs(synth.bf16_bits_to_f32(G.bits_host(out2)).astype(np.float64)
+                  - synth.bf16_bits_to_f32(G.bits_host(out)).astype(np.float64)).max() <= 4e-3
 
 
 def test_config4_fp8_full_size(G):

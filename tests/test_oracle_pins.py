@@ -65,14 +65,12 @@ def test_fp8_encode_known_answers():
 
 
 def test_fp8_encode_exhaustive_over_bf16_against_search_encoder():
-    """All finite bf16 inputs (the only values kv_write ever quantises), strided scales."""
+    """ALL finite bf16 inputs (the only values kv_write ever quantises, 65,280 of them) against
+    the exhaustive-search encoder; their quotients by three other scales on a stride."""
     all_bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
     x = synth.bf16_bits_to_f32(all_bits)
-    sel = np.isfinite(x)
-    # coarse stride over the whole range + every value within the e4m3 dynamic range
-    dense = sel & (np.abs(x) <= 600) & (np.abs(x) >= 2.0 ** -12)
-    pick = np.flatnonzero(dense)[::7].tolist() + np.flatnonzero(sel)[::211].tolist()
-    xs = x[np.array(sorted(set(pick)))]
+    xs = x[np.isfinite(x)]
+    assert len(xs) == 65280
     got = oracle.fp8_encode(xs)
     want = oracle_np.fp8_e4m3_encode_np(xs)
     assert np.array_equal(got, want)
@@ -80,6 +78,9 @@ def test_fp8_encode_exhaustive_over_bf16_against_search_encoder():
     inr = np.abs(xs) <= 448
     t = torch.from_numpy(xs[inr].copy()).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
     assert np.array_equal(got[inr], t)
+    for scale in (np.float32(0.0078125), np.float32(0.0123), np.float32(3.7)):
+        ys = (xs[::13] / scale).astype(np.float32)          # IEEE fp32 division, as kv_write does
+        assert np.array_equal(oracle.fp8_encode(ys), oracle_np.fp8_e4m3_encode_np(ys))
 
 
 # ---------------------------------------------------------------- K1
