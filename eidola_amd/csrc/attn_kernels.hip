@@ -18,6 +18,7 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <algorithm>
 #include <type_traits>
 #include <utility>
 
@@ -1338,7 +1339,8 @@ __device__ __forceinline__ bool find_prefill_item(const AttnParams &p, const int
 // operands, which costs one more bf16 rounding of Q (lse would be off by up to ~5e-3, the
 // outputs stay within a bf16 ulp of the unfolded path) and saves the FMA per score.
 template <bool FP8, bool PRE>
-__global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnParams p) {
+__global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnParams p,
+                                                                   const PfTable tab) {
   constexpr int NT = 4;
   constexpr int kElt = FP8 ? 1 : 2;
   __shared__ __align__(16) uint8_t lds_k[2][kPfKTileBytes];  // double-buffered K tile
@@ -1355,27 +1357,42 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int KS = p.pf_splits;
   const int unit = blockIdx.x / Hkv;
   const int ks_part = KS > 1 ? unit % KS : 0;
-  // one wave looks the item up, the others receive it through LDS
-  __shared__ int item_lds[8];
-  if (wave == 0) {
-    int s0 = 0, tile0 = 0, row00 = 0, qlen0 = 0, L0 = 0;
-    const bool found = find_prefill_item(p, KS > 1 ? unit / KS : unit, s0, tile0, row00, qlen0, L0);
-    if (lane == 0) {
-      item_lds[0] = found;
-      item_lds[1] = s0;
-      item_lds[2] = tile0;
-      item_lds[3] = row00;
-      item_lds[4] = qlen0;
-      item_lds[5] = L0;
+  int s, tile, row0, qlen, L;
+  if (tab.n > 0) {
+    // the host listed the tiles: scalar loads alone (lengths still come from the device arrays)
+    const int item = KS > 1 ? unit / KS : unit;
+    if (item >= tab.n) return;
+    const uint32_t e = tab.e[item];
+    s = (int)(e & 0xffffu);
+    tile = (int)(e >> 16);
+    const const_i32_ptr cu = as_constant(p.cu_seqlens_q), sl = as_constant(p.seq_lens);
+    row0 = cu[s];
+    qlen = cu[s + 1] - row0;
+    L = min(sl[s], p.max_blocks_per_seq * kBlock);
+    if (qlen < p.qlen_lo || qlen > p.qlen_hi || L < qlen || tile * kPfTok >= qlen) return;
+  } else {
+    // one wave looks the item up, the others receive it through LDS
+    __shared__ int item_lds[8];
+    if (wave == 0) {
+      int s0 = 0, tile0 = 0, row00 = 0, qlen0 = 0, L0 = 0;
+      const bool found = find_prefill_item(p, KS > 1 ? unit / KS : unit, s0, tile0, row00, qlen0, L0);
+      if (lane == 0) {
+        item_lds[0] = found;
+        item_lds[1] = s0;
+        item_lds[2] = tile0;
+        item_lds[3] = row00;
+        item_lds[4] = qlen0;
+        item_lds[5] = L0;
+      }
     }
+    __syncthreads();
+    if (!__builtin_amdgcn_readfirstlane(item_lds[0])) return;
+    s = __builtin_amdgcn_readfirstlane(item_lds[1]);
+    tile = __builtin_amdgcn_readfirstlane(item_lds[2]);
+    row0 = __builtin_amdgcn_readfirstlane(item_lds[3]);
+    qlen = __builtin_amdgcn_readfirstlane(item_lds[4]);
+    L = __builtin_amdgcn_readfirstlane(item_lds[5]);
   }
-  __syncthreads();
-  if (!__builtin_amdgcn_readfirstlane(item_lds[0])) return;
-  const int s = __builtin_amdgcn_readfirstlane(item_lds[1]);
-  const int tile = __builtin_amdgcn_readfirstlane(item_lds[2]);
-  const int row0 = __builtin_amdgcn_readfirstlane(item_lds[3]);
-  const int qlen = __builtin_amdgcn_readfirstlane(item_lds[4]);
-  const int L = __builtin_amdgcn_readfirstlane(item_lds[5]);
 
   const int W = p.window;
   const int pos0 = L - qlen;
@@ -2036,16 +2053,52 @@ long long prefill_tiles_bound(int num_q_tokens, int num_seqs) {
   return (long long)num_q_tokens / kPfTok + num_seqs;
 }
 
-hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st) {
-  const long long items = prefill_tiles_bound(num_q_tokens, p.num_seqs) * max(1, p.pf_splits);
+// Lists the query tiles of the launch's class from the host's copies of the lengths, most key
+// chunks first (ties in sequence order, later tiles first).  False (tab->n = 0) when the list
+// does not fit or an index does not fit its field: the kernel then scans on the device.
+bool build_prefill_table(const AttnParams &p, const int32_t *seq_lens_host,
+                         const int32_t *cu_seqlens_q_host, PfTable *tab) {
+  tab->n = 0;
+  if (p.num_seqs > 0xffff) return false;
+  struct Item { int32_t chunks; uint32_t e; };
+  Item items[kPfTableMax];
+  int n = 0;
+  for (int s = 0; s < p.num_seqs; ++s) {
+    const int qlen = cu_seqlens_q_host[s + 1] - cu_seqlens_q_host[s];
+    const int L = (int)std::min<long long>(seq_lens_host[s], (long long)p.max_blocks_per_seq * kBlock);
+    if (qlen < p.qlen_lo || qlen > p.qlen_hi || L < qlen) continue;
+    const int tiles = (qlen + kPfTok - 1) / kPfTok;
+    if (tiles > 0xffff || n + tiles > kPfTableMax) return false;
+    const int pos0 = L - qlen;
+    for (int t = tiles - 1; t >= 0; --t) {
+      const int first = pos0 + t * kPfTok, last = pos0 + std::min((t + 1) * kPfTok, qlen) - 1;
+      const int begin = (p.window > 0 ? std::max(0, first - p.window + 1) : 0) & ~(kBlock - 1);
+      items[n].chunks = (last + 1 - begin + kChunk - 1) / kChunk;
+      items[n].e = (uint32_t)s | (uint32_t)t << 16;
+      ++n;
+    }
+  }
+  std::stable_sort(items, items + n, [](const Item &a, const Item &b) { return a.chunks > b.chunks; });
+  for (int i = 0; i < n; ++i) tab->e[i] = items[i].e;
+  tab->n = n;
+  return n > 0;
+}
+
+hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
+                          const PfTable *tab) {
+  static const PfTable none{};  // n == 0: items found on the device
+  const bool listed = tab && tab->n > 0;
+  const long long items = (listed ? tab->n : prefill_tiles_bound(num_q_tokens, p.num_seqs)) *
+                          (long long)max(1, p.pf_splits);
   dim3 grid((unsigned)(items * p.num_kv_heads));
+  const PfTable &t = listed ? *tab : none;
   const bool pre = p.lse == nullptr;  // an exact lse needs the unfolded softmax factor
   if (fp8) {
-    if (pre) prefill_kernel<true, true><<<grid, kPfWaves * 64, 0, st>>>(p);
-    else prefill_kernel<true, false><<<grid, kPfWaves * 64, 0, st>>>(p);
+    if (pre) prefill_kernel<true, true><<<grid, kPfWaves * 64, 0, st>>>(p, t);
+    else prefill_kernel<true, false><<<grid, kPfWaves * 64, 0, st>>>(p, t);
   } else {
-    if (pre) prefill_kernel<false, true><<<grid, kPfWaves * 64, 0, st>>>(p);
-    else prefill_kernel<false, false><<<grid, kPfWaves * 64, 0, st>>>(p);
+    if (pre) prefill_kernel<false, true><<<grid, kPfWaves * 64, 0, st>>>(p, t);
+    else prefill_kernel<false, false><<<grid, kPfWaves * 64, 0, st>>>(p, t);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.pf_splits <= 1) return e;

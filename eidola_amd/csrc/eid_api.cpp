@@ -19,7 +19,10 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
                             const ItemTable *tab = nullptr);
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
 long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
-hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st);
+hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
+                          const PfTable *tab);
+bool build_prefill_table(const AttnParams &p, const int32_t *seq_lens_host,
+                         const int32_t *cu_seqlens_q_host, PfTable *tab);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
 hipError_t launch_rope_kv_write(const uint16_t *qkv, const int32_t *positions,
                                 const float *cos_sin, int max_pos, uint16_t *q_out,
@@ -864,11 +867,20 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
       if (e != hipSuccess) return hip_fail(e, "split-KV launch");
     }
   }
+  // With the host's copies of the lengths the prefill launch gets its query tiles listed,
+  // heaviest first (not under capture: a captured launch serves whatever lengths a replay finds)
+  eid::PfTable pf_tab;
+  pf_tab.n = 0;
+  auto list_tiles = [&](const eid::AttnParams &q) {
+    if (args->seq_lens_host && args->cu_seqlens_q_host && !capturing)
+      eid::build_prefill_table(q, args->seq_lens_host, args->cu_seqlens_q_host, &pf_tab);
+  };
   if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
     eid::AttnParams pp = p;
     pp.qlen_lo = qmax + 1;
     pp.qlen_hi = 0x7fffffff;
-    e = eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream);
+    list_tiles(pp);
+    e = eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream, &pf_tab);
     if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
   }
   if (args->split_done_event) {
@@ -897,7 +909,8 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   } else if (has_prefill) {  // long chunks: MFMA prefill kernel
     p.qlen_lo = qmax + 1;
     p.qlen_hi = 0x7fffffff;
-    e = eid::launch_prefill(p, desc->num_q_tokens, fp8, st);
+    list_tiles(p);
+    e = eid::launch_prefill(p, desc->num_q_tokens, fp8, st, &pf_tab);
     if (e != hipSuccess) return hip_fail(e, "prefill launch");
   }
   return EID_OK;

@@ -79,6 +79,16 @@ struct ItemTable {
   int32_t blk[kItemTableMax][4];
 };
 
+// Query tiles of a prefill launch listed by the host, heaviest (most keys to walk) first:
+// entry = seq | tile << 16.  The hardware hands workgroups to free slots in id order, so a
+// list sorted by work is longest-processing-time-first scheduling; a workgroup has its item
+// after one scalar load.  n == 0: the kernel finds its item by a scan of the device arrays.
+constexpr int kPfTableMax = 1024;
+struct PfTable {
+  int32_t n;
+  uint32_t e[kPfTableMax];
+};
+
 // What the QKV projection needs to finish as rope_kv_write_kernel would (see oproj_kernels.hip).
 struct RopeArgs {
   const int32_t *positions;
