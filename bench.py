@@ -252,8 +252,15 @@ def compact_pass(w, steps, warmup, torch):
     back-to-back steps / calls, page sets rotated."""
     for i in range(warmup):
         w.step(i)
-    ms_step = event_ms(w.step, steps, torch)
-    ms_attn = event_ms(lambda i: w.attn[i % w.n](), steps, torch)
+    # The core clock settles over the first ~20 ms of a new kind of load (an MFMA-bound kernel
+    # that follows memory-bound ones runs ~10 % slower until then): warm up for that long
+    # and time at least 10 ms of work.
+    est = max(event_ms(w.step, 5, torch), 1e-3)
+    for i in range(int(20.0 / est) + 1):
+        w.step(i)
+    n = max(steps, int(10.0 / est) + 1)
+    ms_step = event_ms(w.step, n, torch)
+    ms_attn = event_ms(lambda i: w.attn[i % w.n](), n, torch)
     return ms_step, ms_attn
 
 
@@ -735,6 +742,99 @@ def overlap_bench(torch):
     return res
 
 
+def timeline_bench(torch, ea, synth, np):
+    """Per-workgroup timeline of the prefill kernel on config 3's prefill rows (host-listed
+    tiles) from the library's measurement aid (eid_debug_set_timeline): when workgroups start
+    and end, how their duration depends on their work (least squares: fixed cost + cost per
+    64-token chunk), the stamps inside the kernel, how busy the device's workgroup slots are
+    over the kernel's span and how long the tail is."""
+    from eidola_amd import _lib
+    lib = _lib.load_library()
+    res = []
+
+    def one(name, w, waves, unit_name, slots_per_cu):
+        n_rec = 1 << 17
+        buf = torch.zeros(n_rec * 8, dtype=torch.int64, device="cuda:0")
+        for i in range(300):   # (past the clock's settling time)
+            w.attn[i % w.n]()
+        torch.cuda.synchronize()
+        lib.eid_debug_set_timeline(buf.data_ptr(), n_rec)
+        try:
+            runs = []
+            for rep in range(3):
+                buf.zero_()
+                for i in range(20):   # the last of back-to-back calls is the one recorded
+                    w.attn[(rep + i) % w.n]()
+                torch.cuda.synchronize()
+                runs.append(buf.view(-1, 8).cpu().numpy().copy())
+        finally:
+            lib.eid_debug_set_timeline(None, 0)
+        r = runs[-1]
+        used = (r[:, 0] != 0) & (r[:, 1] != 0)
+        nwg = (np.nonzero(used)[0].max() // waves) + 1
+        r = r[:nwg * waves].reshape(nwg, waves, 8)
+        ok = (r[:, :, 0] != 0) & (r[:, :, 1] != 0)
+        live = ok.any(axis=1)
+        t0 = np.where(ok, r[:, :, 0], np.iinfo(np.int64).max).min(axis=1)[live]
+        t1 = np.where(ok, r[:, :, 1], 0).max(axis=1)[live]
+        work = (np.where(ok, r[:, :, 2] >> 32, 0).max(axis=1))[live].astype(np.float64)
+        hw = r[:, 0, 2][live] & 0xffffffff
+        marks = None
+        if (r[:, :, 4:7][ok] != 0).all():   # stamps inside the kernel (prefill): mean over the waves
+            rel = np.where(ok[:, :, None], r[:, :, 4:7] - r[:, :, 0:1], 0).sum(axis=1) / np.maximum(1, ok.sum(axis=1))[:, None]
+            tail = np.where(ok, r[:, :, 1] - r[:, :, 6], 0).sum(axis=1) / np.maximum(1, ok.sum(axis=1))
+            marks = np.concatenate([rel[live], tail[live][:, None]], axis=1) / 100.0
+        xcc = r[:, 0, 3][live] & 0xf
+        cu_key = xcc * 4096 + ((hw >> 8) & 0xff)        # XCC, then shader engine / array / CU bits
+        base = t0.min()
+        start = (t0 - base) / 100.0                       # microseconds (100 MHz ticks)
+        end = (t1 - base) / 100.0
+        dur = end - start
+        span = end.max()
+        A = np.stack([np.ones_like(work), work], axis=1)
+        coef, *_ = np.linalg.lstsq(A, dur, rcond=None)
+        ncu = len(np.unique(cu_key))
+        slots = ncu * slots_per_cu
+        pct = lambda q: float(np.percentile(end, q))
+        out = {"config": f"timeline_{name}", "workgroups": int(live.sum()), "cus_seen": int(ncu),
+               "span_us": float(span), "start_us_p50": float(np.percentile(start, 50)),
+               "start_us_first_fill_max": float(np.sort(start)[min(slots, len(start)) - 1]),
+               "start_us_max": float(start.max()),
+               "dur_us_min": float(dur.min()), "dur_us_mean": float(dur.mean()), "dur_us_max": float(dur.max()),
+               f"fit_us_fixed": float(coef[0]), f"fit_us_per_{unit_name}": float(coef[1]),
+               "work_units_total": float(work.sum()), "work_units_max": float(work.max()),
+               "slot_busy_frac": float(dur.sum() / (slots * span)),
+               "end_us_p50": pct(50), "end_us_p90": pct(90), "end_us_p99": pct(99),
+               "xcc_busy_us": [float(dur[xcc == x].sum() / max(1, len(np.unique(cu_key[xcc == x])) * slots_per_cu))
+                               for x in range(8)]}
+        if marks is not None:
+            loop = marks[:, 2] - marks[:, 1]
+            out.update({"to_first_fetch_us": float(marks[:, 0].mean()), "first_tile_us": float((marks[:, 1] - marks[:, 0]).mean()),
+                        "loop_us_per_chunk": float((loop / np.maximum(work, 1)).mean()),
+                        "epilogue_us": float(marks[:, 3].mean())})
+            log(f"[bench] timeline {name}: per wave, start -> first fetch {out['to_first_fetch_us']:.2f} us, "
+                f"first tile in LDS after {out['first_tile_us']:.2f} us more, loop {out['loop_us_per_chunk']:.3f} us per "
+                f"chunk, last chunk -> end {out['epilogue_us']:.2f} us")
+        try:
+            np.savez(os.path.join(ROOT, "gpurun_out", f"timeline_{name}.npz"), start=start, end=end,
+                     work=work, xcc=xcc, hw=hw, marks=marks if marks is not None else np.zeros(0),
+                     records=r[live])
+        except OSError:
+            pass
+        log(f"[bench] timeline {name}: {out['workgroups']} workgroups on {ncu} CUs, span {span:.1f} us; first fill "
+            f"started by {out['start_us_first_fill_max']:.1f} us, last start {start.max():.1f}; duration "
+            f"{dur.min():.1f}/{dur.mean():.1f}/{dur.max():.1f} us (min/mean/max) = {coef[0]:.2f} + {coef[1]:.3f} per "
+            f"{unit_name}; slots busy {100*out['slot_busy_frac']:.1f}% of span; ends p50/p90/p99/max "
+            f"{pct(50):.1f}/{pct(90):.1f}/{pct(99):.1f}/{span:.1f} us")
+        res.append(out)
+
+    full = lambda off: synth.config3(perm_offset=off)
+    wp = Workload(lambda off: subset(full(off), np.arange(8), "config3_prefill_rows", synth), 2, 8,
+                  torch, ea, synth, "varlen")
+    one("config3_prefill_rows", wp, 4, "chunk", 2)
+    return res
+
+
 def cpu_baseline(w, torch, synth, threads):
     """The CPU restatement (oracle, fp32 path) timed on this host over the same batch:
     one full pass over page set 0 of the decode configuration."""
@@ -939,6 +1039,9 @@ def main():
             extra.extend(small_batch_bench(torch, ea, synth))
         if want("overlap"):
             extra.extend(overlap_bench(torch))
+        if want("timeline"):
+            import numpy as np
+            extra.extend(timeline_bench(torch, ea, synth, np))
         if want("stack"):
             extra.extend(stack_bench(torch, ea, synth, fused_qkv=False))
             extra.extend(stack_bench(torch, ea, synth))

@@ -103,7 +103,8 @@ class BatchInfo(C.Structure):
 
 EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_qkv_rope_kv_write", "eid_attn_decode",
            "eid_attn_decode_noalloc", "eid_attn_varlen", "eid_lse_merge", "eid_o_proj",
-           "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
+           "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version",
+           "eid_debug_set_timeline")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
                  "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
                  "eid_sched_block_refs", "eid_sched_build_batch")
@@ -152,6 +153,8 @@ def load_library():
     lib.eid_last_error.restype = C.c_char_p
     lib.eid_version.argtypes = []
     lib.eid_version.restype = C.c_uint32
+    lib.eid_debug_set_timeline.argtypes = [P, C.c_int64]
+    lib.eid_debug_set_timeline.restype = None
     # host-side scheduler (include/eidola_sched.h)
     lib.eid_sched_create.argtypes = [C.POINTER(SchedConfig), C.POINTER(P)]
     lib.eid_sched_create.restype = C.c_int32

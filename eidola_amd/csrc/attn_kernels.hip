@@ -224,6 +224,33 @@ __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_
   }
 }
 
+// Per-wave time stamps for the measurement aid (AttnParams::timeline).
+__device__ __forceinline__ void timeline_start(const AttnParams &p, const int slot) {
+  if (!p.timeline) return;
+  const unsigned long long t = __builtin_amdgcn_s_memrealtime();
+  // HW_ID (register 4, 32 bits) and XCC_ID (register 20, low 4 bits)
+  const unsigned hw = __builtin_amdgcn_s_getreg(4 | (31 << 11));
+  const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11));
+  if ((threadIdx.x & 63) == 0) {
+    p.timeline[(size_t)slot * 8 + 0] = t;
+    p.timeline[(size_t)slot * 8 + 2] = hw;
+    p.timeline[(size_t)slot * 8 + 3] = xcc;
+  }
+}
+__device__ __forceinline__ void timeline_mark(const AttnParams &p, const int slot, const int which) {
+  if (!p.timeline) return;
+  const unsigned long long t = __builtin_amdgcn_s_memrealtime();
+  if ((threadIdx.x & 63) == 0) p.timeline[(size_t)slot * 8 + 4 + which] = t;
+}
+__device__ __forceinline__ void timeline_end(const AttnParams &p, const int slot, const int work) {
+  if (!p.timeline) return;
+  const unsigned long long t = __builtin_amdgcn_s_memrealtime();
+  if ((threadIdx.x & 63) == 0) {
+    p.timeline[(size_t)slot * 8 + 1] = t;
+    p.timeline[(size_t)slot * 8 + 2] |= (unsigned long long)(unsigned)work << 32;
+  }
+}
+
 // Compile-time loop: f(std::integral_constant<int, 0>{}), ..., f(<N - 1>).
 template <int... Is, typename F>
 __device__ __forceinline__ void static_for_impl(std::integer_sequence<int, Is...>, F &&f) {
@@ -647,11 +674,16 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
 
 // Finish a row tile: either normalise with the sink and store bf16 output (+lse), or store
 // the partition's partial (m, l, acc) for the merge kernel.
-template <int NT, bool FP8, bool PAIR = false>
+//
+// SINK_IN: the caller has the lane's sink (log2 units, -inf for none) in `sink_in` already;
+// only where every row tile of a lane belongs to one query head (PAIR = false).
+template <int NT, bool FP8, bool PAIR = false, bool SINK_IN = false>
 __device__ __forceinline__ void finish(const AttnParams &p, const int s, const int kvh,
                                        const int row0, const int qlen, const int tq0,
                                        const bool direct, const int part, float (&m)[NT],
-                                       f32x4 (&lacc)[NT], f32x4 (&acc)[NT][4]) {
+                                       f32x4 (&lacc)[NT], f32x4 (&acc)[NT][4],
+                                       const float sink_in = 0.f) {
+  static_assert(!(PAIR && SINK_IN), "head pairs spread a lane's tiles over two heads");
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
   const int Hq = p.num_q_heads;
@@ -666,7 +698,7 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
     const bool valid = t < qlen;
     if (direct) {
       if (!valid) continue;
-      const float sink2 = p.sinks ? p.sinks[head] * kLog2e : -INFINITY;
+      const float sink2 = SINK_IN ? sink_in : (p.sinks ? p.sinks[head] * kLog2e : -INFINITY);
       const float M = fmaxf(m[nt], sink2);
       const float w = fast_exp2(m[nt] - M);
       const float den = l * w + fast_exp2(sink2 - M);
@@ -1347,6 +1379,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   __shared__ __align__(16) uint8_t lds_v[2][kPfVTileBytes];  // double-buffered V tile
   // PRE: every wave's eight Q fragments, in fragment order (see chunk_pipe)
   __shared__ __align__(16) uint8_t lds_q[PRE ? kPfWaves * 8 * kQFragBytes : 16];
+  __shared__ int item_lds[8];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
@@ -1357,6 +1390,14 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int KS = p.pf_splits;
   const int unit = blockIdx.x / Hkv;
   const int ks_part = KS > 1 ? unit % KS : 0;
+  const int tl_slot = blockIdx.x * kPfWaves + wave;
+  timeline_start(p, tl_slot);
+  const int W = p.window;
+  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
+  // the lane's rows all belong to one query head: its sink is fetched ahead of its use and
+  // parked in LDS (a register held through the chunk loop costs spills)
+  __shared__ float lds_sink[kPfWaves * 64];
+  lds_sink[tid] = p.sinks ? p.sinks[kvh * kGroup + (i16 & 7)] * kLog2e : -INFINITY;
   int s, tile, row0, qlen, L;
   if (tab.n > 0) {
     // the host listed the tiles: scalar loads alone (lengths still come from the device arrays)
@@ -1372,7 +1413,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     if (qlen < p.qlen_lo || qlen > p.qlen_hi || L < qlen || tile * kPfTok >= qlen) return;
   } else {
     // one wave looks the item up, the others receive it through LDS
-    __shared__ int item_lds[8];
     if (wave == 0) {
       int s0 = 0, tile0 = 0, row00 = 0, qlen0 = 0, L0 = 0;
       const bool found = find_prefill_item(p, KS > 1 ? unit / KS : unit, s0, tile0, row00, qlen0, L0);
@@ -1394,7 +1434,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     L = __builtin_amdgcn_readfirstlane(item_lds[5]);
   }
 
-  const int W = p.window;
   const int pos0 = L - qlen;
   const int tq_wg = tile * kPfTok;
   const int pos_first_wg = pos0 + tq_wg;
@@ -1413,28 +1452,6 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   const int pos_last = pos0 + min(tq0 + kPfWaveTok, qlen) - 1;
   const int lo_first = W > 0 ? max(0, pos_first - W + 1) : 0;
   const int lo_last = W > 0 ? max(0, pos_last - W + 1) : 0;
-
-  Frag8 qf[NT][2];
-  RowInfo ri;
-  const float c2 = p.softmax_scale * kLog2e * (FP8 ? p.k_scale[kvh] : 1.0f);
-  load_q<NT, PRE>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri, c2);
-  uint8_t *q_lds = &lds_q[0] + (PRE ? wave * (8 * kQFragBytes) + lane * 16 : 0);
-  if constexpr (PRE) {  // (wave-private: no barrier, the reads wait for the wave's own stores)
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-      for (int h = 0; h < 2; ++h) *(u32x4 *)(q_lds + (2 * nt + h) * kQFragBytes) = qf[nt][h].u;
-  }
-  bool maybe_fresh = true;
-  float m[NT];
-  f32x4 lacc[NT], acc[NT][4];
-#pragma unroll
-  for (int nt = 0; nt < NT; ++nt) {
-    m[nt] = kNegBig;
-    lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
 
   // cooperative loader: thread -> (row of the 64-token chunk, 32-byte segment of the head row)
   // (a wave loads one page of the chunk: its id is wave-uniform and travels in a scalar register)
@@ -1495,11 +1512,34 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     *(u32x4 *)(&lds_v[buf][st_off_v + 16]) = v1;
   };
 
-  if (t_begin < t_end) {
-    fetch(t_begin);
-    stash(t_begin, 0);
+  // the first K/V tile is requested before the Q operands: both are in flight together
+  timeline_mark(p, tl_slot, 0);
+  if (t_begin < t_end) fetch(t_begin);
+
+  Frag8 qf[NT][2];
+  RowInfo ri;
+  load_q<NT, PRE>(p, row0, qlen, wave_active ? tq0 : tq_wg, kvh, pos0, qf, ri, c2);
+  uint8_t *q_lds = &lds_q[0] + (PRE ? wave * (8 * kQFragBytes) + lane * 16 : 0);
+  if constexpr (PRE) {  // (wave-private: no barrier, the reads wait for the wave's own stores)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) *(u32x4 *)(q_lds + (2 * nt + h) * kQFragBytes) = qf[nt][h].u;
   }
+  bool maybe_fresh = true;
+  float m[NT];
+  f32x4 lacc[NT], acc[NT][4];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    m[nt] = kNegBig;
+    lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  if (t_begin < t_end) stash(t_begin, 0);
   __syncthreads();
+  timeline_mark(p, tl_slot, 1);
   int cur = 0;
   for (int tc = t_begin; tc < t_end; tc += kChunk, cur ^= 1) {
     const bool has_next = tc + kChunk < t_end;
@@ -1524,9 +1564,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     if (has_next) stash(tc + kChunk, cur ^ 1);
     __syncthreads();
   }
+  timeline_mark(p, tl_slot, 2);
   if (!wave_active) return;
   if (KS == 1) {
-    finish<NT, FP8>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc);
+    finish<NT, FP8, false, true>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc, lds_sink[tid]);
   } else {
     // partials of this part, one cell per (query token, part, head): finish() addresses cells
     // as (s * ws_rows + t), so the sequence's first row with one row per "sequence" gives the
@@ -1538,6 +1579,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     pp.nparts_max = KS;
     finish<NT, FP8>(pp, row0, kvh, row0, qlen, tq0, false, ks_part, m, lacc, acc);
   }
+  timeline_end(p, tl_slot, (t_end - t_begin + kChunk - 1) / kChunk);
 }
 
 // Merge of the key-range parts of the prefill kernel.  grid = (Hq / 4, num_q_tokens); one wave
@@ -2007,6 +2049,19 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
   return num_items * Hkv <= fill[ntiles == 1 ? 0 : ntiles == 3 ? 1 : 2][fp8 ? 1 : 0];
 }
 
+// Measurement aid: a device buffer of `entries` records of 64 bytes that the next prefill
+// launches of the process fill with per-wave time stamps (null: off).
+// Not thread-safe; launches with more waves than entries leave the buffer alone.
+static unsigned long long *g_timeline = nullptr;
+static long long g_timeline_entries = 0;
+void set_timeline(void *buf, long long entries) {
+  g_timeline = static_cast<unsigned long long *>(buf);
+  g_timeline_entries = buf ? entries : 0;
+}
+static unsigned long long *timeline_for(const long long waves) {
+  return waves <= g_timeline_entries ? g_timeline : nullptr;
+}
+
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same
 // params so that it uses the same partition.
@@ -2093,12 +2148,14 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
   dim3 grid((unsigned)(items * p.num_kv_heads));
   const PfTable &t = listed ? *tab : none;
   const bool pre = p.lse == nullptr;  // an exact lse needs the unfolded softmax factor
+  AttnParams q = p;
+  q.timeline = timeline_for((long long)grid.x * kPfWaves);
   if (fp8) {
-    if (pre) prefill_kernel<true, true><<<grid, kPfWaves * 64, 0, st>>>(p, t);
-    else prefill_kernel<true, false><<<grid, kPfWaves * 64, 0, st>>>(p, t);
+    if (pre) prefill_kernel<true, true><<<grid, kPfWaves * 64, 0, st>>>(q, t);
+    else prefill_kernel<true, false><<<grid, kPfWaves * 64, 0, st>>>(q, t);
   } else {
-    if (pre) prefill_kernel<false, true><<<grid, kPfWaves * 64, 0, st>>>(p, t);
-    else prefill_kernel<false, false><<<grid, kPfWaves * 64, 0, st>>>(p, t);
+    if (pre) prefill_kernel<false, true><<<grid, kPfWaves * 64, 0, st>>>(q, t);
+    else prefill_kernel<false, false><<<grid, kPfWaves * 64, 0, st>>>(q, t);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess || p.pf_splits <= 1) return e;

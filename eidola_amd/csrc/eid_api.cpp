@@ -21,6 +21,7 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
 long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
                           const PfTable *tab);
+void set_timeline(void *buf, long long entries);
 bool build_prefill_table(const AttnParams &p, const int32_t *seq_lens_host,
                          const int32_t *cu_seqlens_q_host, PfTable *tab);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
@@ -598,6 +599,8 @@ extern "C" {
 uint32_t eid_version(void) { return (EID_VERSION_MAJOR << 16) | EID_VERSION_MINOR; }
 
 const char *eid_last_error(void) { return g_err; }
+
+void eid_debug_set_timeline(void *device_buf, int64_t entries) { eid::set_timeline(device_buf, entries); }
 
 int32_t eid_partition_size(const eid_attn_desc *desc) {
   if (check_attn_desc(desc)) return 0;

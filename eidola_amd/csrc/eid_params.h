@@ -66,6 +66,10 @@ struct AttnParams {
   long long exact_items;     // host-side: the launch's exact number of work items when the host
                              // has the sequence lengths, 0 = not known (a bound is launched)
   float softmax_scale;
+  // Measurement aid, null in normal use: wave w of workgroup b of the prefill kernel
+  // stores {start, end} (100 MHz wall-clock ticks), {hardware id, XCC id} and up to
+  // four stamps in between at timeline[(b * waves + w) * 8 ..]; see set_timeline().
+  unsigned long long *timeline;
 };
 
 // Work items of a decode launch listed by the host (it has the sequence lengths): entry =
@@ -83,7 +87,7 @@ struct ItemTable {
 // entry = seq | tile << 16.  The hardware hands workgroups to free slots in id order, so a
 // list sorted by work is longest-processing-time-first scheduling; a workgroup has its item
 // after one scalar load.  n == 0: the kernel finds its item by a scan of the device arrays.
-constexpr int kPfTableMax = 1024;
+constexpr int kPfTableMax = 2048;
 struct PfTable {
   int32_t n;
   uint32_t e[kPfTableMax];

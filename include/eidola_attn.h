@@ -307,6 +307,17 @@ const char *eid_last_error(void);
 /* (major << 16) | minor */
 uint32_t eid_version(void);
 
+/* Measurement aid, no counterpart in the reference and no part of a serving path: hands the
+ * library a DEVICE buffer of `entries` records of 64 bytes (eight uint64).  From then on every
+ * chunked-prefill launch of this process whose waves (four per workgroup) fit the buffer lets
+ * wave w of workgroup b write record 4 b + w:
+ * {start, end} in 100 MHz wall-clock ticks, {hardware id | work units << 32, XCC id}, and in
+ * words 4..6 the prefill kernel's stamps before its first K/V fetch, after the first tile
+ * has arrived and after its last chunk; records of waves without work stay as the caller
+ * left them.  NULL switches it off (the default).
+ * Process-wide and not thread-safe: set it with no eid_* call in flight. */
+void eid_debug_set_timeline(void *device_buf, int64_t entries);
+
 #ifdef __cplusplus
 }
 #endif
