@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # --calibrate-copy).  See profiles/splitkv_decode_config2.md.  A kernel that is not listed
 # (or a non-default batch) reports traffic as null rather than another kernel's figure.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "splitkv_table_kernel<1,bf16,8 waves>": None,   # set from the profile of this tree, see below
+    "splitkv_table_kernel<1,bf16,8 waves>": int((241_266 * 2.0 + 2_146 * 1.0) * 1024),
     "splitkv_kernel<1,bf16,8 waves>": int((241_250 * 2.0 + 2_080 * 1.0) * 1024),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
@@ -385,7 +385,7 @@ def other_configs(a, torch, ea, synth, pool2, check):
         ms_step, ms_attn = compact_pass(w5, max(5, steps // 2), warm, torch)
         t5 += ms_step
         out[key] = hbm(synth.algorithmic_work(w5.batches[0]), ms_attn,
-                       "splitkv_kernel<3,bf16,8 waves>" if layer == 0 else "shortspan_kernel<3,bf16>",
+                       "splitkv_kernel<3,bf16,8 waves>" if layer == 0 else "splitkv_kernel<3,bf16,8 waves>, one item per sequence",
                        {"ms_per_step": ms_step, "partition_size": 512})
         if check:
             order = np.argsort(w5.batches[0].seq_lens)
