@@ -262,82 +262,78 @@ __device__ __forceinline__ void static_for(F &&f) {
 }
 
 // ---------------------------------------------------------------------------------------
-// Software-pipelined form of chunk_step<4, VROW, PRE = true> for the chunks of the prefill
-// kernel that need no masking (all but the one or two at the diagonal and at a window's lower
-// edge).  Same arithmetic, same results bit for bit; what changes is the ORDER of the
-// instruction stream.
+// Software-pipelined chunk of the prefill kernel (PRE = true: softmax factor folded into Q).
 //
 // A gfx950 SIMD issues matrix and vector instructions through one port: a wave's MFMA takes
-// one issue slot (4 cycles) and then keeps the matrix pipe busy for 16, during which three
-// more slots are free for vector instructions, but only if they come NEXT in some wave's
-// stream and do not depend on that MFMA.  Compiler-scheduled attention code runs the two
-// kinds of work one after the other (score MFMAs, then the softmax's vector instructions,
-// then the output MFMAs), and a second wave of the SIMD that happens to be in its vector
-// phase gets the port only while the first is not trying to issue an MFMA.  So the overlap
-// is written into the stream here.  With the four 16-row tiles nt = 0..3 of the wave:
-//   A(nt)  8 MFMAs   S(nt) = K Q(nt)^T - reference maximum (the accumulator's initial value)
-//   B(nt)  vector    lane-local maximum, exp2, conversion to bf16: P(nt)
-//   C(nt)  10 MFMAs  row sums and O(nt) += V^T P(nt)^T
-// the stream is  A(0) | B(0) + A(1) | B(1) + C(0), A(2) | B(2) + C(1), A(3) | B(3) + C(2) | C(3)
-// where "+" means: one MFMA, then the next few vector instructions, a scheduling barrier,
-// and so on, the vector work spread evenly over the stage's MFMAs.  A full stage has 18
-// MFMAs (288 cycles of the matrix pipe) and 8 max3 + 16 exp2 (two slots each) + 8 converts +
-// 4 moves = 52 slots of vector work on top of the MFMAs' own 18: both pipes are busy.
+// the port for about 9 cycles and then keeps the matrix pipe busy for 16, during which
+// vector instructions can issue, but only if they come NEXT in some wave's stream and do not
+// depend on that MFMA.  Compiler-scheduled attention code runs the two kinds of work one
+// after the other, and a second wave of the SIMD overlaps only partly (the port goes to the
+// oldest ready wave).  So the overlap is written into the stream here.  With the four 16-row
+// tiles t = 0..3 of the wave:
+//   A(t)   8 MFMAs   S(t) = K Q(t)^T - reference (the accumulator's initial value zs[t])
+//   B(t)   vector    exp2 of the 16 scores of a lane, conversion to bf16: P(t)
+//   R(t)   2 MFMAs   row sums of P(t)
+//   PV(t)  8 MFMAs   O(t) += V^T P(t)^T
+// the stream is  A(0) | B(0) + A(1),R(0) | B(1) + PV(0),A(2),R(1) | B(2) + PV(1),A(3),R(2) |
+// B(3) + PV(2),R(3) | PV(3), where "+" means: one MFMA, then the next few vector
+// instructions, a scheduling barrier, and so on, the vector work spread over the stage's
+// MFMAs by its issue cost.
 //
-// The rescaling decision uses the lane's own 16 scores: the row maximum (four lanes) exceeds
-// the slack iff some lane's maximum does, so the two cross-lane exchanges per tile are only
-// executed on the few chunks where the reference maximum moves (and on a wave's first
-// pipelined chunk, `maybe_fresh`, where rows may not have a reference yet).
+// The reference of a row is NOT its running maximum.  It is set from the row's first chunks
+// (`track`: chunks that need masking, and the wave's first plain chunk, take the lane-local
+// maximum as chunk_step does and move the reference when it is outgrown by 2^kLazyLog2) and
+// then left alone: exp2(s - reference) may grow far beyond 1 in a later chunk, which costs
+// nothing in fp32 / bf16 until it overflows.  The guard against that is the tile's row sum,
+// which R(t) delivers before PV(t) is issued: if it is not below 2^60 (this includes inf and
+// NaN) the tile's scores are recomputed from the operands still in registers, the reference
+// moves to the row's true maximum, O and l are rescaled, and P is rebuilt.  Scores far BELOW
+// the reference underflow to 0, which is their correct weight next to a row sum >= 1.
+// A plain stage is therefore 16 exp2 + 8 conversions + one compare and one add.
 //
-// The Q operands come from the wave's own LDS copy (q_rd: fragment (nt, half) at
-// (2 nt + half) * 1024 + lane * 16), read at the start of the stage that issues their MFMAs:
-// keeping all eight fragments in registers as well as two tiles' scores would not fit 256 VGPRs.
+// The Q operands come from the wave's own LDS copy (q_rd: fragment (t, half) at
+// (2 t + half) * 1024 + lane * 16): all eight fragments plus two tiles of scores would not fit
+// 256 VGPRs.
 // ---------------------------------------------------------------------------------------
 constexpr int kQFragBytes = 64 * 16;  // one Q fragment of a wave in LDS: 16 bytes per lane
+constexpr float kRowSumGuard = 1152921504606846976.0f;  // 2^60
 
 template <int I>
 using IC = std::integral_constant<int, I>;
 
-// Vector work of stage nt, in order: [Q read and accumulator seed of tile nt + 1] (PRE ops),
-// max3 tree (8), rescale check (1), then (exp2, exp2, convert) x 8.  Issue cycles: 4; exp2 8.
-// One mask op (skipped by a wave-uniform branch on most chunks) precedes the max tree.
-constexpr int pipe_op_cost(const int op, const int pre, const int nmask) {
-  if (op >= pre && op < pre + nmask) return 0;
-  const int e = op - (pre + nmask + 9);
-  return (e >= 0 && e % 3 != 2) ? 8 : 4;
+// Vector work of a stage, in order: [Q read of tile t + 2] (PRE ops), the tracking block (one
+// op, skipped by a wave-uniform branch on most chunks), then (exp2, exp2, convert) x 8.
+// Issue cycles: 4; exp2 8.
+constexpr int pipe_op_cost(const int op, const int pre) {
+  if (op < pre) return 4;
+  if (op == pre) return 0;
+  const int e = op - (pre + 1);
+  return e % 3 != 2 ? 8 : 4;
 }
-constexpr int pipe_cost_before(const int op, const int pre, const int nmask) {
+constexpr int pipe_cost_before(const int op, const int pre) {
   int c = 0;
-  for (int i = 0; i < op; ++i) c += pipe_op_cost(i, pre, nmask);
+  for (int i = 0; i < op; ++i) c += pipe_op_cost(i, pre);
   return c;
 }
 
-//
-// need_mask (wave-uniform): the chunk holds keys that some row must not see (the diagonal, a
-// window's lower edge, the end of the sequence): every score is compared with its row's
-// bounds before the maximum, as in chunk_step, and rows may stay without a reference maximum.
 template <int VROW>
 __device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile_stride,
                                            const uint8_t *v_rd, const uint8_t *q_rd,
-                                           bool &maybe_fresh, float (&m)[4], f32x4 (&lacc)[4],
-                                           f32x4 (&acc)[4][4], const RowInfo &ri, const int tc,
-                                           const bool need_mask) {
+                                           bool &maybe_fresh, float (&m)[4], f32x4 (&zs)[4],
+                                           float (&l)[4], f32x4 (&acc)[4][4], const RowInfo &ri,
+                                           const int tc, const bool need_mask) {
 #define EID_SB() __builtin_amdgcn_sched_barrier(0)
   Frag8 ones;
   ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
   asm volatile("" : "+v"(ones.u));  // kept in registers (else rebuilt from constants at every use)
   Frag8 kf[4][2], vf[4][2], qf[2][2];
-  f32x4 S[2][4], z[2];
+  f32x4 S[2][4], lt;
   Frag8 P[2][2];
+  const bool track = need_mask || maybe_fresh;
   auto read_q = [&](auto t_c) {
     constexpr int t = t_c;
     qf[t & 1][0].u = *(const u32x4 *)(q_rd + (2 * t) * kQFragBytes);
     qf[t & 1][1].u = *(const u32x4 *)(q_rd + (2 * t + 1) * kQFragBytes);
-  };
-  auto build_z = [&](auto t_c) {  // -(reference maximum) of tile t; 0 for a row without one
-    constexpr int t = t_c;
-    const float nb = m[t] == kNegBig ? 0.f : -m[t];
-    z[t & 1] = f32x4{nb, nb, nb, nb};
   };
   // ---- operands of the chunk: K first (the first MFMAs wait for them), Q(0), Q(1), V^T ----
 #pragma unroll
@@ -357,20 +353,70 @@ __device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile
       vf[mt][pr].w[2] = b2[0];
       vf[mt][pr].w[3] = b2[1];
     }
-  build_z(IC<0>{});
-  build_z(IC<1>{});
   EID_SB();
   // MFMA j of A(t): first the four token tiles' first halves, then their second halves
   auto mfma_a = [&](auto t_c, auto j_c) {
     constexpr int t = t_c, j = j_c, b = j & 3;
-    if constexpr (j < 4) S[t & 1][b] = mfma16x32(kf[b][0], qf[t & 1][0], z[t & 1]);
+    if constexpr (j < 4) S[t & 1][b] = mfma16x32(kf[b][0], qf[t & 1][0], zs[t]);
     else S[t & 1][b] = mfma16x32(kf[b][1], qf[t & 1][1], S[t & 1][b]);
   };
-  // MFMA j of C(t): row sums, then the four dim tiles, for token pair 0, then for pair 1
-  auto mfma_c = [&](auto t_c, auto j_c) {
-    constexpr int t = t_c, j = j_c, pr = j / 5, i = j % 5;
-    if constexpr (i == 0) lacc[t] = mfma16x32(ones, P[t & 1][pr], lacc[t]);
-    else acc[t][i - 1] = mfma16x32(vf[i - 1][pr], P[t & 1][pr], acc[t][i - 1]);
+  // MFMA j of PV(t): the four dim tiles for token pair 0, then for pair 1
+  auto mfma_pv = [&](auto t_c, auto j_c) {
+    constexpr int t = t_c, j = j_c, pr = j / 4, i = j % 4;
+    acc[t][i] = mfma16x32(vf[i][pr], P[t & 1][pr], acc[t][i]);
+  };
+  // MFMA j of R(t): row sums of P(t) (every lane of a row receives the sum over its 64 keys)
+  auto mfma_r = [&](auto t_c, auto j_c) {
+    constexpr int t = t_c, j = j_c;
+    if constexpr (j == 0) lt = mfma16x32(ones, P[t & 1][0], f32x4{0.f, 0.f, 0.f, 0.f});
+    else lt = mfma16x32(ones, P[t & 1][1], lt);
+  };
+  auto set_ref = [&](auto t_c, const float m_new) {
+    constexpr int t = t_c;
+    m[t] = m_new;
+    const float nb = m_new == kNegBig ? 0.f : -m_new;
+    zs[t] = f32x4{nb, nb, nb, nb};
+  };
+  auto rescale = [&](auto t_c, const float alpha) {
+    constexpr int t = t_c;
+    l[t] *= alpha;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[t][mt][r] *= alpha;
+  };
+  auto lane_max = [&](const f32x4 (&Sx)[4]) {
+    float mx = max3(Sx[0][0], Sx[0][1], Sx[0][2]);
+#pragma unroll
+    for (int o = 1; o < 7; ++o)
+      mx = max3(mx, Sx[(2 * o + 1) >> 2][(2 * o + 1) & 3], Sx[(2 * o + 2) >> 2][(2 * o + 2) & 3]);
+    return max2(mx, Sx[3][3]);
+  };
+  // The guard of tile t, between R(t) and PV(t); S(t)'s registers and Q(t) are still there.
+  auto guard = [&](auto t_c) {
+    constexpr int t = t_c;
+    if (__any(!(lt[0] < kRowSumGuard))) {  // (rare) some weight of the tile overflowed
+      f32x4(&Sx)[4] = S[t & 1];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        Sx[b] = mfma16x32(kf[b][0], qf[t & 1][0], f32x4{0.f, 0.f, 0.f, 0.f});
+        Sx[b] = mfma16x32(kf[b][1], qf[t & 1][1], Sx[b]);
+      }
+      const float mrow = rowgroup_max(lane_max(Sx));  // (plain chunk: every key is visible)
+      const bool fresh = m[t] == kNegBig;
+      const float m_new = fresh ? mrow : max2(m[t], mrow);
+      rescale(t_c, fresh ? 0.f : fast_exp2(m[t] - m_new));
+      set_ref(t_c, m_new);
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        const float p0 = fast_exp2(Sx[(2 * k) >> 2][(2 * k) & 3] - m_new);
+        const float p1 = fast_exp2(Sx[(2 * k + 1) >> 2][(2 * k + 1) & 3] - m_new);
+        P[t & 1][k >> 2].w[k & 3] = pack_bf16(p0, p1);
+      }
+      lt = mfma16x32(ones, P[t & 1][0], f32x4{0.f, 0.f, 0.f, 0.f});
+      lt = mfma16x32(ones, P[t & 1][1], lt);
+    }
+    l[t] += lt[0];
   };
   __builtin_amdgcn_s_setprio(1);
   static_for<8>([&](auto j) {
@@ -380,63 +426,56 @@ __device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile
   // ---- stages ----
   static_for<4>([&](auto nt_c) {
     constexpr int nt = nt_c;
-    constexpr bool has_c = nt > 0, has_a = nt < 3;
-    constexpr int NM = (has_c ? 10 : 0) + (has_a ? 8 : 0);
-    constexpr int kPre = (nt == 1 || nt == 2) ? 2 : 0;  // read_q(nt + 1) and build_z(nt + 1)
-    constexpr int kMask = 1;
-    constexpr int NV = kPre + kMask + 9 + 24;
-    constexpr int total = pipe_cost_before(NV, kPre, kMask);
-    float mloc = 0.f;
+    constexpr bool has_pv = nt > 0, has_a = nt < 3;
+    constexpr int NM = (has_pv ? 8 : 0) + (has_a ? 8 : 0) + 2;  // R(nt) sits at NM - 4, NM - 3
+    constexpr int NB = NM - 4;                                   // B(nt) is spread over slots 0..NB-1
+    constexpr int kPre = (nt == 1 || nt == 2) ? 1 : 0;           // read_q(nt + 1)
+    constexpr int NV = kPre + 1 + 24;
+    constexpr int total = pipe_cost_before(NV, kPre);
     f32x4(&Sx)[4] = S[nt & 1];
+    if constexpr (has_pv) {
+      guard(IC<nt - 1>{});  // before PV(nt - 1) and before Q(nt + 1) replaces Q(nt - 1)
+      EID_SB();
+    }
     auto vop = [&](auto op_c) {
-      constexpr int op = op_c, o = op - kPre - kMask;
+      constexpr int op = op_c, o = op - kPre - 1;
       if constexpr (op < kPre) {
         constexpr int t1 = nt + 1 < 4 ? nt + 1 : 0;  // (never reached for nt == 3)
-        if constexpr (op == 0) read_q(IC<t1>{});
-        else build_z(IC<t1>{});
-      } else if constexpr (op < kPre + kMask) {  // keys of the lane against the row's bounds
-        if (need_mask) {
-          int pos, lo;
-          ri.bounds(nt, pos, lo);
-          const int j0 = tc + 4 * ((threadIdx.x & 63) >> 4);
-#pragma unroll
-          for (int b = 0; b < 4; ++b)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const int j = j0 + b * kBlock + r;
-              if (j < lo || j > pos) Sx[b][r] = -INFINITY;
-            }
-        }
-      } else if constexpr (o < 8) {  // max3 tree over the lane's 16 scores
-        if constexpr (o == 0) mloc = max3(Sx[0][0], Sx[0][1], Sx[0][2]);
-        else if constexpr (o == 7) mloc = max2(mloc, Sx[3][3]);
-        else mloc = max3(mloc, Sx[(2 * o + 1) >> 2][(2 * o + 1) & 3], Sx[(2 * o + 2) >> 2][(2 * o + 2) & 3]);
-      } else if constexpr (o == 8) {
-        // (rare) the reference maximum of some row has to move, exactly as in chunk_step
-        if (maybe_fresh || __any(mloc > kLazyLog2)) {
-          const bool fresh = m[nt] == kNegBig;
-          const float base = fresh ? 0.f : m[nt];
-          const float mrow = rowgroup_max(mloc);
-          const bool up = mrow > (fresh ? kNegBig : kLazyLog2);
-          if (__any(up)) {
-            const float shift = up ? mrow : 0.f;
-            const float m_new = up ? base + mrow : m[nt];
-            const float alpha = fast_exp2(m[nt] - m_new);
-            m[nt] = m_new;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) lacc[nt][r] *= alpha;
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-              for (int r = 0; r < 4; ++r) acc[nt][mt][r] *= alpha;
+        read_q(IC<t1>{});
+      } else if constexpr (op == kPre) {
+        if (track) {  // a masked chunk or the wave's first plain one: the reference follows the maximum
+          if (need_mask) {
+            int pos, lo;
+            ri.bounds(nt, pos, lo);
+            const int j0 = tc + 4 * ((threadIdx.x & 63) >> 4);
 #pragma unroll
             for (int b = 0; b < 4; ++b)
 #pragma unroll
-              for (int r = 0; r < 4; ++r) Sx[b][r] -= shift;
+              for (int r = 0; r < 4; ++r) {
+                const int j = j0 + b * kBlock + r;
+                if (j < lo || j > pos) Sx[b][r] = -INFINITY;
+              }
+          }
+          const float mloc = lane_max(Sx);
+          if (maybe_fresh || __any(mloc > kLazyLog2)) {
+            const bool fresh = m[nt] == kNegBig;
+            const float base = fresh ? 0.f : m[nt];
+            const float mrow = rowgroup_max(mloc);
+            const bool up = mrow > (fresh ? kNegBig : kLazyLog2);
+            if (__any(up)) {
+              const float shift = up ? mrow : 0.f;
+              const float m_new = up ? base + mrow : m[nt];
+              rescale(nt_c, fast_exp2(m[nt] - m_new));
+              set_ref(nt_c, m_new);
+#pragma unroll
+              for (int b = 0; b < 4; ++b)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) Sx[b][r] -= shift;
+            }
           }
         }
       } else {
-        constexpr int e = o - 9, k = e / 3;  // convert k packs exp2 2k and 2k + 1
+        constexpr int e = o, k = e / 3;  // convert k packs exp2 2k and 2k + 1
         if constexpr (e % 3 != 2) {
           constexpr int i = 2 * k + e % 3;
           Sx[i >> 2][i & 3] = fast_exp2(Sx[i >> 2][i & 3]);
@@ -449,20 +488,29 @@ __device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile
         }
       }
     };
-    // vector op `op` goes behind MFMA number (cycles of the ops before it) * NM / (all cycles)
+    // MFMA in slot s: PV(nt - 1), then A(nt + 1), with R(nt) in slots NM - 4 and NM - 3
     static_for<NM>([&](auto s_c) {
       constexpr int s = s_c;
-      if constexpr (has_c && s < 10) mfma_c(IC<nt - 1>{}, s_c);
-      else mfma_a(IC<nt + 1>{}, IC<(has_c ? s - 10 : s)>{});
-      static_for<NV>([&](auto op_c) {
-        constexpr int op = op_c;
-        if constexpr (pipe_cost_before(op, kPre, kMask) * NM / total == s) vop(op_c);
-      });
+      if constexpr (s == NM - 4) mfma_r(nt_c, IC<0>{});
+      else if constexpr (s == NM - 3) mfma_r(nt_c, IC<1>{});
+      else {
+        constexpr int q = s < NM - 4 ? s : s - 2;  // index among the stage's other MFMAs
+        if constexpr (has_pv && q < 8) mfma_pv(IC<nt - 1>{}, IC<q>{});
+        else mfma_a(IC<(nt + 1 < 4 ? nt + 1 : 0)>{}, IC<(has_pv ? q - 8 : q)>{});
+      }
+      if constexpr (s < NB) {
+        static_for<NV>([&](auto op_c) {
+          constexpr int op = op_c;
+          if constexpr (pipe_cost_before(op, kPre) * NB / total == s) vop(op_c);
+        });
+      }
       EID_SB();
     });
   });
-  static_for<10>([&](auto j) {
-    mfma_c(IC<3>{}, j);
+  guard(IC<3>{});
+  EID_SB();
+  static_for<8>([&](auto j) {
+    mfma_pv(IC<3>{}, j);
     EID_SB();
   });
   __builtin_amdgcn_s_setprio(0);
@@ -1529,10 +1577,15 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   bool maybe_fresh = true;
   float m[NT];
   f32x4 lacc[NT], acc[NT][4];
+  // PRE: the rows' row sums as scalars and the MFMA seeds -(reference) of the four tiles
+  float lsum[NT];
+  f32x4 zs[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     m[nt] = kNegBig;
     lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    lsum[nt] = 0.f;
+    zs[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -1549,8 +1602,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
       const uint8_t *v_rd = &lds_v[cur][0] + (4 * g + (i16 >> 2)) * kPfVRowBytes + 8 * (i16 & 3);
       const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
       if constexpr (PRE) {
-        chunk_pipe<kPfVRowBytes>(kt, kBlock * kPfKRowBytes, v_rd, q_lds, maybe_fresh, m, lacc, acc, ri, tc,
-                                 need_mask);
+        chunk_pipe<kPfVRowBytes>(kt, kBlock * kPfKRowBytes, v_rd, q_lds, maybe_fresh, m, zs, lsum, acc, ri,
+                                 tc, need_mask);
       } else {
         Frag8 kf[4][2];
 #pragma unroll
@@ -1566,6 +1619,10 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
   }
   timeline_mark(p, tl_slot, 2);
   if (!wave_active) return;
+  if constexpr (PRE) {
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) lacc[nt] = f32x4{lsum[nt], lsum[nt], lsum[nt], lsum[nt]};
+  }
   if (KS == 1) {
     finish<NT, FP8, false, true>(p, s, kvh, row0, qlen, tq0, true, 0, m, lacc, acc, lds_sink[tid]);
   } else {

@@ -292,14 +292,16 @@ def test_prefill_chunks_and_decodes_mixed(G, window):
     assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, f"prefill mixed w={window}, no lse")
 
 
-@pytest.mark.parametrize("shape", ["rising", "falling", "deep"])
+@pytest.mark.parametrize("shape", ["rising", "falling", "deep", "spikes"])
 @pytest.mark.parametrize("window", [0, 100])
 def test_prefill_scores_far_from_zero(G, shape, window):
-    """Scores that climb by tens of log2 units per 64-key chunk (the reference maximum of the
-    lazy softmax moves on every chunk), fall as fast (later chunks underflow against it), or sit
-    some 70 log2 units below zero throughout (a row's first maximum is far from the value its
-    accumulator starts at).  Prefill rows and a few decode / verify rows, with lse (unfolded
-    softmax factor) and without (factor folded into the Q operands)."""
+    """Scores that climb by tens of log2 units per 64-key chunk (the reference of the prefill
+    kernel's softmax is outgrown again and again: its row-sum guard has to trip and recover),
+    fall as fast (later chunks underflow against it), sit some 70 log2 units below zero
+    throughout (a row's first maximum is far from the value its accumulator starts at), or
+    are ordinary except for single keys of some KV heads that score ~130 log2 units higher
+    (only some rows of some chunks overflow).  Prefill rows and a few decode / verify rows,
+    with lse (unfolded softmax factor) and without (factor folded into the Q operands)."""
     seq_lens, q_lens = [600, 333, 64, 700, 90], [64, 333, 64, 5, 1]
     b = make_batch(seq_lens, q_lens, window=window, seed=61)
     q, k, v, sinks = logical_tensors(b)
@@ -313,9 +315,15 @@ def test_prefill_scores_far_from_zero(G, shape, window):
     elif shape == "falling":
         qf += 1
         kf -= pos / 16
-    else:                        # about -50 nats everywhere
+    elif shape == "deep":        # about -50 nats everywhere
         qf -= 1
         kf += np.float32(6.25)
+    else:                        # q offset 1, a few keys offset 12 on two KV heads: +96 nats there
+        qf += 1
+        rng = np.random.default_rng(5)
+        hot = rng.choice(kf.shape[0], size=24, replace=False)
+        kf[hot[:12], 2] += np.float32(12)
+        kf[hot[12:], 5] += np.float32(12)
     q, k = synth.f32_to_bf16_bits(qf), synth.f32_to_bf16_bits(kf)
     sinks = None if shape == "deep" else sinks
     kc, vc = cpu_caches(b, k, v)
