@@ -1,0 +1,139 @@
+"""Host tests of the OpenAI-compatible engine shim (eidola_amd/engine_shim.py), in the style of
+the reference's fake-engine tests (/root/reference/crates/eidola-app-core/tests/local_models.rs:
+855-861): the shim is started the way the reference starts its engine (same flags, polled on
+/health) with the CPU echo engine behind it, and answers the body the reference sends."""
+import json
+import os
+import socket
+import subprocess
+import sys
+import threading
+import time
+import urllib.error
+import urllib.request
+
+import pytest
+
+from eidola_amd import engine_shim as shim
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def reference_body(model, messages, max_completion_tokens, stream=False, include_usage=False):
+    """The outer shape of chat_completion_request_body (eidola-common/src/lib.rs:116-139)."""
+    body = {"model": model, "messages": messages, "max_completion_tokens": max_completion_tokens}
+    if stream:
+        body["stream"] = True
+        if include_usage:
+            body["stream_options"] = {"include_usage": True}
+    return body
+
+
+def post(port, body, raw=False):
+    data = body if isinstance(body, bytes) else json.dumps(body).encode()
+    req = urllib.request.Request(f"http://127.0.0.1:{port}/v1/chat/completions", data=data,
+                                 headers={"Content-Type": "application/json"})
+    with urllib.request.urlopen(req, timeout=10) as r:
+        payload = r.read()
+        return (r.status, r.headers, payload) if raw else json.loads(payload)
+
+
+@pytest.fixture()
+def server():
+    srv = shim.make_server("127.0.0.1", 0, shim.FakeEngine(), "local/test-model")
+    t = threading.Thread(target=srv.serve_forever, daemon=True)
+    t.start()
+    yield srv.server_address[1]
+    srv.shutdown()
+    srv.server_close()
+
+
+def test_flags_of_the_reference_are_accepted():
+    a = shim.parse_args(["-m", "/models/x.gguf", "--host", "127.0.0.1", "--port", "18080", "--alias",
+                         "local/x", "-c", "8192", "-ngl", "999", "--jinja", "--no-webui"])
+    assert (a.model, a.host, a.port, a.alias, a.ctx_size, a.n_gpu_layers) == \
+        ("/models/x.gguf", "127.0.0.1", 18080, "local/x", 8192, 999)
+    assert a.jinja and a.no_webui and a.engine == "synthetic"
+
+
+def test_health_and_models(server):
+    with urllib.request.urlopen(f"http://127.0.0.1:{server}/health", timeout=5) as r:
+        assert r.status == 200 and json.loads(r.read()) == {"status": "ok"}
+    with urllib.request.urlopen(f"http://127.0.0.1:{server}/v1/models", timeout=5) as r:
+        assert json.loads(r.read())["data"][0]["id"] == "local/test-model"
+    with pytest.raises(urllib.error.HTTPError) as e:
+        urllib.request.urlopen(f"http://127.0.0.1:{server}/nope", timeout=5)
+    assert e.value.code == 404
+
+
+def test_blocking_completion_has_the_openai_shape(server):
+    msgs = [{"role": "system", "content": "be brief"}, {"role": "user", "content": "abc déf"}]
+    r = post(server, reference_body("local/test-model", msgs, 64))
+    assert r["object"] == "chat.completion" and r["model"] == "local/test-model"
+    c = r["choices"][0]
+    assert c["index"] == 0 and c["finish_reason"] == "stop"
+    assert c["message"] == {"role": "assistant", "content": "féd cba"}
+    u = r["usage"]
+    assert u["prompt_tokens"] == len(shim.render_prompt(msgs))
+    assert u["total_tokens"] == u["prompt_tokens"] + u["completion_tokens"]
+    # the budget cuts the answer: finish_reason says so
+    r = post(server, reference_body("m", [{"role": "user", "content": "0123456789"}], 4))
+    assert r["choices"][0] == {"index": 0, "finish_reason": "length",
+                               "message": {"role": "assistant", "content": "9876"}}
+
+
+def test_streaming_completion_is_sse_with_usage_and_done(server):
+    status, headers, payload = post(server, reference_body("m", [{"role": "user", "content": "héllo"}], 32,
+                                                           stream=True, include_usage=True), raw=True)
+    assert status == 200 and headers["Content-Type"].startswith("text/event-stream")
+    events = [e[len(b"data: "):] for e in payload.split(b"\n\n") if e.startswith(b"data: ")]
+    assert events[-1] == b"[DONE]"
+    chunks = [json.loads(e) for e in events[:-1]]
+    assert all(c["object"] == "chat.completion.chunk" for c in chunks)
+    assert chunks[0]["choices"][0]["delta"]["role"] == "assistant"
+    text = "".join(c["choices"][0]["delta"].get("content", "") for c in chunks if c["choices"])
+    assert text == "olléh"
+    assert chunks[-2]["choices"][0]["finish_reason"] == "stop" and chunks[-2]["choices"][0]["delta"] == {}
+    assert chunks[-1]["choices"] == [] and chunks[-1]["usage"]["completion_tokens"] == len("olléh".encode())
+    # without stream_options there is no usage chunk
+    _, _, payload = post(server, reference_body("m", [{"role": "user", "content": "x"}], 8, stream=True), raw=True)
+    assert b'"usage"' not in payload and payload.rstrip().endswith(b"data: [DONE]")
+
+
+@pytest.mark.parametrize("body", [b"{not json", json.dumps({"model": "m"}).encode(),
+                                  json.dumps({"messages": [], "max_completion_tokens": 4}).encode(),
+                                  json.dumps({"messages": [{"role": "user", "content": "x"}],
+                                              "max_completion_tokens": 0}).encode()])
+def test_bad_requests_get_a_400_with_an_error_object(server, body):
+    with pytest.raises(urllib.error.HTTPError) as e:
+        post(server, body)
+    assert e.value.code == 400
+    assert json.loads(e.value.read())["error"]["type"] == "invalid_request_error"
+
+
+def test_started_and_polled_the_way_the_reference_does():
+    """The reference spawns the engine with its flags, stdin/stdout null, and polls /health
+    until it answers 2xx (local_models.rs:1612-1626, 2020-2063)."""
+    with socket.socket() as s:
+        s.bind(("127.0.0.1", 0))
+        port = s.getsockname()[1]
+    child = subprocess.Popen(
+        [sys.executable, "-m", "eidola_amd.engine_shim", "-m", "/nonexistent/model.gguf", "--host",
+         "127.0.0.1", "--port", str(port), "--alias", "local/echo", "-c", "4096", "-ngl", "999", "--jinja",
+         "--no-webui", "--engine", "fake"],
+        cwd=ROOT, stdin=subprocess.DEVNULL, stdout=subprocess.DEVNULL, stderr=subprocess.PIPE)
+    try:
+        deadline, ready = time.time() + 30, False
+        while time.time() < deadline and child.poll() is None:
+            try:
+                with urllib.request.urlopen(f"http://127.0.0.1:{port}/health", timeout=1) as r:
+                    ready = 200 <= r.status < 300
+                    break
+            except (urllib.error.URLError, ConnectionError, socket.timeout):
+                time.sleep(0.1)
+        assert ready, child.stderr.read().decode() if child.poll() is not None else "never became ready"
+        r = post(port, reference_body("local/echo", [{"role": "user", "content": "ping"}], 16))
+        assert r["choices"][0]["message"]["content"] == "gnip" and r["model"] == "local/echo"
+    finally:
+        child.terminate()
+        child.wait(timeout=10)
