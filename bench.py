@@ -742,6 +742,56 @@ def overlap_bench(torch):
     return res
 
 
+def gather_bench(torch, ea, synth, np):
+    """What a pure gather of config 2's pages sustains (eidola_amd/csrc/probe_gather.hip): the
+    decode kernel's access pattern and grid shapes with no attention arithmetic, against the
+    same 300,000-page pools and the same rotated page sets, so the decode kernel's 491.7 MB per
+    launch can be read against what the memory system gives a kernel that only loads."""
+    import ctypes as C
+    lib = C.CDLL(os.path.join(ROOT, "eidola_amd", "csrc", "libeid_probe.so"))
+    lib.eid_probe_gather.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                     C.c_void_p, C.c_void_p]
+    lib.eid_probe_gather.restype = C.c_int
+    w = Workload(lambda off: synth.config2(perm_offset=off), 8, 7, torch, ea, synth, "decode")
+    sink = torch.zeros(4, dtype=torch.int32, device="cuda:0")
+    st = torch.cuda.current_stream().cuda_stream
+    res = []
+    tables, npages = {}, None
+    for kind in ("shuffled", "contiguous"):
+        per_set = []
+        for s, b in enumerate(w.batches):
+            nblk = (b.seq_lens.astype(np.int64) + 15) // 16
+            pages = np.concatenate([b.block_table[q, :n] for q, n in enumerate(nblk)]).astype(np.int32)
+            if kind == "contiguous":
+                pages = np.arange(s * len(pages), (s + 1) * len(pages), dtype=np.int32)
+            per_set.append(torch.from_numpy(pages).to("cuda:0"))
+        tables[kind], npages = per_set, len(per_set[0])
+        tables[kind + "_x8"] = [torch.cat([t[:npages // 32 * 32] for t in per_set])]
+    for kind, ppw, delay, lds, rows in (
+            ("shuffled", 32, 0, 75, 0), ("shuffled", 32, 0, 0, 0), ("shuffled", 16, 0, 75, 0), ("shuffled", 64, 0, 75, 0),
+            ("contiguous", 32, 0, 75, 0), ("shuffled", 32, 40, 75, 0), ("shuffled", 32, 128, 75, 0),
+            ("shuffled", 32, 0, 75, 1), ("shuffled", 32, 0, 0, 1), ("contiguous", 32, 0, 75, 1), ("contiguous", 32, 0, 0, 1),
+            ("shuffled_x8", 32, 0, 75, 0), ("shuffled_x8", 32, 0, 75, 1), ("contiguous_x8", 32, 0, 75, 1)):
+        nwg = npages // ppw
+        if kind.endswith("_x8"):  # all eight page sets in one launch: the rate without the ends
+            nwg *= w.n
+
+        def run(i):
+            rc = lib.eid_probe_gather(w.k_cache.data_ptr(), w.v_cache.data_ptr(),
+                                      tables[kind][i % len(tables[kind])].data_ptr(), nwg, ppw, delay, lds * 1024, rows, sink.data_ptr(), st)
+            assert rc == 0
+        for i in range(10):
+            run(i)
+        ms = event_ms(run, 100, torch)
+        nbytes = nwg * ppw * 2 * 16384
+        r = {"config": f"gather_probe_{kind}_{ppw}_pages_per_wg_delay_{delay}_lds_{lds}k_{'rows' if rows else 'heads'}", "ms": ms, "bytes": nbytes,
+             "GBps": nbytes / ms / 1e6, "workgroups": nwg}
+        log(f"[bench] gather probe, {kind} pages, {ppw} per workgroup ({nwg} workgroups, {lds} KiB LDS, a wave reads {'whole rows' if rows else 'one head'}), {delay} ALU "
+            f"links per batch: {ms*1e3:.1f} us for {nbytes/1e6:.1f} MB = {r['GBps']:.0f} GB/s = {100*r['GBps']/HBM_PEAK_GBS:.1f}% of peak")
+        res.append(r)
+    return res
+
+
 def timeline_bench(torch, ea, synth, np):
     """Per-workgroup timeline of the prefill kernel on config 3's prefill rows (host-listed
     tiles) from the library's measurement aid (eid_debug_set_timeline): when workgroups start
@@ -1042,6 +1092,9 @@ def main():
         if want("timeline"):
             import numpy as np
             extra.extend(timeline_bench(torch, ea, synth, np))
+        if want("gather"):
+            import numpy as np
+            extra.extend(gather_bench(torch, ea, synth, np))
         if want("stack"):
             extra.extend(stack_bench(torch, ea, synth, fused_qkv=False))
             extra.extend(stack_bench(torch, ea, synth))
