@@ -13,7 +13,7 @@
 // the N dimension, so lane (i16, g) = (lane % 16, lane / 16) of a result tile holds features
 // 4g..4g+3 of token i16: four consecutive bf16 of an output row, one 8-byte store.
 //
-// Two kernels:
+// Three kernels:
 //   oproj_skinny_kernel  T <= 64 (decode batches).  HBM-bound: the weight (N*K*2 bytes) is
 //                        streamed once.  One workgroup per 16 features (per 32 when that
 //                        keeps the workgroups within one per CU); its 8 waves deal the
@@ -22,8 +22,13 @@
 //   oproj_tiled_kernel   any T.  128 x 128 (or, for batches too small to fill the device
 //                        with that, 64 x 64) tokens x features per workgroup, K in steps of
 //                        64 through double-buffered, row-padded LDS tiles.
+//   oproj_wide_kernel    prefill-sized T (thousands of tokens).  256 tokens x 192 features per
+//                        workgroup, one workgroup of 8 waves per CU, K in steps of 64 through
+//                        two LDS stages filled by direct global -> LDS loads.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
+#include <type_traits>
 
 #include "eid_device.h"
 #include "eid_params.h"
@@ -437,6 +442,152 @@ __global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Wide kernel (prefill-sized batches).  One workgroup per CU; workgroup tile = 16 WT WM tokens
+// x 16 WF WN features, wave (wm, wn) owns 16 WT tokens x 16 WF features.  K advances 64
+// elements per step through two LDS stages that the loads fill directly
+// (global_load_lds_dwordx4: a wave instruction moves 8 rows x 128 bytes, no registers), the
+// eight 16-byte segments of a row permuted by (row / 2) % 8 so that fragment reads are free of
+// bank conflicts.  One barrier per step, placed between its two 32-element halves: by then the
+// stage of the next step has had a whole step to arrive, the first half's fragments of the
+// next step are fetched from LDS while the second half's MFMAs run, and the stage just
+// finished is handed to the loads of the step after next.
+// Requires K % 64 == 0 and N % 16 == 0.
+// ---------------------------------------------------------------------------------------
+namespace {
+typedef __attribute__((address_space(1))) const void dma_gptr_t;
+typedef __attribute__((address_space(3))) void dma_lptr_t;
+}  // namespace
+
+template <int WF, int WT, int WN, int WM>
+__global__ __launch_bounds__(64 * WN * WM, 1) void oproj_wide_kernel(
+    const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
+    const uint16_t *__restrict__ bias, const uint16_t *resid,
+    uint16_t *out, const int T, const int N, const int K, const int tiles_m,
+    const int tiles_n) {
+  constexpr int kNF = 16 * WF * WN, kNT = 16 * WT * WM, kWaves = WN * WM;
+  constexpr int kRows = kNF + kNT, kStage = kRows * 128;
+  constexpr int kPieces = kRows / 8;  // 1 KiB pieces of a stage
+  static_assert(kPieces % kWaves == 0 && kNF % 16 == 0, "pieces are dealt evenly to the waves");
+  constexpr int kPer = kPieces / kWaves;
+  __shared__ __align__(1024) uint8_t stage0[kStage];
+  __shared__ __align__(1024) uint8_t stage1[kStage];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int i16 = lane & 15, g = lane >> 4;
+  const int wm = wave / WN, wn = wave % WN;
+
+  // XCD-aware tile order, as in the tiled kernel
+  const int total = tiles_m * tiles_n;
+  const int xcd = blockIdx.x & 7, nth = blockIdx.x >> 3;
+  const int logical = xcd * (total >> 3) + min(xcd, total & 7) + nth;
+  const int group_size = 8 * tiles_n;
+  const int first_m = (logical / group_size) * 8;
+  const int rows = min(tiles_m - first_m, 8);
+  const int in_group = logical % group_size;
+  const int tm = first_m + in_group % rows, tn = in_group / rows;
+  const int m0 = tm * kNT, n0 = tn * kNF;
+
+  // loader: piece p = wave + kWaves j covers stage rows 8 p .. 8 p + 7 (weight rows first, then
+  // token rows); lane (r, s) = (lane / 8, lane % 8) fills slot s of row r with the row's
+  // segment s ^ ((row / 2) % 8)
+  const uint16_t *src[kPer];
+#pragma unroll
+  for (int j = 0; j < kPer; ++j) {
+    const int row = (wave + kWaves * j) * 8 + (lane >> 3);
+    const int seg = (lane & 7) ^ ((row >> 1) & 7);  // (kNF % 16 == 0: the same for either part)
+    src[j] = row < kNF ? w + (size_t)min(n0 + row, N - 1) * K + seg * 8
+                       : a + (size_t)min(m0 + row - kNF, T - 1) * K + seg * 8;
+  }
+  auto dma = [&](uint8_t *stage, const int k0) {
+#pragma unroll
+    for (int j = 0; j < kPer; ++j)
+      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(src[j] + k0),
+                                       (dma_lptr_t *)(stage + (wave + kWaves * j) * 1024), 16, 0, 0);
+  };
+  // reader: lane (i16, g) wants segment 4 half + g of row i16 of a 16-row tile
+  const uint32_t slot = (uint32_t)(g ^ ((i16 >> 1) & 7));
+  const uint32_t rd_w = (uint32_t)(wn * 16 * WF + i16) * 128 + slot * 16;
+  const uint32_t rd_a = (uint32_t)(kNF + wm * 16 * WT + i16) * 128 + slot * 16;
+  auto read = [&](const uint8_t *stage, const int half, Frag8 (&wf)[WF], Frag8 (&af)[WT]) {
+#pragma unroll
+    for (int x = 0; x < WF; ++x) wf[x].u = *(const u32x4 *)(stage + ((rd_w + x * 2048) ^ (half * 64)));
+#pragma unroll
+    for (int x = 0; x < WT; ++x) af[x].u = *(const u32x4 *)(stage + ((rd_a + x * 2048) ^ (half * 64)));
+  };
+  f32x4 acc[WF][WT];
+#pragma unroll
+  for (int ft = 0; ft < WF; ++ft)
+#pragma unroll
+    for (int tt = 0; tt < WT; ++tt) acc[ft][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  auto mfmas = [&](const Frag8 (&wf)[WF], const Frag8 (&af)[WT]) {
+#pragma unroll
+    for (int ft = 0; ft < WF; ++ft)
+#pragma unroll
+      for (int tt = 0; tt < WT; ++tt) acc[ft][tt] = mfma16x32(wf[ft], af[tt], acc[ft][tt]);
+  };
+
+  const int nk = K / 64;
+  Frag8 wf0[WF], af0[WT], wf1[WF], af1[WT];
+  auto step = [&](uint8_t *cur, uint8_t *nxt, const int i) {
+    read(cur, 1, wf1, af1);
+    mfmas(wf0, af0);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0), lgkmcnt(0): my share of step i + 1 has landed, my reads of `cur` are done
+    __syncthreads();
+    if (i + 2 < nk) dma(cur, (i + 2) * 64);
+    read(nxt, 0, wf0, af0);  // (in the last step: a stage nobody needs, still this workgroup's memory)
+    mfmas(wf1, af1);
+  };
+  dma(stage0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __syncthreads();
+  if (nk > 1) dma(stage1, 64);
+  read(stage0, 0, wf0, af0);
+  for (int i = 0; i < nk; i += 2) {
+    step(stage0, stage1, i);
+    if (i + 1 < nk) step(stage1, stage0, i + 1);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // no load may still be writing this workgroup's LDS when it ends
+
+  // epilogue: the bias of this lane's features once, then token tile by token tile all residual
+  // loads of the tile at once (clamped addresses, so that no load sits under a lane's branch).
+  // (Requesting the residual before the last steps of the loop was measured: slower.)
+  int ncol[WF];
+  float bv[WF][4];
+#pragma unroll
+  for (int ft = 0; ft < WF; ++ft) {
+    ncol[ft] = n0 + wn * 16 * WF + ft * 16 + 4 * g;
+    u32x2 b = {0u, 0u};
+    if (bias) b = *(const u32x2 *)(bias + min(ncol[ft], N - 4));
+    bv[ft][0] = bf16_bits_to_f32(b[0] & 0xffffu);
+    bv[ft][1] = bf16_bits_to_f32(b[0] >> 16);
+    bv[ft][2] = bf16_bits_to_f32(b[1] & 0xffffu);
+    bv[ft][3] = bf16_bits_to_f32(b[1] >> 16);
+  }
+#pragma unroll
+  for (int tt = 0; tt < WT; ++tt) {
+    const int t = m0 + wm * 16 * WT + tt * 16 + i16;
+    const size_t row_off = (size_t)min(t, T - 1) * N;
+    u32x2 rv[WF];
+#pragma unroll
+    for (int ft = 0; ft < WF; ++ft) rv[ft] = u32x2{0u, 0u};
+    if (resid) {
+#pragma unroll
+      for (int ft = 0; ft < WF; ++ft) rv[ft] = *(const u32x2 *)(resid + row_off + min(ncol[ft], N - 4));
+    }
+#pragma unroll
+    for (int ft = 0; ft < WF; ++ft) {
+      const f32x4 c = acc[ft][tt];
+      u32x2 o;
+      o[0] = pack_bf16(c[0] + bv[ft][0] + bf16_bits_to_f32(rv[ft][0] & 0xffffu),
+                       c[1] + bv[ft][1] + bf16_bits_to_f32(rv[ft][0] >> 16));
+      o[1] = pack_bf16(c[2] + bv[ft][2] + bf16_bits_to_f32(rv[ft][1] & 0xffffu),
+                       c[3] + bv[ft][3] + bf16_bits_to_f32(rv[ft][1] >> 16));
+      if (t < T && ncol[ft] < N) *(u32x2 *)(out + row_off + ncol[ft]) = o;
+    }
+  }
+}
+
 int device_cus();  // attn_kernels.hip
 
 hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *bias,
@@ -468,6 +619,25 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
     else
       oproj_skinny_kernel<4, 1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     return hipGetLastError();
+  }
+  // Tiled or wide?  Both cover the output in rounds of workgroups (two 128 x 128 tiles or one
+  // 256 x 192 tile per CU at a time); the wide kernel does 1.45 times the work per unit of time
+  // (measured, 2880 x 4096: 91 against 135 us at 4,216 tokens), so it wins once its rounds are
+  // reasonably full.  EID_OPROJ_KERNEL=wide|tiled overrides the choice (tests, measurements).
+  {
+    const int cus = device_cus();
+    const long tw = (long)((T + 255) / 256) * ((N + 191) / 192);
+    const long tb = (long)((T + 127) / 128) * ((N + 127) / 128);
+    const double wide_cost = (double)((tw + cus - 1) / cus) * (256.0 * 192.0);
+    const double tiled_cost = (double)((tb + 2 * cus - 1) / (2 * cus)) * (2.0 * 128.0 * 128.0) * 1.45;
+    bool wide = 4 * tb >= 3 * cus && wide_cost < tiled_cost;
+    if (const char *e = getenv("EID_OPROJ_KERNEL")) wide = e[0] == 'w' ? true : e[0] == 't' ? false : wide;
+    if (wide) {
+      const int tiles_m = (T + 255) / 256, tiles_n = (N + 191) / 192;
+      oproj_wide_kernel<6, 4, 2, 4><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                      tiles_m, tiles_n);
+      return hipGetLastError();
+    }
   }
   // The 128 x 128 tile once it gives most CUs a workgroup, else 64 x 64 (measured
   // crossover for 2880 x 4096: between 1,024 and 1,500 tokens, 184 and 276 big tiles).

@@ -99,14 +99,42 @@ def test_tiled_kernel_shapes(G, T, N, K, with_bias, with_res):
     _run(G, T, N, K, with_bias, with_res, seed=T + K)
 
 
+@pytest.mark.parametrize("T,N,K", [(65, 2880, 4096), (128, 128, 64), (129, 16, 128), (200, 144, 576),
+                                   (257, 2880, 512), (1000, 1040, 1024), (513, 208, 192),
+                                   (2790, 1648, 192)])
+@pytest.mark.parametrize("with_bias,with_res", [(False, False), (True, True)])
+def test_wide_kernel_shapes(G, monkeypatch, T, N, K, with_bias, with_res):
+    # the 256 x 192 kernel forced onto shapes it would not be chosen for: ragged token and
+    # feature tiles, one and many K steps (odd and even counts), a single workgroup
+    monkeypatch.setenv("EID_OPROJ_KERNEL", "wide")
+    _run(G, T, N, K, with_bias, with_res, seed=T + K + 1)
+
+
+def test_wide_and_tiled_kernels_agree(G, monkeypatch):
+    a = synth.normal_bf16((700, 1024), 21, synth.TID_Q)
+    w = synth.normal_bf16((400, 1024), 21, synth.TID_K)
+    a_d, w_d = G.bf16_dev(a), G.bf16_dev(w)
+    monkeypatch.setenv("EID_OPROJ_KERNEL", "tiled")
+    o_t = G.bits_host(ea.o_proj(a_d, w_d))
+    monkeypatch.setenv("EID_OPROJ_KERNEL", "wide")
+    o_w = G.bits_host(ea.o_proj(a_d, w_d))
+    torch.cuda.synchronize()
+    # the same products summed in the same K order by the same MFMA: bit for bit
+    assert np.array_equal(o_t, o_w)
+
+
 @pytest.mark.parametrize("T", [33, 300])
 def test_residual_updated_in_place(G, T):
     _run(G, T, 2880, 4096, True, True, inplace=True)
 
 
 def test_prefill_sized_batch_against_the_oracle(G):
-    # the bench workload's shape for a chunked-prefill step (4,216 tokens)
+    # the bench workload's shape for a chunked-prefill step (4,216 tokens): the wide kernel
     _run(G, 4216, 2880, 4096, True, True, seed=12)
+
+
+def test_prefill_sized_batch_in_place(G):
+    _run(G, 2600, 2880, 4096, True, True, seed=13, inplace=True)
 
 
 def test_both_kernels_agree_across_the_switch(G):
