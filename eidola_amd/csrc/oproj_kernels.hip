@@ -22,9 +22,10 @@
 //   oproj_tiled_kernel   any T.  128 x 128 (or, for batches too small to fill the device
 //                        with that, 64 x 64) tokens x features per workgroup, K in steps of
 //                        64 through double-buffered, row-padded LDS tiles.
-//   oproj_wide_kernel    prefill-sized T (thousands of tokens).  256 tokens x 192 features per
-//                        workgroup, one workgroup of 8 waves per CU, K in steps of 64 through
-//                        two LDS stages filled by direct global -> LDS loads.
+//   oproj_wide_kernel    T above ~1,000.  K in steps of 64 through two LDS stages filled by
+//                        direct global -> LDS loads; 128 x 128 tokens x features per workgroup
+//                        of 4 waves, two workgroups per CU, or (when that fills whole rounds of
+//                        the device better) 256 x 192 per workgroup of 8 waves, one per CU.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -62,6 +63,48 @@ __device__ __forceinline__ void oproj_store(const f32x4 acc, const uint16_t *bia
   o[0] = pack_bf16(v[0], v[1]);
   o[1] = pack_bf16(v[2], v[3]);
   *(u32x2 *)(out + row_off + n) = o;
+}
+
+// Epilogue of the tiled kernels: acc[ft][tt] holds features n_lane + 16 ft .. + 3 of token
+// t_lane + 16 tt.  The bias of this lane's features once, then token tile by token tile all
+// residual loads of the tile at once (clamped addresses, so that no load sits under a lane's
+// branch and none waits for the one before), bf16 rounding, 8-byte stores.
+template <int WF, int WT>
+__device__ __forceinline__ void oproj_epilogue(const f32x4 (&acc)[WF][WT], const uint16_t *bias,
+                                               const uint16_t *resid, uint16_t *out, const int T,
+                                               const int N, const int t_lane, const int n_lane) {
+  float bv[WF][4];
+#pragma unroll
+  for (int ft = 0; ft < WF; ++ft) {
+    u32x2 b = {0u, 0u};
+    if (bias) b = *(const u32x2 *)(bias + min(n_lane + 16 * ft, N - 4));
+    bv[ft][0] = bf16_bits_to_f32(b[0] & 0xffffu);
+    bv[ft][1] = bf16_bits_to_f32(b[0] >> 16);
+    bv[ft][2] = bf16_bits_to_f32(b[1] & 0xffffu);
+    bv[ft][3] = bf16_bits_to_f32(b[1] >> 16);
+  }
+#pragma unroll
+  for (int tt = 0; tt < WT; ++tt) {
+    const int t = t_lane + 16 * tt;
+    const size_t row_off = (size_t)min(t, T - 1) * N;
+    u32x2 rv[WF];
+#pragma unroll
+    for (int ft = 0; ft < WF; ++ft) rv[ft] = u32x2{0u, 0u};
+    if (resid) {
+#pragma unroll
+      for (int ft = 0; ft < WF; ++ft) rv[ft] = *(const u32x2 *)(resid + row_off + min(n_lane + 16 * ft, N - 4));
+    }
+#pragma unroll
+    for (int ft = 0; ft < WF; ++ft) {
+      const f32x4 c = acc[ft][tt];
+      u32x2 o;
+      o[0] = pack_bf16(c[0] + bv[ft][0] + bf16_bits_to_f32(rv[ft][0] & 0xffffu),
+                       c[1] + bv[ft][1] + bf16_bits_to_f32(rv[ft][0] >> 16));
+      o[1] = pack_bf16(c[2] + bv[ft][2] + bf16_bits_to_f32(rv[ft][1] & 0xffffu),
+                       c[3] + bv[ft][3] + bf16_bits_to_f32(rv[ft][1] >> 16));
+      if (t < T && n_lane + 16 * ft < N) *(u32x2 *)(out + row_off + n_lane + 16 * ft) = o;
+    }
+  }
 }
 
 constexpr int kSkWaves = 8;
@@ -430,20 +473,11 @@ __global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
     if (i + 1 < nk) step(1, i + 1);
   }
 
-#pragma unroll
-  for (int tt = 0; tt < WT; ++tt) {
-    const int t = m0 + wm * kWave + tt * 16 + i16;
-    if (t >= T) continue;
-#pragma unroll
-    for (int ft = 0; ft < WT; ++ft) {
-      const int n = n0 + wn * kWave + ft * 16 + 4 * g;
-      if (n < N) oproj_store(acc[ft][tt], bias, resid, out, (size_t)t * N, n);
-    }
-  }
+  oproj_epilogue<WT, WT>(acc, bias, resid, out, T, N, m0 + wm * kWave + i16, n0 + wn * kWave + 4 * g);
 }
 
 // ---------------------------------------------------------------------------------------
-// Wide kernel (prefill-sized batches).  One workgroup per CU; workgroup tile = 16 WT WM tokens
+// Wide kernel (prefill-sized batches).  OCC workgroups per CU; workgroup tile = 16 WT WM tokens
 // x 16 WF WN features, wave (wm, wn) owns 16 WT tokens x 16 WF features.  K advances 64
 // elements per step through two LDS stages that the loads fill directly
 // (global_load_lds_dwordx4: a wave instruction moves 8 rows x 128 bytes, no registers), the
@@ -459,8 +493,8 @@ typedef __attribute__((address_space(1))) const void dma_gptr_t;
 typedef __attribute__((address_space(3))) void dma_lptr_t;
 }  // namespace
 
-template <int WF, int WT, int WN, int WM>
-__global__ __launch_bounds__(64 * WN * WM, 1) void oproj_wide_kernel(
+template <int WF, int WT, int WN, int WM, int OCC>
+__global__ __launch_bounds__(64 * WN * WM, OCC) void oproj_wide_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
     uint16_t *out, const int T, const int N, const int K, const int tiles_m,
@@ -549,43 +583,7 @@ __global__ __launch_bounds__(64 * WN * WM, 1) void oproj_wide_kernel(
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // no load may still be writing this workgroup's LDS when it ends
 
-  // epilogue: the bias of this lane's features once, then token tile by token tile all residual
-  // loads of the tile at once (clamped addresses, so that no load sits under a lane's branch).
-  // (Requesting the residual before the last steps of the loop was measured: slower.)
-  int ncol[WF];
-  float bv[WF][4];
-#pragma unroll
-  for (int ft = 0; ft < WF; ++ft) {
-    ncol[ft] = n0 + wn * 16 * WF + ft * 16 + 4 * g;
-    u32x2 b = {0u, 0u};
-    if (bias) b = *(const u32x2 *)(bias + min(ncol[ft], N - 4));
-    bv[ft][0] = bf16_bits_to_f32(b[0] & 0xffffu);
-    bv[ft][1] = bf16_bits_to_f32(b[0] >> 16);
-    bv[ft][2] = bf16_bits_to_f32(b[1] & 0xffffu);
-    bv[ft][3] = bf16_bits_to_f32(b[1] >> 16);
-  }
-#pragma unroll
-  for (int tt = 0; tt < WT; ++tt) {
-    const int t = m0 + wm * 16 * WT + tt * 16 + i16;
-    const size_t row_off = (size_t)min(t, T - 1) * N;
-    u32x2 rv[WF];
-#pragma unroll
-    for (int ft = 0; ft < WF; ++ft) rv[ft] = u32x2{0u, 0u};
-    if (resid) {
-#pragma unroll
-      for (int ft = 0; ft < WF; ++ft) rv[ft] = *(const u32x2 *)(resid + row_off + min(ncol[ft], N - 4));
-    }
-#pragma unroll
-    for (int ft = 0; ft < WF; ++ft) {
-      const f32x4 c = acc[ft][tt];
-      u32x2 o;
-      o[0] = pack_bf16(c[0] + bv[ft][0] + bf16_bits_to_f32(rv[ft][0] & 0xffffu),
-                       c[1] + bv[ft][1] + bf16_bits_to_f32(rv[ft][0] >> 16));
-      o[1] = pack_bf16(c[2] + bv[ft][2] + bf16_bits_to_f32(rv[ft][1] & 0xffffu),
-                       c[3] + bv[ft][3] + bf16_bits_to_f32(rv[ft][1] >> 16));
-      if (t < T && ncol[ft] < N) *(u32x2 *)(out + row_off + ncol[ft]) = o;
-    }
-  }
+  oproj_epilogue<WF, WT>(acc, bias, resid, out, T, N, m0 + wm * 16 * WT + i16, n0 + wn * 16 * WF + 4 * g);
 }
 
 int device_cus();  // attn_kernels.hip
@@ -620,22 +618,31 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
       oproj_skinny_kernel<4, 1><<<grid, block, 0, st>>>(a, w, bias, resid, out, T, N, K);
     return hipGetLastError();
   }
-  // Tiled or wide?  Both cover the output in rounds of workgroups (two 128 x 128 tiles or one
-  // 256 x 192 tile per CU at a time); the wide kernel does 1.45 times the work per unit of time
-  // (measured, 2880 x 4096: 91 against 135 us at 4,216 tokens), so it wins once its rounds are
-  // reasonably full.  EID_OPROJ_KERNEL=wide|tiled overrides the choice (tests, measurements).
+  // Which tiling?  Every kernel covers the output in rounds of workgroups, and a workgroup that
+  // walks all of K takes about as long whatever its tile (the K steps' load latency): measured
+  // for 2880 x 4096, a round of the 256 x 192 kernel (one workgroup per CU) takes ~85 us and a
+  // round of the direct-to-LDS 128 x 128 kernel (two per CU) ~63 us.  The cheaper plan wins;
+  // batches too small to give three quarters of the CUs a 128 x 128 tile take 64 x 64 tiles.
+  // EID_OPROJ_KERNEL=wide|mid|tiled overrides the choice (tests, measurements); "tiled" is the
+  // register-staged kernel that the direct-to-LDS ones replaced above ~1,000 tokens.
   {
     const int cus = device_cus();
     const long tw = (long)((T + 255) / 256) * ((N + 191) / 192);
     const long tb = (long)((T + 127) / 128) * ((N + 127) / 128);
-    const double wide_cost = (double)((tw + cus - 1) / cus) * (256.0 * 192.0);
-    const double tiled_cost = (double)((tb + 2 * cus - 1) / (2 * cus)) * (2.0 * 128.0 * 128.0) * 1.45;
-    bool wide = 4 * tb >= 3 * cus && wide_cost < tiled_cost;
-    if (const char *e = getenv("EID_OPROJ_KERNEL")) wide = e[0] == 'w' ? true : e[0] == 't' ? false : wide;
-    if (wide) {
+    const double wide_cost = (double)((tw + cus - 1) / cus) * 85.0;
+    const double mid_cost = (double)((tb + 2 * cus - 1) / (2 * cus)) * 63.0;
+    int plan = 4 * tb < 3 * cus ? 0 : wide_cost < mid_cost ? 2 : 1;  // 0 = 64 x 64 tiles, 1 = mid, 2 = wide
+    if (const char *e = getenv("EID_OPROJ_KERNEL")) plan = e[0] == 'w' ? 2 : e[0] == 'm' ? 1 : e[0] == 't' ? 0 : plan;
+    if (plan == 2) {
       const int tiles_m = (T + 255) / 256, tiles_n = (N + 191) / 192;
-      oproj_wide_kernel<6, 4, 2, 4><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                                      tiles_m, tiles_n);
+      oproj_wide_kernel<6, 4, 2, 4, 1><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                         tiles_m, tiles_n);
+      return hipGetLastError();
+    }
+    if (plan == 1) {
+      const int tiles_m = (T + 127) / 128, tiles_n = (N + 127) / 128;
+      oproj_wide_kernel<4, 4, 2, 2, 2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                         tiles_m, tiles_n);
       return hipGetLastError();
     }
   }

@@ -103,10 +103,12 @@ def test_tiled_kernel_shapes(G, T, N, K, with_bias, with_res):
                                    (257, 2880, 512), (1000, 1040, 1024), (513, 208, 192),
                                    (2790, 1648, 192)])
 @pytest.mark.parametrize("with_bias,with_res", [(False, False), (True, True)])
-def test_wide_kernel_shapes(G, monkeypatch, T, N, K, with_bias, with_res):
-    # the 256 x 192 kernel forced onto shapes it would not be chosen for: ragged token and
-    # feature tiles, one and many K steps (odd and even counts), a single workgroup
-    monkeypatch.setenv("EID_OPROJ_KERNEL", "wide")
+@pytest.mark.parametrize("kernel", ["wide", "mid"])
+def test_wide_kernel_shapes(G, monkeypatch, kernel, T, N, K, with_bias, with_res):
+    # the direct-to-LDS kernels (256 x 192 and 128 x 128 tiles) forced onto shapes they would
+    # not be chosen for: ragged token and feature tiles, one and many K steps (odd and even
+    # counts), a single workgroup
+    monkeypatch.setenv("EID_OPROJ_KERNEL", kernel)
     _run(G, T, N, K, with_bias, with_res, seed=T + K + 1)
 
 
@@ -118,9 +120,11 @@ def test_wide_and_tiled_kernels_agree(G, monkeypatch):
     o_t = G.bits_host(ea.o_proj(a_d, w_d))
     monkeypatch.setenv("EID_OPROJ_KERNEL", "wide")
     o_w = G.bits_host(ea.o_proj(a_d, w_d))
+    monkeypatch.setenv("EID_OPROJ_KERNEL", "mid")
+    o_m = G.bits_host(ea.o_proj(a_d, w_d))
     torch.cuda.synchronize()
     # the same products summed in the same K order by the same MFMA: bit for bit
-    assert np.array_equal(o_t, o_w)
+    assert np.array_equal(o_t, o_w) and np.array_equal(o_t, o_m)
 
 
 @pytest.mark.parametrize("T", [33, 300])
@@ -134,7 +138,7 @@ def test_prefill_sized_batch_against_the_oracle(G):
 
 
 def test_prefill_sized_batch_in_place(G):
-    _run(G, 2600, 2880, 4096, True, True, seed=13, inplace=True)
+    _run(G, 2600, 2880, 4096, True, True, seed=13, inplace=True)  # (128 x 128 direct-to-LDS tiles)
 
 
 def test_both_kernels_agree_across_the_switch(G):
