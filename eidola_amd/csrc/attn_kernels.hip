@@ -316,9 +316,13 @@ constexpr int pipe_cost_before(const int op, const int pre) {
   return c;
 }
 
-template <int VROW>
-__device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile_stride,
-                                           const uint8_t *v_rd, const uint8_t *q_rd,
+// SWZ: the tiles were written by direct global -> LDS loads: 128-byte rows whose 16-byte
+// segments are permuted (K: by (row / 2) % 8; V: pairs of segments by (row / 2) % 4).  The
+// second half of a lane's K operand is then at `k_rd ^ 16` (passed as k_rd_hi) and V's dim
+// tile mt at byte (32 mt) ^ v_sw of its row.
+template <int VROW, bool SWZ = false>
+__device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const uint8_t *k_rd_hi, const int k_tile_stride,
+                                           const uint8_t *v_rd, const int v_sw, const uint8_t *q_rd,
                                            bool &maybe_fresh, float (&m)[4], f32x4 (&zs)[4],
                                            float (&l)[4], f32x4 (&acc)[4][4], const RowInfo &ri,
                                            const int tc, const bool need_mask) {
@@ -340,14 +344,15 @@ __device__ __forceinline__ void chunk_pipe(const uint8_t *k_rd, const int k_tile
   for (int b = 0; b < 4; ++b) kf[b][0].u = *(const u32x4 *)(k_rd + b * k_tile_stride);
   read_q(IC<0>{});
 #pragma unroll
-  for (int b = 0; b < 4; ++b) kf[b][1].u = *(const u32x4 *)(k_rd + b * k_tile_stride + 16);
+  for (int b = 0; b < 4; ++b) kf[b][1].u = *(const u32x4 *)(k_rd_hi + b * k_tile_stride);
   read_q(IC<1>{});
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr) {
-      const u32x2 a = lds_read_tr16(v_rd + (2 * pr) * (kBlock * VROW) + 32 * mt);
-      const u32x2 b2 = lds_read_tr16(v_rd + (2 * pr + 1) * (kBlock * VROW) + 32 * mt);
+      const uint8_t *v_mt = v_rd + (SWZ ? (32 * mt) ^ v_sw : 32 * mt);
+      const u32x2 a = lds_read_tr16(v_mt + (2 * pr) * (kBlock * VROW));
+      const u32x2 b2 = lds_read_tr16(v_mt + (2 * pr + 1) * (kBlock * VROW));
       vf[mt][pr].w[0] = a[0];
       vf[mt][pr].w[1] = a[1];
       vf[mt][pr].w[2] = b2[0];
@@ -1360,6 +1365,8 @@ __global__ __launch_bounds__(kShortWaves * 64, (NT == 1 ? 4 : 2)) void shortspan
 // each batch of 64 sequences the longest come first, and within a sequence the latest
 // (heaviest) tile comes first, so the long-running workgroups start early.
 // ---------------------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void pf_gptr_t;
+typedef __attribute__((address_space(3))) void pf_lptr_t;
 constexpr int kPfWaves = 4;
 constexpr int kPfWaveTok = 8;                     // query tokens per wave (x 8 heads = 64 rows)
 constexpr int kPfTok = kPfWaves * kPfWaveTok;     // query tokens per workgroup
@@ -1423,8 +1430,19 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
                                                                    const PfTable tab) {
   constexpr int NT = 4;
   constexpr int kElt = FP8 ? 1 : 2;
-  __shared__ __align__(16) uint8_t lds_k[2][kPfKTileBytes];  // double-buffered K tile
-  __shared__ __align__(16) uint8_t lds_v[2][kPfVTileBytes];  // double-buffered V tile
+  // DMA (bf16 cache, folded softmax factor): the K/V tiles go straight from the pages into LDS
+  // (global_load_lds_dwordx4: a wave instruction moves 8 token rows x 128 bytes of one KV head),
+  // no staging registers, no ds_write; 128-byte rows with permuted segments (see chunk_pipe).
+  // Four separate arrays: the compiler can then tell the tile being loaded from the one being
+  // read and puts no wait for the loads in front of the reads.
+  constexpr bool DMA = PRE && !FP8;
+  constexpr int kDmaTile = kChunk * 128;
+  __shared__ __align__(16) uint8_t lds_k[2][DMA ? 16 : kPfKTileBytes];  // double-buffered K tile
+  __shared__ __align__(16) uint8_t lds_v[2][DMA ? 16 : kPfVTileBytes];  // double-buffered V tile
+  __shared__ __align__(1024) uint8_t dma_k0[DMA ? kDmaTile : 16];
+  __shared__ __align__(1024) uint8_t dma_k1[DMA ? kDmaTile : 16];
+  __shared__ __align__(1024) uint8_t dma_v0[DMA ? kDmaTile : 16];
+  __shared__ __align__(1024) uint8_t dma_v1[DMA ? kDmaTile : 16];
   // PRE: every wave's eight Q fragments, in fragment order (see chunk_pipe)
   __shared__ __align__(16) uint8_t lds_q[PRE ? kPfWaves * 8 * kQFragBytes : 16];
   __shared__ int item_lds[8];
@@ -1560,9 +1578,35 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     *(u32x4 *)(&lds_v[buf][st_off_v + 16]) = v1;
   };
 
+  // DMA loader: wave w moves the chunk's page w (tile rows 16 w .. 16 w + 15) as two pieces of
+  // 8 rows per tensor; lane (r, sl) = (lane / 8, lane % 8) fills slot sl of its row.  Rows past
+  // the sequence end repeat its last row (real, finite data; their scores are masked), as the
+  // pages behind them may never have been written.
+  const int dma_r = lane >> 3, dma_sl = lane & 7;
+  auto dma = [&](uint8_t *kbuf, uint8_t *vbuf, const int tc) {
+    const int blk = clamp_page(bt[min(tc / kBlock + wave, nblk_total - 1)], p.last_block);
+    const uint8_t *kp = p.k_cache + (size_t)blk * page_bytes + (uint32_t)kvh * 128;
+    const uint8_t *vp = p.v_cache + (size_t)blk * page_bytes + (uint32_t)kvh * 128;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int row = 8 * h + dma_r;  // row of the page = tile row - 16 wave
+      const int tok = min(tc + 16 * wave + row, L - 1);
+      const uint32_t off = (uint32_t)(tok & 15) * row_bytes;
+      const int kseg = dma_sl ^ (4 * h + (dma_r >> 1));
+      const int vseg = dma_sl ^ ((dma_r >> 1) << 1);
+      __builtin_amdgcn_global_load_lds((pf_gptr_t *)(kp + off + kseg * 16),
+                                       (pf_lptr_t *)(kbuf + (2 * wave + h) * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((pf_gptr_t *)(vp + off + vseg * 16),
+                                       (pf_lptr_t *)(vbuf + (2 * wave + h) * 1024), 16, 0, 0);
+    }
+  };
+
   // the first K/V tile is requested before the Q operands: both are in flight together
   timeline_mark(p, tl_slot, 0);
-  if (t_begin < t_end) fetch(t_begin);
+  if (t_begin < t_end) {
+    if constexpr (DMA) dma(dma_k0, dma_v0, t_begin);
+    else fetch(t_begin);
+  }
 
   Frag8 qf[NT][2];
   RowInfo ri;
@@ -1590,6 +1634,30 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
+  if constexpr (DMA) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's share of the first tile is in LDS
+    __syncthreads();
+    timeline_mark(p, tl_slot, 1);
+    const int sw_k = (i16 >> 1) & 7;
+    const uint32_t k_off = (uint32_t)i16 * 128 + (uint32_t)((2 * g) ^ sw_k) * 16;
+    const int v_row = 4 * g + (i16 >> 2);
+    const uint32_t v_off = (uint32_t)v_row * 128 + 8 * (i16 & 3);
+    const int v_sw = 32 * ((v_row >> 1) & 3);
+    auto iter = [&](uint8_t *kcur, uint8_t *vcur, uint8_t *knxt, uint8_t *vnxt, const int tc) {
+      if (tc + kChunk < t_end) dma(knxt, vnxt, tc + kChunk);
+      if (wave_active && tc <= pos_last && tc + kChunk > lo_first) {
+        const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
+        chunk_pipe<128, true>(kcur + k_off, kcur + (k_off ^ 16), kBlock * 128, vcur + v_off, v_sw, q_lds,
+                              maybe_fresh, m, zs, lsum, acc, ri, tc, need_mask);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): my share of the next tile has landed
+      __syncthreads();
+    };
+    for (int tc = t_begin; tc < t_end; tc += 2 * kChunk) {
+      iter(dma_k0, dma_v0, dma_k1, dma_v1, tc);
+      if (tc + kChunk < t_end) iter(dma_k1, dma_v1, dma_k0, dma_v0, tc + kChunk);
+    }
+  } else {
   if (t_begin < t_end) stash(t_begin, 0);
   __syncthreads();
   timeline_mark(p, tl_slot, 1);
@@ -1602,8 +1670,8 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
       const uint8_t *v_rd = &lds_v[cur][0] + (4 * g + (i16 >> 2)) * kPfVRowBytes + 8 * (i16 & 3);
       const bool need_mask = (tc < lo_last) || (tc + kChunk > pos_first + 1);
       if constexpr (PRE) {
-        chunk_pipe<kPfVRowBytes>(kt, kBlock * kPfKRowBytes, v_rd, q_lds, maybe_fresh, m, zs, lsum, acc, ri,
-                                 tc, need_mask);
+        chunk_pipe<kPfVRowBytes>(kt, kt + 16, kBlock * kPfKRowBytes, v_rd, 0, q_lds, maybe_fresh, m, zs, lsum,
+                                 acc, ri, tc, need_mask);
       } else {
         Frag8 kf[4][2];
 #pragma unroll
@@ -1616,6 +1684,7 @@ __global__ __launch_bounds__(kPfWaves * 64, 2) void prefill_kernel(const AttnPar
     }
     if (has_next) stash(tc + kChunk, cur ^ 1);
     __syncthreads();
+  }
   }
   timeline_mark(p, tl_slot, 2);
   if (!wave_active) return;
