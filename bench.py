@@ -967,7 +967,7 @@ def main():
                     help="experiment: no host-side lengths for the library (desc.sum_kv_len = 0, no "
                          "seq_lens_host): the kernels size and plan the launch themselves")
     ap.add_argument("--only", default="",
-                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack,overlap "
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack,overlap,gather,timeline "
                          "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
