@@ -789,6 +789,39 @@ def gather_bench(torch, ea, synth, np):
         log(f"[bench] gather probe, {kind} pages, {ppw} per workgroup ({nwg} workgroups, {lds} KiB LDS, a wave reads {'whole rows' if rows else 'one head'}), {delay} ALU "
             f"links per batch: {ms*1e3:.1f} us for {nbytes/1e6:.1f} MB = {r['GBps']:.0f} GB/s = {100*r['GBps']/HBM_PEAK_GBS:.1f}% of peak")
         res.append(r)
+    # the same access patterns against pages that stay in cache (64 distinct pages, 2 MiB of K and
+    # V): what one CU's vector memory path takes in per unit of time, by the shape of a wave's read
+    rng = np.random.default_rng(1)
+    for nwg, rows in ((256, 0), (256, 1), (1, 0), (1, 1)):
+        ppw = 256
+        tab = torch.from_numpy(rng.integers(0, 64, size=nwg * ppw, dtype=np.int32)).to("cuda:0")
+
+        def run_c(i):
+            assert lib.eid_probe_gather(w.k_cache.data_ptr(), w.v_cache.data_ptr(), tab.data_ptr(), nwg, ppw, 0,
+                                        75 * 1024, rows, sink.data_ptr(), st) == 0
+        for i in range(3):
+            run_c(i)
+        ms = event_ms(run_c, 10, torch)
+        nbytes = nwg * ppw * 2 * 16384
+        per_cu = nbytes / ms / 1e6 / min(nwg, 256)
+        log(f"[bench] gather probe, 64 cache-resident pages, {nwg} workgroups, a wave reads "
+            f"{'whole rows' if rows else 'one head'}: {ms*1e3:.1f} us = {per_cu:.1f} GB/s per CU")
+        res.append({"config": f"gather_probe_cached_{nwg}_wg_{'rows' if rows else 'heads'}", "ms": ms,
+                    "GBps_per_cu": per_cu})
+    # LDS fragment reads (probe_lds.hip)
+    lib.eid_probe_lds_read.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+    lib.eid_probe_lds_read.restype = C.c_int
+    iters = 2000
+    for mode, name in ((0, "linear"), (1, "128-byte rows, permuted segments"), (2, "144-byte rows")):
+        for threads in (256, 512, 1024):
+            def run_l(i):
+                assert lib.eid_probe_lds_read(mode, 256, threads, iters, sink.data_ptr(), st) == 0
+            run_l(0)
+            ms = event_ms(run_l, 3, torch)
+            per_cu = iters * 16 * (threads // 64) * 1024 / ms / 1e6  # GB/s
+            log(f"[bench] LDS read probe, {name}, {threads // 64} waves per CU: {ms*1e3:.1f} us, "
+                f"{per_cu:.0f} GB/s per CU = {per_cu / 2.4:.0f} B/clk at 2.4 GHz")
+            res.append({"config": f"lds_read_probe_mode{mode}_{threads}", "ms": ms, "GBps_per_cu": per_cu})
     return res
 
 
