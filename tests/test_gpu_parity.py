@@ -166,6 +166,21 @@ def test_garbage_beyond_sequence_end_is_never_used(G):
     assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "poison tail")
 
 
+def test_prefill_rows_never_use_garbage_beyond_sequence_end(G):
+    """The prefill kernel loads whole 64-token tiles: the rows of a tile past seq_len (unwritten
+    slots of the last page, NaN patterns here, and pages the table does not even hold) must not
+    reach the output, with and without an lse (the two softmax variants load tiles differently)."""
+    b = make_batch([45, 100, 333, 1000], [40, 64, 200, 9])
+    q, k, v, sinks = logical_tensors(b, seed=31)
+    kc, vc = cpu_caches(b, k, v)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    ref, lse = oracle_out(b, q, kc, vc, sinks)
+    assert_close(G.run_attn(b, q, kc_d, vc_d, sinks), ref, "prefill poison tail")
+    out, lse_gpu = G.run_attn(b, q, kc_d, vc_d, sinks, return_lse=True)
+    assert_close(out, ref, "prefill poison tail, lse asked for")
+    assert np.all(np.isfinite(lse_gpu))
+
+
 # ---------------------------------------------------------------- varlen: verify rows
 @pytest.mark.parametrize("window", [0, 128])
 @pytest.mark.parametrize("partition", [0, 512])
