@@ -15,6 +15,7 @@
 #include <atomic>
 #include "eid_device.h"
 #include "eid_params.h"
+#include <hip/hip_ext.h>
 
 #include <cstdio>
 #include <cstdlib>
@@ -2188,6 +2189,16 @@ static unsigned long long *timeline_for(const long long waves) {
   return waves <= g_timeline_entries ? g_timeline : nullptr;
 }
 
+// Measurement aid: a pair of HIP events that the next decode launches with a host-listed item
+// table attach to the split-KV kernel's own dispatch (hipExtLaunchKernelGGL): the time between
+// them is the kernel's duration as a profiler reports it, without the gaps that events recorded
+// around a launch include.  Null: off.  Not thread-safe.
+static hipEvent_t g_kernel_start = nullptr, g_kernel_stop = nullptr;
+void set_kernel_events(void *start, void *stop) {
+  g_kernel_start = static_cast<hipEvent_t>(start);
+  g_kernel_stop = static_cast<hipEvent_t>(stop);
+}
+
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same
 // params so that it uses the same partition.
@@ -2200,6 +2211,11 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   if (tab && ntiles == 1 && p.nparts_max > 1 && !p.dynamic_partition && !p.share_cus &&
       waves_for(p.num_kv_heads) == 8) {
     dim3 grid((unsigned)tab->n, p.num_kv_heads / 8);
+    if (g_kernel_start && g_kernel_stop && !fp8) {
+      void *kargs[] = {const_cast<AttnParams *>(&p), const_cast<ItemTable *>(tab)};
+      return hipExtLaunchKernel(reinterpret_cast<const void *>(splitkv_table_kernel<1, false, 8>), grid, dim3(512),
+                                kargs, 0, st, g_kernel_start, g_kernel_stop, 0);
+    }
     if (fp8 && p.fp8_pair) splitkv_table_kernel<1, true, 4, true><<<grid, 256, 0, st>>>(p, *tab);
     else if (fp8) splitkv_table_kernel<1, true, 8><<<grid, 512, 0, st>>>(p, *tab);
     else splitkv_table_kernel<1, false, 8><<<grid, 512, 0, st>>>(p, *tab);

@@ -22,6 +22,7 @@ long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, in
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
                           const PfTable *tab);
 void set_timeline(void *buf, long long entries);
+void set_kernel_events(void *start, void *stop);
 bool build_prefill_table(const AttnParams &p, const int32_t *seq_lens_host,
                          const int32_t *cu_seqlens_q_host, PfTable *tab);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
@@ -601,6 +602,10 @@ uint32_t eid_version(void) { return (EID_VERSION_MAJOR << 16) | EID_VERSION_MINO
 const char *eid_last_error(void) { return g_err; }
 
 void eid_debug_set_timeline(void *device_buf, int64_t entries) { eid::set_timeline(device_buf, entries); }
+
+void eid_debug_set_kernel_events(void *start_event, void *stop_event) {
+  eid::set_kernel_events(start_event, stop_event);
+}
 
 int32_t eid_partition_size(const eid_attn_desc *desc) {
   if (check_attn_desc(desc)) return 0;

@@ -751,6 +751,36 @@ def test_host_copies_of_the_lengths_plan_the_launches(G, kv_dtype, window, parti
     assert np.array_equal(both, out)   # the sum adds nothing the arrays do not say
 
 
+def test_kernel_events_time_the_split_kv_dispatch(G):
+    """eid_debug_set_kernel_events: a decode call on the host-listed path attaches the two events
+    to the split-KV kernel's dispatch; the outputs do not change, the time between the events is
+    a kernel's worth, and once switched off the events are left alone."""
+    from eidola_amd import _lib
+    lib = _lib.load_library()
+    rng = np.random.default_rng(77)
+    seq_lens = rng.integers(3000, 9000, size=24)
+    b = make_batch(seq_lens, [1] * len(seq_lens), partition=0)
+    q, k, v, sinks = logical_tensors(b, seed=9)
+    kc_d, vc_d = G.gpu_caches(b, k, v)
+    plain = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=True, hint=True)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    e1.record()
+    torch.cuda.synchronize()
+    lib.eid_debug_set_kernel_events(e0.cuda_event, e1.cuda_event)
+    try:
+        timed = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=True, hint=True)
+    finally:
+        lib.eid_debug_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    assert np.array_equal(timed, plain)
+    ms = e0.elapsed_time(e1)
+    assert 0.005 < ms < 5.0, ms    # ~0.3 GB of KV: tens of microseconds, not the back-to-back records
+    again = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=True, hint=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(again, plain) and e0.elapsed_time(e1) == ms
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_seeded_small_batches_with_long_contexts(G, seed):
     """One to six sequences with contexts drawn log-uniformly up to 20,000 tokens: the
