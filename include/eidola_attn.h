@@ -17,7 +17,8 @@
  *    queried on first use; per calling thread and device, one helper stream and two events,
  *    created by the thread's first mixed prefill + decode call of eid_attn_varlen and
  *    destroyed when the thread ends; per device, the static workspace of
- *    eid_attn_decode_noalloc.
+ *    eid_attn_decode_noalloc; per process, what the eid_debug_* measurement aids were last
+ *    given (a buffer pointer, two events; all null unless a measurement set them).
  *  - All work is enqueued asynchronously on the caller's `hipStream_t`
  *    (passed as `void *`; NULL = the default stream).
  *  - Every function returns an `eid_status` (0 = OK, negative = error) and never
