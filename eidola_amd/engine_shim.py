@@ -16,11 +16,14 @@ embedding, paged KV cache managed by eidola_amd.Scheduler, sink attention throug
 kernels, output projection, residual) with seeded random weights, a byte-level tokenizer and
 greedy sampling.  No checkpoint is read (none exists on the box), there is no MLP / MoE and
 no learned norm, so the text it produces is deterministic noise; the request handling, the
-continuous use of the scheduler and the kernels per generated token are real.
+continuous batching of concurrent requests through the scheduler (prefill chunks and decode
+rows of different requests in one ragged attention call per layer) and the kernels per
+generated token are real.
 `--engine fake` swaps the model for a CPU echo so the HTTP layer can be tested anywhere.
 """
 import argparse
 import json
+import queue
 import threading
 import time
 import uuid
@@ -59,11 +62,31 @@ class FakeEngine:
             yield EOS
 
 
+class _Request:
+    """One generation in flight inside SyntheticAttentionEngine."""
+
+    def __init__(self, seq_id, prompt_ids, max_new_tokens):
+        self.seq_id, self.prompt, self.budget = seq_id, prompt_ids, max_new_tokens
+        self.fed = 0              # prompt tokens already in the KV cache
+        self.last = None          # the sampled token to feed next
+        self.produced = 0
+        self.out = queue.Queue()  # tokens, then _DONE (or an exception to re-raise)
+
+
+_DONE = object()
+
+
 class SyntheticAttentionEngine:
-    """Attention-only stack with seeded random weights on cuda:0; one request at a time."""
+    """Attention-only stack with seeded random weights on cuda:0 behind a continuous-batching
+    loop: requests from any number of HTTP threads join a shared step (up to `max_seqs`
+    sequences), in which sequences still reading their prompt contribute a prefill chunk and
+    the others one decode row; the scheduler builds the ragged batch and every layer's
+    attention is ONE eid_attn_varlen call over it (eid_attn_decode when every row is a decode
+    row)."""
     name = "synthetic"
 
-    def __init__(self, layers=4, ctx=4096, seed=0, num_blocks=None):
+    def __init__(self, layers=4, ctx=4096, seed=0, num_blocks=None, max_seqs=16, chunk=512,
+                 step_tokens=2048):
         import numpy as np
         import torch
         import eidola_amd as ea
@@ -71,10 +94,11 @@ class SyntheticAttentionEngine:
         ea.load_library()
         dev = "cuda:0"
         self.dev, self.layers, self.ctx = dev, layers, ctx
+        self.max_seqs, self.chunk, self.step_tokens = max_seqs, chunk, step_tokens
         self.H, self.NQKV = 2880, (64 + 2 * 8) * 64
         self.geoms = [ea.AttnGeometry(window=128 if l % 2 == 0 else 0) for l in range(layers)]
         self.max_blocks = (ctx + 15) // 16
-        self.num_blocks = num_blocks or 2 * self.max_blocks
+        self.num_blocks = num_blocks or (max_seqs + 1) * self.max_blocks
         g = torch.Generator(device=dev).manual_seed(seed)
         rnd = lambda *shape, scale: (torch.randn(shape, device=dev, generator=g) * scale).to(torch.bfloat16)
         self.emb = rnd(VOCAB, self.H, scale=1.0)
@@ -86,23 +110,27 @@ class SyntheticAttentionEngine:
         self.vc = [torch.zeros_like(k) for k in self.kc]
         self.cos_sin = torch.from_numpy(ea.yarn_cos_sin(ctx + 1)).to(dev)
         self.sched = ea.Scheduler(self.num_blocks, self.max_blocks)
-        self.lock = threading.Lock()
+        self.cv = threading.Condition()
+        self.waiting, self.active = [], []
         self.next_id = 1
+        self.steps = self.mixed_steps = self.max_step_seqs = 0   # (for tests and curiosity)
+        self.worker = None
 
     def _norm(self, h):
         x = h.float()
         return (x * self.torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6)).to(self.torch.bfloat16)
 
-    def forward(self, seq_id, token_ids):
-        """Appends `token_ids` to sequence `seq_id` (one prefill chunk or one decode token) and
-        returns the logits of the last position, fp32 [VOCAB]."""
-        torch, ea, np = self.torch, self.ea, self.np
-        T = len(token_ids)
-        b = self.sched.build_batch([seq_id], [T])
+    def forward(self, seq_ids, token_lists):
+        """Appends token_lists[i] to sequence seq_ids[i] (a prefill chunk or one decode token
+        each) and returns the logits of every sequence's last position, fp32 [len(seq_ids), VOCAB]."""
+        torch, ea = self.torch, self.ea
+        q_lens = [len(t) for t in token_lists]
+        T = sum(q_lens)
+        b = self.sched.build_batch(seq_ids, q_lens)
         to_dev = lambda a: torch.from_numpy(a).to(self.dev)
         bt, slots, cu, sl, pos = (to_dev(b.block_table), to_dev(b.slot_mapping), to_dev(b.cu_seqlens_q),
                                   to_dev(b.seq_lens), to_dev(b.positions))
-        hidden = self.emb[torch.tensor(token_ids, device=self.dev)].clone()
+        hidden = self.emb[torch.tensor([t for ts in token_lists for t in ts], device=self.dev)].clone()
         for l in range(self.layers):
             g, x = self.geoms[l], self._norm(hidden)
             if T <= 64:   # projection, rotary embedding, split and KV write in one launch
@@ -110,7 +138,7 @@ class SyntheticAttentionEngine:
             else:
                 qkv = ea.o_proj(x, self.wqkv[l])
                 q = ea.rope_kv_write(g, qkv, pos, self.cos_sin, self.kc[l], self.vc[l], slots)
-            if T == 1:
+            if b.max_q_len == 1:
                 out = ea.attn_decode(g, q, self.kc[l], self.vc[l], bt, sl, max_kv_len=b.max_kv_len,
                                      sinks=self.sinks[l], sum_kv_len=b.sum_kv_len, seq_lens_host=b.seq_lens,
                                      block_table_host=b.block_table)
@@ -119,28 +147,82 @@ class SyntheticAttentionEngine:
                                      max_kv_len=b.max_kv_len, sinks=self.sinks[l], sum_kv_len=b.sum_kv_len,
                                      seq_lens_host=b.seq_lens, cu_seqlens_q_host=b.cu_seqlens_q)
             ea.o_proj(out, self.wo[l], residual=hidden, out=hidden)
-        return (self._norm(hidden[-1:]).float() @ self.emb.float().t())[0]
+        last = torch.from_numpy(b.cu_seqlens_q[1:].astype("int64") - 1).to(self.dev)
+        return self._norm(hidden[last]).float() @ self.emb.float().t()
 
-    def generate(self, prompt_ids, max_new_tokens, chunk=512):
-        """Greedy decoding: prefill in chunks of `chunk` tokens, then one token per step.
-        Yields byte tokens, EOS on a genuine stop (see FakeEngine.generate)."""
+    # ---- the batching loop -----------------------------------------------------------------
+    def _step(self):
+        """One shared step over the active requests: prefill chunks within a token budget for
+        those still reading their prompt, one decode row for the others."""
         torch = self.torch
-        prompt_ids = list(prompt_ids)[-(self.ctx - max(1, max_new_tokens)):] or [EOS]
-        with self.lock:
-            seq_id, self.next_id = self.next_id, self.next_id + 1
-            self.sched.add_seq(seq_id)
+        ids, toks, reqs, room = [], [], [], self.step_tokens
+        for r in self.active:
+            if r.fed < len(r.prompt):
+                n = min(self.chunk, len(r.prompt) - r.fed, room)
+                if n <= 0:
+                    continue              # this step's token budget is spent: next step
+                piece = r.prompt[r.fed:r.fed + n]
+            else:
+                piece, n = [r.last], 1
+            room -= n
+            ids.append(r.seq_id)
+            toks.append(piece)
+            reqs.append(r)
+        logits = self.forward(ids, toks)
+        picks = torch.argmax(logits[:, :EOS + 1], dim=-1).tolist()
+        self.steps += 1
+        self.mixed_steps += len({len(t) > 1 for t in toks}) == 2
+        self.max_step_seqs = max(self.max_step_seqs, len(ids))
+        for r, piece, tok in zip(reqs, toks, picks):
+            if r.fed < len(r.prompt):
+                r.fed += len(piece)
+                if r.fed < len(r.prompt):
+                    continue              # more prompt to read: nothing sampled yet
+            r.last = tok
+            r.produced += 1
+            r.out.put(tok)                # (EOS included: a genuine stop)
+            if tok == EOS or r.produced == r.budget or self.sched.seq_len(r.seq_id) + 1 > self.ctx:
+                self._retire(r)
+
+    def _retire(self, r, error=None):
+        self.active.remove(r)
+        self.sched.free_seq(r.seq_id)
+        r.out.put(error if error is not None else _DONE)
+
+    def _run(self):
+        while True:
+            with self.cv:
+                while not self.waiting and not self.active:
+                    self.cv.wait()
+                while self.waiting and len(self.active) < self.max_seqs:
+                    r = self.waiting.pop(0)
+                    self.sched.add_seq(r.seq_id)
+                    self.active.append(r)
             try:
-                logits = None
-                for i in range(0, len(prompt_ids), chunk):
-                    logits = self.forward(seq_id, prompt_ids[i:i + chunk])
-                for i in range(max_new_tokens):
-                    tok = int(torch.argmax(logits[:EOS + 1]).item())
-                    yield tok                      # (EOS included: a genuine stop)
-                    if tok == EOS or i + 1 == max_new_tokens or self.sched.seq_len(seq_id) + 1 > self.ctx:
-                        return
-                    logits = self.forward(seq_id, [tok])
-            finally:
-                self.sched.free_seq(seq_id)
+                self._step()
+            except Exception as e:        # a failed step fails the requests in it, not the process
+                for r in list(self.active):
+                    self._retire(r, e)
+
+    def generate(self, prompt_ids, max_new_tokens):
+        """Greedy decoding through the shared batching loop.  Yields byte tokens, EOS on a
+        genuine stop (see FakeEngine.generate)."""
+        prompt_ids = list(prompt_ids)[-(self.ctx - max(1, max_new_tokens)):] or [EOS]
+        with self.cv:
+            if self.worker is None:
+                self.worker = threading.Thread(target=self._run, name="eidola-engine-steps", daemon=True)
+                self.worker.start()
+            r = _Request(self.next_id, prompt_ids, max_new_tokens)
+            self.next_id += 1
+            self.waiting.append(r)
+            self.cv.notify()
+        while True:
+            tok = r.out.get()
+            if tok is _DONE:
+                return
+            if isinstance(tok, Exception):
+                raise tok
+            yield tok
 
 
 class Handler(BaseHTTPRequestHandler):
@@ -260,6 +342,8 @@ def parse_args(argv=None):
     ap.add_argument("--engine", choices=["synthetic", "fake"], default="synthetic")
     ap.add_argument("--layers", type=int, default=4, help="attention blocks of the synthetic model")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("-np", "--parallel", type=int, default=16,
+                    help="sequences that may share a step (llama-server's name for its slots)")
     return ap.parse_args(argv)
 
 
@@ -272,7 +356,8 @@ def make_server(host, port, engine, alias):
 
 def main(argv=None):
     a = parse_args(argv)
-    engine = FakeEngine() if a.engine == "fake" else SyntheticAttentionEngine(a.layers, a.ctx_size, a.seed)
+    engine = FakeEngine() if a.engine == "fake" else SyntheticAttentionEngine(a.layers, a.ctx_size, a.seed,
+                                                                             max_seqs=max(1, a.parallel))
     srv = make_server(a.host, a.port, engine, a.alias or a.model)
     try:
         srv.serve_forever()
