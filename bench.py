@@ -854,6 +854,38 @@ def gather_bench(torch, ea, synth, np):
     return res
 
 
+def shim_bench(torch):
+    """The engine shim's synthetic stack (8 attention blocks) under concurrent requests: the same
+    16 generations (prompts of 100...1,600 bytes, 48 new tokens each) one at a time and all at
+    once, i.e. what sharing steps between requests buys."""
+    import threading
+    from eidola_amd import engine_shim as shim
+    eng = shim.SyntheticAttentionEngine(layers=8, ctx=4096, seed=1, max_seqs=16)
+    prompts = [shim.render_prompt([{"role": "user", "content": "x" * (100 * (i + 1))}]) for i in range(16)]
+    list(eng.generate(prompts[0], 4))       # warm-up
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_seq = sum(len(list(eng.generate(p, 48))) for p in prompts)
+    t_seq = time.perf_counter() - t0
+    counts = [0] * len(prompts)
+
+    def run(i):
+        counts[i] = len(list(eng.generate(prompts[i], 48)))
+    steps0 = eng.steps
+    t0 = time.perf_counter()
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(len(prompts))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    t_par = time.perf_counter() - t0
+    log(f"[bench] engine shim, 16 requests x 48 new tokens, 8 attention blocks: one at a time {t_seq*1e3:.0f} ms "
+        f"({n_seq / t_seq:.0f} tokens/s), all at once {t_par*1e3:.0f} ms ({sum(counts) / t_par:.0f} tokens/s) in "
+        f"{eng.steps - steps0} shared steps, up to {eng.max_step_seqs} sequences per step")
+    return [{"config": "engine_shim_16_requests", "sequential_s": t_seq, "concurrent_s": t_par,
+             "tokens": sum(counts), "steps": eng.steps - steps0}]
+
+
 def timeline_bench(torch, ea, synth, np):
     """Per-workgroup timeline of the prefill kernel on config 3's prefill rows (host-listed
     tiles) from the library's measurement aid (eid_debug_set_timeline): when workgroups start
@@ -1029,7 +1061,7 @@ def main():
                     help="experiment: no host-side lengths for the library (desc.sum_kv_len = 0, no "
                          "seq_lens_host): the kernels size and plan the launch themselves")
     ap.add_argument("--only", default="",
-                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack,overlap,gather,timeline "
+                    help="with --all: comma-separated subset of 2w,3,4,5,sched,rope,oproj,prefill,small,stack,overlap,gather,timeline,shim "
                          "(default: everything), e.g. to profile one configuration")
     ap.add_argument("--unfused", action="store_true",
                     help="decode steps as two launches (eid_kv_write, then eid_attn_decode) "
@@ -1165,6 +1197,8 @@ def main():
         if want("timeline"):
             import numpy as np
             extra.extend(timeline_bench(torch, ea, synth, np))
+        if want("shim"):
+            extra.extend(shim_bench(torch))
         if want("gather"):
             import numpy as np
             extra.extend(gather_bench(torch, ea, synth, np))
