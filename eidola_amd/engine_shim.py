@@ -67,6 +67,7 @@ class _Request:
 
     def __init__(self, seq_id, prompt_ids, max_new_tokens):
         self.seq_id, self.prompt, self.budget = seq_id, prompt_ids, max_new_tokens
+        self.blocks = (len(prompt_ids) + max_new_tokens + 15) // 16   # pages it may come to hold
         self.fed = 0              # prompt tokens already in the KV cache
         self.last = None          # the sampled token to feed next
         self.produced = 0
@@ -112,6 +113,7 @@ class SyntheticAttentionEngine:
         self.sched = ea.Scheduler(self.num_blocks, self.max_blocks)
         self.cv = threading.Condition()
         self.waiting, self.active = [], []
+        self.committed = 0        # pages the active requests may come to hold between them
         self.next_id = 1
         self.steps = self.mixed_steps = self.max_step_seqs = 0   # (for tests and curiosity)
         self.worker = None
@@ -186,6 +188,7 @@ class SyntheticAttentionEngine:
 
     def _retire(self, r, error=None):
         self.active.remove(r)
+        self.committed -= r.blocks
         self.sched.free_seq(r.seq_id)
         r.out.put(error if error is not None else _DONE)
 
@@ -194,9 +197,13 @@ class SyntheticAttentionEngine:
             with self.cv:
                 while not self.waiting and not self.active:
                     self.cv.wait()
-                while self.waiting and len(self.active) < self.max_seqs:
+                # admission in arrival order, while a slot is free and the pool could hold the
+                # request to its last token (a request is never evicted once it runs)
+                while (self.waiting and len(self.active) < self.max_seqs
+                       and self.committed + self.waiting[0].blocks <= self.num_blocks):
                     r = self.waiting.pop(0)
                     self.sched.add_seq(r.seq_id)
+                    self.committed += r.blocks
                     self.active.append(r)
             try:
                 self._step()
@@ -275,11 +282,14 @@ class Handler(BaseHTTPRequestHandler):
         if req.get("stream"):
             return self._stream(req, rid, created, model, prompt, gen)
         out, finish = bytearray(), "length"
-        for tok in gen:
-            if tok == EOS:
-                finish = "stop"
-                break
-            out.append(tok)
+        try:
+            for tok in gen:
+                if tok == EOS:
+                    finish = "stop"
+                    break
+                out.append(tok)
+        except Exception as e:     # the engine failed this request: say so, keep serving
+            return self._error(500, f"engine error: {e}", "server_error")
         self._json(200, {
             "id": rid, "object": "chat.completion", "created": created, "model": model,
             "choices": [{"index": 0, "finish_reason": finish,
@@ -305,20 +315,23 @@ class Handler(BaseHTTPRequestHandler):
 
         event(chunk({"role": "assistant", "content": ""}))
         n, finish, pending = 0, "length", bytearray()
-        for tok in gen:
-            if tok == EOS:
-                finish = "stop"
-                break
-            n += 1
-            pending.append(tok)
-            try:   # only whole UTF-8 sequences go out
-                text = pending.decode("utf-8")
-            except UnicodeDecodeError:
-                if len(pending) < 4:
-                    continue
-                text = pending.decode("utf-8", "replace")
-            pending.clear()
-            event(chunk({"content": text}))
+        try:
+            for tok in gen:
+                if tok == EOS:
+                    finish = "stop"
+                    break
+                n += 1
+                pending.append(tok)
+                try:   # only whole UTF-8 sequences go out
+                    text = pending.decode("utf-8")
+                except UnicodeDecodeError:
+                    if len(pending) < 4:
+                        continue
+                    text = pending.decode("utf-8", "replace")
+                pending.clear()
+                event(chunk({"content": text}))
+        except Exception as e:     # the engine failed mid-stream: an error event, then the usual end
+            event({"error": {"message": f"engine error: {e}", "type": "server_error", "code": 500}})
         if pending:
             event(chunk({"content": pending.decode("utf-8", "replace")}))
         event(chunk({}, finish))

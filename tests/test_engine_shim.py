@@ -111,6 +111,36 @@ def test_bad_requests_get_a_400_with_an_error_object(server, body):
     assert json.loads(e.value.read())["error"]["type"] == "invalid_request_error"
 
 
+class _FailingEngine:
+    """Yields two tokens, then fails the way a GPU step would."""
+    name = "failing"
+
+    def generate(self, prompt_ids, max_new_tokens):
+        yield ord("o")
+        yield ord("k")
+        raise RuntimeError("step failed")
+
+
+def test_an_engine_failure_is_a_500_or_an_error_event_and_the_server_lives_on():
+    srv = shim.make_server("127.0.0.1", 0, _FailingEngine(), "local/test-model")
+    threading.Thread(target=srv.serve_forever, daemon=True).start()
+    port = srv.server_address[1]
+    try:
+        msgs = [{"role": "user", "content": "x"}]
+        with pytest.raises(urllib.error.HTTPError) as e:
+            post(port, reference_body("m", msgs, 8))
+        assert e.value.code == 500 and json.loads(e.value.read())["error"]["type"] == "server_error"
+        status, _, payload = post(port, reference_body("m", msgs, 8, stream=True), raw=True)
+        assert status == 200 and b'"content": "o"' in payload and b'"content": "k"' in payload
+        assert b'"server_error"' in payload
+        assert payload.rstrip().endswith(b"data: [DONE]")
+        with urllib.request.urlopen(f"http://127.0.0.1:{port}/health", timeout=5) as r:
+            assert r.status == 200
+    finally:
+        srv.shutdown()
+        srv.server_close()
+
+
 def test_started_and_polled_the_way_the_reference_does():
     """The reference spawns the engine with its flags, stdin/stdout null, and polls /health
     until it answers 2xx (local_models.rs:1612-1626, 2020-2063)."""

@@ -95,6 +95,24 @@ def test_concurrent_requests_are_batched_into_shared_steps(engine):
     assert engine.sched.free_blocks == free0 and not engine.active and not engine.waiting
 
 
+def test_requests_wait_for_pages_instead_of_failing():
+    """A pool too small for all requests at once: admission waits until the running ones have
+    returned their pages; every request completes."""
+    eng = shim.SyntheticAttentionEngine(layers=2, ctx=512, seed=5, num_blocks=40, max_seqs=8)
+    prompts = [list(range(1, 200)) for _ in range(5)]           # 199 + 8 tokens -> 13 pages each
+    outs = [None] * len(prompts)
+
+    def run(i):
+        outs[i] = list(eng.generate(prompts[i], 8))
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(len(prompts))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert all(o is not None and 1 <= len(o) <= 8 for o in outs)
+    assert eng.max_step_seqs <= 3 and eng.committed == 0 and eng.sched.free_blocks == 40
+
+
 def test_generation_is_deterministic_and_frees_its_blocks(engine):
     prompt = shim.render_prompt([{"role": "user", "content": "hello"}])
     free0 = engine.sched.free_blocks
