@@ -72,27 +72,52 @@ struct RowInfo {
 //
 // QLDS (the prefill kernel without lse): the Q operands of row tile nt are read from the wave's
 // LDS copy (q_rd, see chunk_pipe) when the tile's turn comes, instead of being held in `qf`.
+// V^T operands of a chunk from its LDS tile: [dim tile][page pair].  `v_sw` != 0: rows of 128
+// bytes whose 32-byte pairs of segments are permuted by (row / 2) % 4 (tiles written by direct
+// global -> LDS loads, see chunk_pipe); dim tile mt then sits at byte (32 mt) ^ v_sw of its row.
+template <int VROW>
+__device__ __forceinline__ void read_vt(const uint8_t *v_rd, const int v_sw, Frag8 (&vf)[4][2]) {
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr) {
+      const uint8_t *v_mt = v_rd + ((32 * mt) ^ v_sw);
+      const u32x2 a = lds_read_tr16(v_mt + (2 * pr) * (kBlock * VROW));
+      const u32x2 b2 = lds_read_tr16(v_mt + (2 * pr + 1) * (kBlock * VROW));
+      vf[mt][pr].w[0] = a[0];
+      vf[mt][pr].w[1] = a[1];
+      vf[mt][pr].w[2] = b2[0];
+      vf[mt][pr].w[3] = b2[1];
+    }
+}
+
+template <int NT, bool PRE, bool PAIR, bool QLDS>
+__device__ __forceinline__ void chunk_core(const Frag8 (&kf)[4][2], const Frag8 (&vf)[4][2],
+                                           const Frag8 (&qf_regs)[NT][2], const RowInfo &ri,
+                                           const int tc, const bool need_mask, const float c2,
+                                           float (&m)[NT], f32x4 (&lacc)[NT],
+                                           f32x4 (&acc)[NT][4], const uint8_t *q_rd);
+
 template <int NT, int VROW = kVRowBytes, bool PRE = false, bool PAIR = false, bool QLDS = false>
 __device__ __forceinline__ void chunk_step(const Frag8 (&kf)[4][2], const uint8_t *v_rd,
                                            const Frag8 (&qf_regs)[NT][2], const RowInfo &ri,
                                            const int tc, const bool need_mask, const float c2,
                                            float (&m)[NT], f32x4 (&lacc)[NT],
                                            f32x4 (&acc)[NT][4], const uint8_t *q_rd = nullptr) {
+  Frag8 vf[4][2];
+  read_vt<VROW>(v_rd, 0, vf);
+  chunk_core<NT, PRE, PAIR, QLDS>(kf, vf, qf_regs, ri, tc, need_mask, c2, m, lacc, acc, q_rd);
+}
+
+template <int NT, bool PRE, bool PAIR, bool QLDS>
+__device__ __forceinline__ void chunk_core(const Frag8 (&kf)[4][2], const Frag8 (&vf)[4][2],
+                                           const Frag8 (&qf_regs)[NT][2], const RowInfo &ri,
+                                           const int tc, const bool need_mask, const float c2,
+                                           float (&m)[NT], f32x4 (&lacc)[NT],
+                                           f32x4 (&acc)[NT][4], const uint8_t *q_rd) {
   const int g = (threadIdx.x & 63) >> 4;
   Frag8 ones;  // bf16 1.0 in every slot: a row of ones in place of V^T yields row sums of P
   ones.u = u32x4{0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-  Frag8 vf[4][2];  // [dim tile][page pair]
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {
-      const u32x2 a = lds_read_tr16(v_rd + (2 * pr) * (kBlock * VROW) + 32 * mt);
-      const u32x2 b2 = lds_read_tr16(v_rd + (2 * pr + 1) * (kBlock * VROW) + 32 * mt);
-      vf[mt][pr].w[0] = a[0];
-      vf[mt][pr].w[1] = a[1];
-      vf[mt][pr].w[2] = b2[0];
-      vf[mt][pr].w[3] = b2[1];
-    }
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
     Frag8 qf_nt[2];
@@ -557,13 +582,23 @@ struct FirstPages {
   int id[4] = {0, 0, 0, 0};
 };
 
-template <int NT, bool FP8, bool PAIR = false>
+// No partials inside the key range (the default `emit` of attend).
+struct NoEmit {
+  __device__ __forceinline__ void operator()(int) const {}
+};
+
+// `emit_every` > 0 (a multiple of the chunk): after every `emit_every` keys from t_begin, except
+// at the end of the range, emit(k) is called with k = 0, 1, ...: the caller stores the partial
+// of that stretch and resets m / lacc / acc, and the loop goes on with the next stretch, its
+// page ids already under way (a range of several partitions walked without a new start).
+template <int NT, bool FP8, bool PAIR = false, class Emit = NoEmit>
 __device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
                                        const int t_begin, const int t_end, const int seq_len,
                                        const int pos_first, const int lo_last,
                                        const Frag8 (&qf)[NT][2], const RowInfo &ri,
                                        uint8_t *wave_lds, float (&m)[NT], f32x4 (&lacc)[NT],
-                                       f32x4 (&acc)[NT][4], const FirstPages &first = FirstPages{}) {
+                                       f32x4 (&acc)[NT][4], const FirstPages &first = FirstPages{},
+                                       const int emit_every = 0, const Emit emit = Emit{}) {
   const int lane = threadIdx.x & 63;
   const int i16 = lane & 15, g = lane >> 4;
   const int Hkv = p.num_kv_heads;
@@ -607,6 +642,7 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
     for (int b = 0; b < kPages; ++b) blk[b] = bt[min(t_begin / kBlock + b, nblk_total - 1)];
   }
 
+  int emit_left = emit_every, emit_k = 0;
   for (int ti = t_begin; ti < t_end; ti += kIter) {
     const int nbi = min(kPages, (t_end - ti + kBlock - 1) / kBlock);
 
@@ -627,8 +663,10 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
         const uint8_t *vp = p.v_cache + page_off;
 #pragma unroll
         for (int e = 0; e < kElt; ++e) {
-          kraw[b][e] = ldg128(kp + 16 * e);
-          vraw[b][e] = ldg128(vp + 16 * e);
+          // (head pairs: a load instruction takes whole 128-byte lines, and nothing of a line
+          // is asked for again: the streaming hint is worth a tenth of the run time there)
+          kraw[b][e] = PAIR ? __builtin_nontemporal_load((const u32x4 *)(kp + 16 * e)) : ldg128(kp + 16 * e);
+          vraw[b][e] = PAIR ? __builtin_nontemporal_load((const u32x4 *)(vp + 16 * e)) : ldg128(vp + 16 * e);
         }
       }
     }
@@ -723,6 +761,144 @@ __device__ __forceinline__ void attend(const AttnParams &p, const int s, const i
     const bool need_mask = (tc < lo_last) || (tc + kIter > pos_first + 1);
     chunk_step<NT, kVRowBytes, false, PAIR>(kf, lds_rd, qf, ri, tc, need_mask, c2, m, lacc, acc);
     }  // sub
+    if constexpr (!std::is_same<Emit, NoEmit>::value) {
+      emit_left -= kIter;
+      if (emit_left == 0 && ti + kIter < t_end) {  // (wave-uniform)
+        emit(emit_k++);
+        emit_left = emit_every;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// The same over a bf16 cache, with the K/V chunk brought in by direct global -> LDS loads.
+//
+// What the memory system gives a gather of KV pages depends on the shape of a load
+// instruction: when 8 consecutive lanes take the eight 16-byte pieces of one 128-byte line
+// (a head's row of one token) and the load carries the non-temporal hint, a plain gather of
+// the pages runs at 6.6 - 6.9 TB/s; when every line is picked up in halves by two
+// instructions and lanes 16 apart, as the MFMA operand layout would have a register load do,
+// it runs at 5.8 - 6.2 TB/s, and the hint makes that worse.  A lane cannot both sit in an
+// 8-lane line group and hold its own row's operand slice, so the chunk goes through LDS:
+// global_load_lds_dwordx4 moves 8 token rows x 128 bytes per instruction into a wave-private
+// tile of 64 rows x 128 bytes for K and one for V (segments permuted as in chunk_pipe, which
+// keeps the ds_read_b128 K reads and the transposing V reads free of bank conflicts).  The
+// operands of a chunk are read into registers first; then the loads of the NEXT chunk are
+// issued into the same two tiles, and they are in flight for the whole of this chunk's
+// arithmetic: one tile pair per wave is enough, and no staging registers are held.
+// Rows past the end of the sequence repeat its last row (finite data, masked scores).
+//
+// The fused write of the newest token (NT == 1, p.k_new): its row is stored into the cache
+// first and the loads of the chunk that holds it are issued after that store has completed,
+// so the row arrives with the rest of its page.
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void dma_gptr_t;
+typedef __attribute__((address_space(3))) void dma_lptr_t;
+constexpr int kDmaTileBytes = kChunk * 128;          // 64 token rows of one KV head
+constexpr int kWaveDmaBytes = 2 * kDmaTileBytes;     // K tile, V tile
+constexpr int kDmaAux = 2;                           // non-temporal (streaming) loads
+
+template <int NT, class Emit = NoEmit>
+__device__ __forceinline__ void attend_dma(const AttnParams &p, const int s, const int kvh,
+                                           const int t_begin, const int t_end, const int seq_len,
+                                           const int pos_first, const int lo_last,
+                                           const Frag8 (&qf)[NT][2], const RowInfo &ri,
+                                           uint8_t *wave_lds, float (&m)[NT], f32x4 (&lacc)[NT],
+                                           f32x4 (&acc)[NT][4], const FirstPages &first = FirstPages{},
+                                           const int emit_every = 0, const Emit emit = Emit{}) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, g = lane >> 4;
+  const uint32_t row_bytes = (uint32_t)p.num_kv_heads * (kHeadDim * 2);
+  const size_t page_bytes = (size_t)kBlock * row_bytes;
+  const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
+  const int nblk_total = (t_end + kBlock - 1) / kBlock;
+  const float c2 = p.softmax_scale * kLog2e;
+  uint8_t *ktile = wave_lds, *vtile = wave_lds + kDmaTileBytes;
+  // loader: lane (r, sl) = (lane / 8, lane % 8) fills slot sl of row 8 h + r of a page
+  const int dr = lane >> 3, dsl = lane & 7;
+  const uint32_t head_off = (uint32_t)kvh * (kHeadDim * 2);
+  // operand reads (see chunk_pipe<128, SWZ>)
+  const int sw_k = (i16 >> 1) & 7;
+  const uint8_t *k_rd = ktile + (uint32_t)i16 * 128 + (uint32_t)((2 * g) ^ sw_k) * 16;
+  const uint8_t *k_rd_hi = ktile + (((uint32_t)i16 * 128 + (uint32_t)((2 * g) ^ sw_k) * 16) ^ 16);
+  const int v_row = 4 * g + (i16 >> 2);
+  const uint8_t *v_rd = vtile + (uint32_t)v_row * 128 + 8 * (i16 & 3);
+  const int v_sw = 32 * ((v_row >> 1) & 3);
+
+  auto pages_of = [&](const int ti, int (&blk)[4]) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) blk[b] = bt[min(ti / kBlock + b, nblk_total - 1)];
+  };
+  auto issue = [&](const int ti, const int (&blk)[4]) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const size_t page_off = (size_t)clamp_page(blk[b], p.last_block) * page_bytes + head_off;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int tok = min(ti + b * kBlock + 8 * h + dr, seq_len - 1);
+        const size_t off = page_off + (uint32_t)(tok & (kBlock - 1)) * row_bytes;
+        const int kseg = dsl ^ (4 * h + (dr >> 1));
+        const int vseg = dsl ^ ((dr >> 1) << 1);
+        __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.k_cache + off + kseg * 16),
+                                         (dma_lptr_t *)(ktile + (2 * b + h) * 1024), 16, 0, kDmaAux);
+        __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.v_cache + off + vseg * 16),
+                                         (dma_lptr_t *)(vtile + (2 * b + h) * 1024), 16, 0, kDmaAux);
+      }
+    }
+  };
+
+  // newest token: into the cache before anything of its page is requested
+  if (NT == 1 && p.k_new && seq_len - 1 >= t_begin && seq_len - 1 < t_end) {  // wave-uniform
+    const int pos_new = seq_len - 1;
+    const int page = clamp_page(bt[pos_new / kBlock], p.last_block);
+    if (lane < 16) {
+      const int kv = lane >> 3, c = lane & 7;
+      const uint16_t *from = (kv ? p.v_new : p.k_new) + ((size_t)s * p.num_kv_heads + kvh) * kHeadDim + c * 8;
+      uint8_t *to = const_cast<uint8_t *>(kv ? p.v_cache : p.k_cache) + (size_t)page * page_bytes +
+                    (uint32_t)(pos_new & (kBlock - 1)) * row_bytes + head_off + c * 16;
+      *(u32x4 *)to = *(const u32x4 *)from;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the row is in place before its page is read
+  }
+
+  int blk[4], blk_next[4];
+  if (first.have) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) blk[b] = first.id[b];
+  } else {
+    pages_of(t_begin, blk);
+  }
+  issue(t_begin, blk);
+  if (t_begin + kChunk < t_end) pages_of(t_begin + kChunk, blk_next);
+
+  int emit_left = emit_every, emit_k = 0;
+  for (int ti = t_begin; ti < t_end; ti += kChunk) {
+    // this chunk's tiles have landed
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    Frag8 kf[4][2], vf[4][2];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      kf[b][0].u = *(const u32x4 *)(k_rd + b * (kBlock * 128));
+      kf[b][1].u = *(const u32x4 *)(k_rd_hi + b * (kBlock * 128));
+    }
+    read_vt<128>(v_rd, v_sw, vf);
+    // ... and are in registers: the tiles are free for the next chunk, which streams in while
+    // this one is computed
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (ti + kChunk < t_end) {
+      issue(ti + kChunk, blk_next);
+      if (ti + 2 * kChunk < t_end) pages_of(ti + 2 * kChunk, blk_next);
+    }
+    const bool need_mask = (ti < lo_last) || (ti + kChunk > pos_first + 1);
+    chunk_core<NT, false, false, false>(kf, vf, qf, ri, ti, need_mask, c2, m, lacc, acc, nullptr);
+    if constexpr (!std::is_same<Emit, NoEmit>::value) {
+      emit_left -= kChunk;
+      if (emit_left == 0 && ti + kChunk < t_end) {  // (wave-uniform)
+        emit(emit_k++);
+        emit_left = emit_every;
+      }
+    }
   }
 }
 
@@ -1068,7 +1244,7 @@ __global__ __launch_bounds__(64) void plan_kernel(const AttnParams p, int32_t *p
 
 // One work item: wave `wave` of the workgroup attends the rows of KV head `kvh` over
 // partition it.part (P tokens) of sequence it.seq and writes the output or the partial.
-template <int NT, bool FP8, bool PAIR = false>
+template <int NT, bool FP8, bool PAIR = false, bool DMA = false>
 __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem &it, const int P,
                                              const int kvh, const int wave, uint8_t *lds,
                                              const FirstPages &first = FirstPages{},
@@ -1094,8 +1270,11 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
-  attend<NT, FP8, PAIR>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes,
-                        m, lacc, acc, first);
+  if constexpr (DMA)
+    attend_dma<NT>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveDmaBytes, m, lacc, acc, first);
+  else
+    attend<NT, FP8, PAIR>(p, s, kvh, t0, t1, L, pos0, lo_last, qf, ri, lds + wave * kWaveLdsBytes,
+                          m, lacc, acc, first);
   finish<NT, FP8, PAIR>(p, s, kvh, row0, qlen, tq0, nparts == 1, part, m, lacc, acc);
 }
 
@@ -1111,11 +1290,15 @@ __device__ __forceinline__ void splitkv_item(const AttnParams &p, const WorkItem
 // the grid's y dimension grows by RS.  Both waves load the head's K/V (the second from cache).
 //
 // PAIR (fp8 decode rows): every wave owns two neighbouring KV heads, see chunk_step.
-template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
-__global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(const AttnParams p) {
+//
+// DMA (bf16 cache): the chunks come in by direct global -> LDS loads (attend_dma); 16 KiB of LDS
+// per wave, i.e. one 8-wave workgroup per CU.
+template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false, bool DMA = false>
+__global__ __launch_bounds__(WAVES * 64, ((NT == 1 && !DMA) ? 4 : 2)) void splitkv_kernel(const AttnParams p) {
   static_assert(RS == 1 || (NT == 4 && WAVES % RS == 0), "row groups are 8 tokens = four tiles");
   static_assert(!PAIR || RS == 1, "head pairs have one row group");
-  __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
+  static_assert(!DMA || (!FP8 && RS == 1), "direct loads: bf16 cache, one row group");
+  __shared__ __align__(1024) uint8_t lds[WAVES * (DMA ? kWaveDmaBytes : kWaveLdsBytes)];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = (blockIdx.y * (WAVES / RS) + wave / RS) * (PAIR ? 2 : 1);
   const int tq0 = (wave % RS) * (NT * 16 / kGroup);
@@ -1134,7 +1317,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
     it.row0 = v.row0;
     it.qlen = v.qlen;
     it.seq_len = v.seq_len;
-    splitkv_item<NT, FP8, PAIR>(p, it, 1 << 30, kvh, wave, lds, FirstPages{}, tq0);
+    splitkv_item<NT, FP8, PAIR, DMA>(p, it, 1 << 30, kvh, wave, lds, FirstPages{}, tq0);
     return;
   }
   if (planned_out(p, blockIdx.x)) return;
@@ -1168,7 +1351,7 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_kernel(
   it.seq_len = __builtin_amdgcn_readfirstlane(item_lds[6]);
   // the merge launch that follows reads the partition from here instead of re-deriving it
   if (!p.plan && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = P;
-  splitkv_item<NT, FP8, PAIR>(p, it, P, kvh, wave, lds, FirstPages{}, tq0);
+  splitkv_item<NT, FP8, PAIR, DMA>(p, it, P, kvh, wave, lds, FirstPages{}, tq0);
 }
 
 // The same for a decode launch whose items the host has listed (q_len 1, row = sequence):
@@ -1186,10 +1369,10 @@ __device__ __forceinline__ WorkItem table_item(const AttnParams &p, const ItemTa
   return it;
 }
 
-template <int NT, bool FP8, int WAVES, bool PAIR = false>
-__global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_table_kernel(
+template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
+__global__ __launch_bounds__(WAVES * 64, ((NT == 1 && !DMA) ? 4 : 2)) void splitkv_table_kernel(
     const AttnParams p, const ItemTable tab) {
-  __shared__ __align__(16) uint8_t lds[WAVES * kWaveLdsBytes];
+  __shared__ __align__(1024) uint8_t lds[WAVES * (DMA ? kWaveDmaBytes : kWaveLdsBytes)];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = (blockIdx.y * WAVES + wave) * (PAIR ? 2 : 1);
   if ((int)blockIdx.x >= tab.n) return;
@@ -1200,7 +1383,183 @@ __global__ __launch_bounds__(WAVES * 64, (NT == 1 ? 4 : 2)) void splitkv_table_k
   first.have = tab.has_blk;  // compiler copy the whole list into private memory)
 #pragma unroll
   for (int b = 0; b < 4; ++b) first.id[b] = tab.blk[blockIdx.x][b];
-  splitkv_item<NT, FP8, PAIR>(p, it, P, kvh, wave, lds, first);
+  splitkv_item<NT, FP8, PAIR, DMA>(p, it, P, kvh, wave, lds, first);
+}
+
+// ---------------------------------------------------------------------------------------
+// Even split.  One workgroup per work item leaves much of the device idle on long launches:
+// every item pays a dispatch, the item lookup, the loads of Q and of its first page ids and, at
+// its end, the hardware's wait for the partial stores before the slot is handed on (about
+// 10 us next to 42 us of streaming for a 512-key item of five query rows, with nothing of the
+// CU in flight meanwhile where one workgroup fits a CU), and a batch of ragged sequences cut
+// into one device fill of items leaves a third of the slots idle behind the longest items.
+// Here the launch's units - 64-key chunks (run-time partition) or partitions of the caller's
+// size - are laid out sequence after sequence and cut into gridDim.x equal, contiguous ranges
+// of `q` units: workgroup b walks units [b q, (b + 1) q), from the middle of one sequence
+// through whole sequences into the start of another.  Q is loaded once per sequence visited,
+// the page-id prefetch runs through, and partials are stored where a range leaves a
+// (sequence, partition) cell: at the end of the range, at the end of a sequence, and every
+// `partition` keys when the caller fixed the partition.  Equal unit counts are equal work.
+//
+// Run-time partition: the pieces of a sequence have no common size.  Piece index = workgroup
+// id - id of the workgroup holding the sequence's first unit; the workgroup that holds the
+// first unit records the sequence's number of pieces in p.seq_parts for the merge, and the
+// plan slot receives kEvenFlag | q.  With q >= kEvenMinChunks a sequence of n chunks has at
+// most ceil(n / kEvenMinChunks) + 1 pieces, which is what the workspace is sized for.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ SeqView view_seq_uniform(const AttnParams &p, const int s) {
+  // (s is wave-uniform: the loads go through the scalar unit)
+  SeqView v{0, 0, 0, 0};
+  if (s < p.num_seqs) {
+    v.seq_len = min(as_constant(p.seq_lens)[s], p.max_blocks_per_seq * kBlock);
+    v.row0 = s;
+    v.qlen = 1;
+    if (p.cu_seqlens_q) {
+      const const_i32_ptr cu = as_constant(p.cu_seqlens_q);
+      v.row0 = cu[s];
+      v.qlen = cu[s + 1] - v.row0;
+    }
+    if (v.qlen >= p.qlen_lo && v.qlen <= p.qlen_hi && v.qlen <= p.ws_rows && v.seq_len >= v.qlen)
+      v.span = v.seq_len - kv_begin(v.seq_len, v.qlen, p.window);
+  }
+  return v;
+}
+
+// Units of a sequence in an even split: chunks, or partitions of the caller's size.
+__device__ __forceinline__ int even_units(const AttnParams &p, const int span) {
+  return p.dynamic_partition ? (span + kChunk - 1) / kChunk : num_partitions(p, span, p.partition);
+}
+
+// Quota and start of workgroup `b` of `G`: q = units per workgroup, (seq, unit) = where its
+// range begins.  False when the range is empty.  Executed by one wave.
+__device__ __forceinline__ bool even_find_start(const AttnParams &p, const int b, const int G,
+                                                int &q, int &seq, int &unit) {
+  const int lane = threadIdx.x & 63;
+  long long C = 0;
+  for (int s0 = 0; s0 < p.num_seqs; s0 += 64) C += even_units(p, view_seq(p, s0 + lane).span);
+  C = wave_total64(C);
+  q = (int)max(uniform_div(C + G - 1, G), (long long)(p.dynamic_partition ? kEvenMinChunks : 1));
+  const long long start = (long long)b * q;
+  if (start >= C) return false;
+  long long base = 0;
+  for (int s0 = 0; s0 < p.num_seqs; s0 += 64) {
+    const int n = even_units(p, view_seq(p, s0 + lane).span);
+    const int incl = wave_inclusive_scan(n, lane);
+    const int total = __builtin_amdgcn_readlane(incl, 63);
+    if (start < base + total) {
+      const int rel = (int)(start - base);
+      const int idx = __builtin_ctzll(__ballot(incl > rel));
+      seq = s0 + idx;
+      unit = rel - (__builtin_amdgcn_readlane(incl, idx) - __builtin_amdgcn_readlane(n, idx));
+      return true;
+    }
+    base += total;
+  }
+  return false;
+}
+
+// (two waves per SIMD, i.e. all 256 registers: eight waves per CU; the head-pair kernel moves
+// half the bytes per wave and load, and keeps sixteen)
+template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
+__global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kernel(const AttnParams p,
+                                                                                const EvenTable tab) {
+  __shared__ __align__(1024) uint8_t lds[WAVES * (DMA ? kWaveDmaBytes : kWaveLdsBytes)];
+  __shared__ int start_lds[4];
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int kvh = (blockIdx.y * WAVES + wave) * (PAIR ? 2 : 1);
+  const int b = blockIdx.x;
+  const bool dyn = p.dynamic_partition != 0;
+  int q, s, u;
+  if (tab.n > 0) {
+    if (b >= tab.n) return;
+    q = tab.q;
+    const uint32_t e = tab.start[b];
+    s = (int)(e & 0xffffu);
+    u = (int)(e >> 16);
+  } else {
+    if (wave == 0) {
+      int q0 = 0, s0 = 0, u0 = 0;
+      const bool found = even_find_start(p, b, gridDim.x, q0, s0, u0);
+      if ((threadIdx.x & 63) == 0) {
+        start_lds[0] = found ? q0 : 0;
+        start_lds[1] = s0;
+        start_lds[2] = u0;
+      }
+    }
+    __syncthreads();
+    q = __builtin_amdgcn_readfirstlane(start_lds[0]);
+    if (q == 0) return;
+    s = __builtin_amdgcn_readfirstlane(start_lds[1]);
+    u = __builtin_amdgcn_readfirstlane(start_lds[2]);
+  }
+  // the merge that follows reads the mode (and, with the caller's partition, its size) from here
+  if (b == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = dyn ? (kEvenFlag | q) : p.partition;
+  const int U = dyn ? kChunk : p.partition;  // keys per unit
+  uint8_t *wave_lds = lds + wave * (DMA ? kWaveDmaBytes : kWaveLdsBytes);
+  int rem = q;
+  bool first_seq = true;
+  SeqView v = view_seq_uniform(p, s);
+  while (rem > 0 && s < p.num_seqs) {
+    const int n_s = even_units(p, v.span);
+    const int n_here = min(rem, n_s - u);
+    const int s_now = s, u_now = u;
+    const SeqView v_now = v;
+    // next sequence of this class (its lengths are requested before this one is walked)
+    rem -= n_here;
+    u = 0;
+    do {
+      ++s;
+      v = view_seq_uniform(p, s);
+    } while (s < p.num_seqs && v.span <= 0);
+    if (n_here <= 0) continue;  // (only a malformed start: the range begins past a sequence's end)
+    const int L = v_now.seq_len, qlen = v_now.qlen, row0 = v_now.row0;
+    const int kb = kv_begin(L, qlen, p.window);
+    const int t0 = kb + u_now * U;
+    const int t1 = min(kb + (u_now + n_here) * U, L);
+    const int pos0 = L - qlen;
+    const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
+    // the piece (run-time partition) or the first partition (caller's) and the sequence's count
+    int part, nparts;
+    if (dyn) {
+      // units before this sequence: (b q + units of the range used up so far) - u_now
+      part = first_seq ? (u_now + q - 1) / q : 0;
+      // first workgroup of the sequence holds its unit 0: the sequence starts `off` units into it
+      const int off = first_seq ? (q - (u_now % q)) % q : q - (rem + n_here);
+      nparts = (off + n_s - 1) / q + 1;
+      if (part == 0 && wave == 0 && blockIdx.y == 0 && (threadIdx.x & 63) == 0) p.seq_parts[s_now] = nparts;
+    } else {
+      part = u_now;
+      nparts = n_s;
+    }
+    first_seq = false;
+    Frag8 qf[NT][2];
+    RowInfo ri;
+    load_q<NT, false, PAIR>(p, row0, qlen, 0, kvh, pos0, qf, ri);
+    float m[NT];
+    f32x4 lacc[NT], acc[NT][4];
+    auto reset = [&]() {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        m[nt] = kNegBig;
+        lacc[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+    };
+    reset();
+    const bool direct = nparts == 1;
+    auto emit = [&](const int k) {
+      finish<NT, FP8, PAIR>(p, s_now, kvh, row0, qlen, 0, false, part + k, m, lacc, acc);
+      reset();
+    };
+    if constexpr (DMA)
+      attend_dma<NT>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, FirstPages{},
+                     dyn ? 0 : U, emit);
+    else
+      attend<NT, FP8, PAIR>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc,
+                            FirstPages{}, dyn ? 0 : U, emit);
+    finish<NT, FP8, PAIR>(p, s_now, kvh, row0, qlen, 0, direct, dyn ? part : part + n_here - 1, m, lacc, acc);
+  }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1793,8 +2152,13 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   if (L < qlen) return;
   // run-time partition: recorded by the split-KV launch of this class; else the caller's
   const int P = p.plan_slot ? p.plan_slot[0] : p.partition;
-  if (P < 64 || (P & 63) != 0) return;  // (a slot no split-KV launch has written: nothing to merge)
-  const int nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
+  int nparts;
+  if (P & kEvenFlag) {  // an even split with pieces of no common size left the count per sequence
+    nparts = min(p.seq_parts[s], p.nparts_max);
+  } else {
+    if (P < 64 || (P & 63) != 0) return;  // (a slot no split-KV launch has written: nothing to merge)
+    nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
+  }
   if (nparts <= 1) return;
 
   const int g = lane >> 4, q = lane & 15;
@@ -2024,28 +2388,30 @@ int device_cus() {
   return cus;
 }
 
-template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
+template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false, bool DMA = false>
 static int fill_of() {
-  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES, RS, PAIR>, WAVES * 64);
+  static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES, RS, PAIR, DMA>, WAVES * 64);
   return fill;
 }
 
-template <int NT, bool FP8>
+template <int NT, bool FP8, bool DMA = false>
 static int fill_t(int waves) {
   switch (waves) {
-    case 8: return fill_of<NT, FP8, 8>();
-    case 4: return fill_of<NT, FP8, 4>();
-    case 2: return fill_of<NT, FP8, 2>();
-    default: return fill_of<NT, FP8, 1>();
+    case 8: return fill_of<NT, FP8, 8, 1, false, DMA>();
+    case 4: return fill_of<NT, FP8, 4, 1, false, DMA>();
+    case 2: return fill_of<NT, FP8, 2, 1, false, DMA>();
+    default: return fill_of<NT, FP8, 1, 1, false, DMA>();
   }
 }
 
 static int waves_for(int Hkv) { return Hkv >= 8 ? 8 : Hkv; }
 
 // Workgroups of the split-KV instantiation (ntiles, fp8, Hkv) the device holds at once.
-int splitkv_fill(int ntiles, bool fp8, int Hkv, bool pair) {
+int splitkv_fill(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
   if (pair && fp8 && ntiles == 1) return fill_of<1, true, 4, 1, true>();  // two KV heads per wave
   const int waves = waves_for(Hkv);
+  if (dma && !fp8 && ntiles < 8)
+    return ntiles == 1 ? fill_t<1, false, true>(waves) : ntiles == 3 ? fill_t<3, false, true>(waves) : fill_t<4, false, true>(waves);
   if (ntiles == 8) return fp8 ? fill_of<4, true, 8, 2>() : fill_of<4, false, 8, 2>();  // two row groups
   if (ntiles == 16) return fp8 ? fill_of<4, true, 8, 4>() : fill_of<4, false, 8, 4>();  // four
   if (fp8) return ntiles == 1 ? fill_t<1, true>(waves) : ntiles == 3 ? fill_t<3, true>(waves) : fill_t<4, true>(waves);
@@ -2091,6 +2457,12 @@ static long long item_bound(const AttnParams &p) {
 template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
   dim3 grid((unsigned)item_bound(p), p.num_kv_heads / (WAVES / RS) / (PAIR ? 2 : 1));
+  if constexpr (!FP8 && RS == 1) {
+    if (p.dma) {  // (never beside a prefill launch: its LDS leaves no room for one)
+      splitkv_kernel<NT, FP8, WAVES, RS, PAIR, true><<<grid, WAVES * 64, 0, st>>>(p);
+      return hipGetLastError();
+    }
+  }
   // With a prefill launch beside it (mixed batch, p.share_cus): one 8-wave workgroup per CU.
   // A second resident workgroup adds little to a kernel that streams from HBM (it only
   // covers the prologues of many short items), while half of the CU's registers left free
@@ -2199,6 +2571,96 @@ void set_kernel_events(void *start, void *stop) {
   g_kernel_stop = static_cast<hipEvent_t>(stop);
 }
 
+// Workgroups of an even split: resident all at once, one 8-wave workgroup per CU (eight waves
+// keep a CU's share of the memory system busy; of two resident workgroups the younger mostly
+// waits), smaller workgroups so that a CU holds eight waves.  EID_EVEN_WGS_PER_CU overrides
+// the number per CU for measurements.
+template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
+static int even_fill_of() {
+  static const int fill = device_fill(splitkv_even_kernel<NT, FP8, WAVES, PAIR, DMA>, WAVES * 64);
+  return fill;
+}
+template <int NT, bool FP8, bool DMA = false>
+static int even_fill_t(int waves) {
+  switch (waves) {
+    case 8: return even_fill_of<NT, FP8, 8, false, DMA>();
+    case 4: return even_fill_of<NT, FP8, 4, false, DMA>();
+    case 2: return even_fill_of<NT, FP8, 2, false, DMA>();
+    default: return even_fill_of<NT, FP8, 1, false, DMA>();
+  }
+}
+int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
+  static const int per_cu_env = [] {
+    const char *e = getenv("EID_EVEN_WGS_PER_CU");
+    return e ? atoi(e) : 0;
+  }();
+  int fill, waves;
+  if (pair && fp8 && ntiles == 1) {
+    fill = even_fill_of<1, true, 4, true>();
+    waves = 4;
+  } else {
+    waves = waves_for(Hkv);
+    if (fp8) fill = ntiles == 1 ? even_fill_t<1, true>(waves) : ntiles == 3 ? even_fill_t<3, true>(waves) : even_fill_t<4, true>(waves);
+    else if (dma) fill = ntiles == 1 ? even_fill_t<1, false, true>(waves) : ntiles == 3 ? even_fill_t<3, false, true>(waves) : even_fill_t<4, false, true>(waves);
+    else fill = ntiles == 1 ? even_fill_t<1, false>(waves) : ntiles == 3 ? even_fill_t<3, false>(waves) : even_fill_t<4, false>(waves);
+  }
+  const int per_cu = per_cu_env > 0 ? per_cu_env : (pair && fp8 && ntiles == 1) ? 4 : max(1, 8 / waves);
+  return max(1, min(fill, per_cu * device_cus()) / (Hkv > 8 ? Hkv / 8 : 1));
+}
+
+template <int NT, bool FP8, int WAVES, bool PAIR = false>
+static hipError_t launch_even_w(const AttnParams &p, const EvenTable &tab, hipStream_t st) {
+  dim3 grid((unsigned)(tab.n > 0 ? tab.n : p.even_wgs), p.num_kv_heads / WAVES / (PAIR ? 2 : 1));
+  if constexpr (!FP8) {
+    if (p.dma) {
+      splitkv_even_kernel<NT, FP8, WAVES, PAIR, true><<<grid, WAVES * 64, 0, st>>>(p, tab);
+      return hipGetLastError();
+    }
+  }
+  // (p.share_cus: one 8-wave workgroup per CU by a request for unused dynamic LDS, see launch_splitkv_w)
+  const int kPad = (WAVES == 8 && p.share_cus) ? 16384 : 0;
+  if (kPad > 0) {
+    static std::atomic<bool> allowed[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {
+      e = hipFuncSetAttribute((const void *)splitkv_even_kernel<NT, FP8, WAVES, PAIR>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kPad);
+      if (e != hipSuccess) return e;
+      if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
+    }
+  }
+  splitkv_even_kernel<NT, FP8, WAVES, PAIR><<<grid, WAVES * 64, kPad, st>>>(p, tab);
+  return hipGetLastError();
+}
+template <int NT, bool FP8>
+static hipError_t launch_even_t(const AttnParams &p, const EvenTable &tab, hipStream_t st) {
+  switch (waves_for(p.num_kv_heads)) {
+    case 8: return launch_even_w<NT, FP8, 8>(p, tab, st);
+    case 4: return launch_even_w<NT, FP8, 4>(p, tab, st);
+    case 2: return launch_even_w<NT, FP8, 2>(p, tab, st);
+    default: return launch_even_w<NT, FP8, 1>(p, tab, st);
+  }
+}
+// Even split (see splitkv_even_kernel); `tab` may be null (starts found on the device).
+hipError_t launch_even(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
+                       const EvenTable *tab) {
+  static const EvenTable none{};
+  const EvenTable &t = tab ? *tab : none;
+  p.plan = nullptr;
+  p.plan_slot = plan_slot;
+  if (fp8) {
+    if (ntiles == 1 && p.fp8_pair) return launch_even_w<1, true, 4, true>(p, t, st);
+    if (ntiles == 1) return launch_even_t<1, true>(p, t, st);
+    if (ntiles == 3) return launch_even_t<3, true>(p, t, st);
+    return launch_even_t<4, true>(p, t, st);
+  }
+  if (ntiles == 1) return launch_even_t<1, false>(p, t, st);
+  if (ntiles == 3) return launch_even_t<3, false>(p, t, st);
+  return launch_even_t<4, false>(p, t, st);
+}
+
 // p.target_items must hold splitkv_fill(ntiles, fp8, Hkv).  On return p.plan is set when a
 // plan kernel was run for this launch; the merge launch that follows is given the same
 // params so that it uses the same partition.
@@ -2213,11 +2675,13 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
     dim3 grid((unsigned)tab->n, p.num_kv_heads / 8);
     if (g_kernel_start && g_kernel_stop && !fp8) {
       void *kargs[] = {const_cast<AttnParams *>(&p), const_cast<ItemTable *>(tab)};
-      return hipExtLaunchKernel(reinterpret_cast<const void *>(splitkv_table_kernel<1, false, 8>), grid, dim3(512),
-                                kargs, 0, st, g_kernel_start, g_kernel_stop, 0);
+      return hipExtLaunchKernel(p.dma ? reinterpret_cast<const void *>(splitkv_table_kernel<1, false, 8, false, true>)
+                                      : reinterpret_cast<const void *>(splitkv_table_kernel<1, false, 8>),
+                                grid, dim3(512), kargs, 0, st, g_kernel_start, g_kernel_stop, 0);
     }
     if (fp8 && p.fp8_pair) splitkv_table_kernel<1, true, 4, true><<<grid, 256, 0, st>>>(p, *tab);
     else if (fp8) splitkv_table_kernel<1, true, 8><<<grid, 512, 0, st>>>(p, *tab);
+    else if (p.dma) splitkv_table_kernel<1, false, 8, false, true><<<grid, 512, 0, st>>>(p, *tab);
     else splitkv_table_kernel<1, false, 8><<<grid, 512, 0, st>>>(p, *tab);
     return hipGetLastError();
   }

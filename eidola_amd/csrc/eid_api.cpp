@@ -14,9 +14,12 @@
 namespace eid {
 hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
                           const ItemTable *tab = nullptr);
-int splitkv_fill(int ntiles, bool fp8, int Hkv, bool pair = false);
+int splitkv_fill(int ntiles, bool fp8, int Hkv, bool pair = false, bool dma = false);
 hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream_t st,
                             const ItemTable *tab = nullptr);
+hipError_t launch_even(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
+                       const EvenTable *tab);
+int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma);
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
 long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
@@ -128,6 +131,7 @@ int32_t check_attn_desc(const eid_attn_desc *d) {
 struct Plan {
   int32_t partition, nparts_max, ws_rows;
   bool dynamic;
+  size_t parts_bytes;            // per-sequence piece counts of an even split (run-time partition)
   size_t ml_bytes, acc_bytes;
   int32_t pf_splits;             // key-range parts per prefill tile (1 = no split)
   size_t pf_ml_bytes, pf_acc_bytes;
@@ -199,6 +203,15 @@ Plan make_plan(const eid_attn_desc *d) {
   }
   pl.partition = P;
   pl.nparts_max = (span + P - 1) / P;
+  // Run-time partition: the launch is cut into equal ranges of chunks (at least P keys each),
+  // whose ends fall anywhere in a sequence: one more piece than whole partitions, and the
+  // count of every sequence's pieces goes through the workspace to the merge.
+  pl.parts_bytes = 0;
+  if (pl.dynamic && pl.nparts_max > 1) {
+    pl.nparts_max += 1;
+    pl.parts_bytes = ((size_t)d->num_seqs * sizeof(int32_t) + 255) / 256 * 256;
+  }
+  if (getenv("EID_EXP_ODD") && pl.nparts_max > 1) pl.nparts_max |= 1;
   pl.ws_rows = std::min(d->max_q_len, short_q_max(d));
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
   pl.ml_bytes = (cells * 2 * sizeof(float) + 255) / 256 * 256;
@@ -239,7 +252,7 @@ int32_t check_attn_args(const eid_attn_desc *d, const eid_attn_args *a, bool nee
   if (!need_ws) return EID_OK;
   const Plan pl = make_plan(d);
   const size_t need =
-      eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
+      eid::kPlanBytes + pl.parts_bytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
   if (!a->workspace || a->workspace_bytes < need)
     return fail(EID_ERR_WORKSPACE, "workspace of %zu bytes needed, %zu given", need,
                 a->workspace ? a->workspace_bytes : (size_t)0);
@@ -267,12 +280,13 @@ eid::AttnParams make_params(const eid_attn_desc *d, const eid_attn_args *a, cons
   uint8_t *ws = static_cast<uint8_t *>(a->workspace);
   p.plan = nullptr;
   p.plan_slot = nullptr;
-  p.ws_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes);
-  p.ws_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes);
+  const size_t head = eid::kPlanBytes + pl.parts_bytes;  // plan slots, then the piece counts
+  p.seq_parts = reinterpret_cast<int32_t *>(ws + eid::kPlanBytes);
+  p.ws_ml = reinterpret_cast<float *>(ws + head);
+  p.ws_acc = reinterpret_cast<_Float16 *>(ws + head + pl.ml_bytes);
   p.pf_splits = pl.pf_splits;
-  p.pf_ml = reinterpret_cast<float *>(ws + eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes);
-  p.pf_acc = reinterpret_cast<_Float16 *>(ws + eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes +
-                                          pl.pf_ml_bytes);
+  p.pf_ml = reinterpret_cast<float *>(ws + head + pl.ml_bytes + pl.acc_bytes);
+  p.pf_acc = reinterpret_cast<_Float16 *>(ws + head + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes);
   p.num_q_tokens = d->num_q_tokens;
   p.sum_kv_len = d->sum_kv_len;
   p.num_seqs = d->num_seqs;
@@ -509,7 +523,18 @@ struct ClassPlan {
   bool skip = false;      // no sequence of this class: launch nothing
   bool short_span = false;
   bool merge = false;     // some sequence has more than one partition
+  bool even = false;      // even split: equal contiguous ranges of the launch's units
 };
+
+// EID_EVEN=0 switches the even split off (the launches then take one workgroup per item), for
+// A/B measurements.
+bool even_allowed() {
+  static const bool on = [] {
+    const char *e = getenv("EID_EVEN");
+    return !(e && atoi(e) == 0);
+  }();
+  return on;
+}
 
 // Sets p.partition / p.dynamic_partition / p.exact_items for the class [qlen_lo, qlen_hi] and
 // says which kernel serves it.  Without host lengths this is the plan made from the
@@ -518,22 +543,40 @@ struct ClassPlan {
 // storage are then left to the kernels' own planning.
 ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan &pl,
                      eid::AttnParams &p, int ntiles, int32_t qlen_lo, int32_t qlen_hi,
-                     bool decode, eid::ItemTable *table = nullptr, bool no_heap = false,
-                     bool capturing = false) {
+                     bool decode, eid::EvenTable *etab, eid::ItemTable *table = nullptr,
+                     bool no_heap = false, bool capturing = false) {
   ClassPlan cp;
   if (table) table->n = table->has_blk = 0;
+  etab->n = etab->q = 0;
   const bool fp8 = d->kv_dtype == EID_KV_FP8_E4M3;
   p.qlen_lo = qlen_lo;
   p.qlen_hi = qlen_hi;
   p.partition = pl.partition;
   p.dynamic_partition = pl.dynamic ? 1 : 0;
   p.exact_items = 0;
-  p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0);
+  // bf16 cache and no prefill launch beside this one: the chunks stream in by direct global -> LDS loads
+  static const bool no_dma = getenv("EID_NO_DMA") != nullptr;  // for A/B measurements
+  p.dma = (!fp8 && !p.share_cus && !no_dma) ? 1 : 0;
+  p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0);
   cp.short_span = use_shortspan(d, pl, ntiles);
   cp.merge = pl.nparts_max > 1;
   constexpr int32_t kHostPlanMaxSeqs = 8192;  // beyond that the host pass is no longer free
   const int32_t *cu = decode ? nullptr : a->cu_seqlens_q_host;
-  if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) return cp;
+  // even split: one row group per KV head (no sequence of the class has more rows than a wave takes)
+  const bool even_ok = even_allowed() && pl.nparts_max > 1 && !cp.short_span &&
+                       (ntiles == 1 || ntiles == 3 || ntiles == 4);
+  p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0) : 0;
+  if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) {
+    // Without the lengths: a run-time partition always takes the even split (every workgroup
+    // finds its range by a scan of the device arrays); the caller's partition takes it when
+    // the bound on its items says that the launch is several device fills long.
+    if (even_ok) {
+      const long long span_sum = d->sum_kv_len > 0 && d->window == 0
+                                     ? d->sum_kv_len : (long long)d->num_seqs * max_span(d);
+      cp.even = pl.dynamic || span_sum / pl.partition + d->num_seqs >= 4LL * p.even_wgs;
+    }
+    return cp;
+  }
   int32_t stack_store[3 * eid::kStackPlanSeqs];  // 12 KiB: most batches need no heap at all
   std::vector<int32_t> heap_store;
   int32_t *store = stack_store;
@@ -552,9 +595,44 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
     return cp;
   }
   if (pl.nparts_max == 1) return cp;  // workgroup w serves sequence w: nothing to refine
+  const bool small_batch = pl.dynamic && eid::shortspan_applies(ntiles, fp8, c.items(eid::kShortSpanMax, pl.nparts_max),
+                                                                d->num_kv_heads);
+  // Even split: the launch's units (chunks, or partitions of the caller's size when there are
+  // at least two of them per workgroup) cut into equal contiguous ranges, one per workgroup.
+  const long long U = pl.dynamic ? eid::kChunk : pl.partition;
+  if (even_ok && !small_batch) {
+    long long C = 0;
+    for (size_t i = 0; i < c.n; ++i)
+      C += pl.dynamic ? (c.spans[i] + U - 1) / U : std::min<long long>((c.spans[i] + U - 1) / U, pl.nparts_max);
+    const long long G = p.even_wgs;
+    const long long q = std::max<long long>((C + G - 1) / G, pl.dynamic ? eid::kEvenMinChunks : 1);
+    const long long n = (C + q - 1) / q;
+    if (pl.dynamic || (C >= 2 * G && !(decode && table && C <= eid::kItemTableMax))) {
+      cp.even = true;
+      p.exact_items = n;
+      // where every workgroup's range starts, and whether any sequence is cut
+      bool cut = false;
+      long long pos = 0;  // units before sequence i
+      for (size_t i = 0; i < c.n; ++i) {
+        const long long n_s = pl.dynamic ? (c.spans[i] + U - 1) / U
+                                         : std::min<long long>((c.spans[i] + U - 1) / U, pl.nparts_max);
+        if (!pl.dynamic) cut = cut || n_s > 1;
+        else cut = cut || pos / q != (pos + n_s - 1) / q;
+        if (n <= eid::kEvenTableMax && c.seq[i] <= 0xffff)
+          for (long long b = (pos + q - 1) / q; b * q < pos + n_s; ++b)
+            etab->start[b] = (uint32_t)c.seq[i] | (uint32_t)(b * q - pos) << 16;
+        pos += n_s;
+      }
+      if (n <= eid::kEvenTableMax && (long long)d->max_kv_len / U + 1 < 0xffff && d->num_seqs <= 0xffff) {
+        etab->n = (int32_t)n;
+        etab->q = (int32_t)q;
+      }
+      cp.merge = cut;
+      return cp;
+    }
+  }
   if (pl.dynamic) {
-    const long long at512 = c.items(eid::kShortSpanMax, pl.nparts_max);
-    if (eid::shortspan_applies(ntiles, fp8, at512, d->num_kv_heads)) {
+    if (small_batch) {
       cp.short_span = true;  // small batch: one wave per chunk (see make_plan)
       p.partition = eid::kShortSpanMax;
     } else {
@@ -615,7 +693,7 @@ int32_t eid_partition_size(const eid_attn_desc *desc) {
 size_t eid_workspace_bytes(const eid_attn_desc *desc) {
   if (check_attn_desc(desc)) return 0;
   const Plan pl = make_plan(desc);
-  return eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
+  return eid::kPlanBytes + pl.parts_bytes + pl.ml_bytes + pl.acc_bytes + pl.pf_ml_bytes + pl.pf_acc_bytes;
 }
 
 int32_t eid_kv_write(const eid_attn_desc *desc, const void *k_new, const void *v_new,
@@ -764,14 +842,16 @@ static int32_t decode_launch(const eid_attn_desc *desc, const eid_attn_args *arg
   p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
   eid::ItemTable table;  // (8 KiB on the stack; only `n` entries are ever read)
-  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &table, no_heap, capturing);
+  eid::EvenTable etab;   // (4 KiB)
+  const ClassPlan cp = plan_class(desc, args, pl, p, 1, 1, 1, true, &etab, &table, no_heap, capturing);
   if (cp.skip) return EID_OK;  // (every sequence empty or malformed: nothing is written)
   const eid::ItemTable *tab = table.n > 0 ? &table : nullptr;
   // spans of at most 8 chunks, or a small batch in partitions of that size: one workgroup
   // per (sequence, partition, KV head), a chunk per wave
   if (cp.short_span) p.plan_slot = plan_slots;  // (the kernel records its partition there)
-  hipError_t e = cp.short_span ? eid::launch_shortspan(p, 1, fp8, st, tab)
-                               : eid::launch_splitkv(p, 1, fp8, plan_slots, st, tab);
+  hipError_t e = cp.even         ? eid::launch_even(p, 1, fp8, plan_slots, st, &etab)
+                 : cp.short_span ? eid::launch_shortspan(p, 1, fp8, st, tab)
+                                 : eid::launch_splitkv(p, 1, fp8, plan_slots, st, tab);
   if (cp.short_span) p.plan_slot = nullptr;     // (the merge of this call takes p.partition)
   if (e != hipSuccess) return hip_fail(e, "split-KV launch");
   if (args->split_done_event) {
@@ -802,7 +882,7 @@ int32_t eid_attn_decode_noalloc(const eid_attn_desc *desc, const eid_attn_args *
     return fail(EID_ERR_INVALID_ARG, "decode needs max_q_len == 1 and num_q_tokens == num_seqs");
   if (int32_t rc = check_attn_args(desc, args, true, false, false)) return rc;
   const Plan pl = make_plan(desc);
-  const size_t need = eid::kPlanBytes + pl.ml_bytes + pl.acc_bytes;
+  const size_t need = eid::kPlanBytes + pl.parts_bytes + pl.ml_bytes + pl.acc_bytes;
   if (need > eid::kStaticScratchBytes)
     return fail(EID_ERR_WORKSPACE,
                 "this batch needs %zu bytes of split-KV workspace; the library's static array holds "
@@ -839,7 +919,9 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool only_verify = uniform && desc->max_q_len > 2 && desc->max_q_len <= qmax;
   const bool only_prefill = uniform && desc->max_q_len > qmax;
   int32_t *plan_slots = static_cast<int32_t *>(args->workspace);
+  eid::EvenTable etab;  // (4 KiB)
   auto launch_split = [&](const ClassPlan &cp, const int ntiles, int32_t *slot) {
+    if (cp.even) return eid::launch_even(p, ntiles, fp8, slot, st, &etab);
     if (!cp.short_span) return eid::launch_splitkv(p, ntiles, fp8, slot, st);
     p.plan = nullptr;  // the short-span kernel works with the host's partition
     p.plan_slot = slot;  // ... and records it for a merge called by itself afterwards
@@ -869,7 +951,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   ClassPlan cp1;
   cp1.skip = true;
   if (!only_verify && !only_prefill) {
-    cp1 = plan_class(desc, args, pl, p, 1, 1, 2, false, nullptr, false, capturing);
+    cp1 = plan_class(desc, args, pl, p, 1, 1, 2, false, &etab, nullptr, false, capturing);
     if (!cp1.skip) {
       e = launch_split(cp1, 1, plan_slots);
       if (e != hipSuccess) return hip_fail(e, "split-KV launch");
@@ -901,7 +983,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   }
   if (desc->max_q_len > 2 && !only_prefill) {  // q_len 3..6: three tiles
     const int vt = verify_tiles(desc);
-    const ClassPlan cp3 = plan_class(desc, args, pl, p, vt, 3, qmax, false, nullptr, false, capturing);
+    const ClassPlan cp3 = plan_class(desc, args, pl, p, vt, 3, qmax, false, &etab, nullptr, false, capturing);
     if (!cp3.skip) {
       e = launch_split(cp3, vt, plan_slots + 2);
       if (e != hipSuccess) return hip_fail(e, "split-KV (verify) launch");

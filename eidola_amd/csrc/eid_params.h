@@ -25,6 +25,8 @@ constexpr int kPlanBytes = 256;         // head of the workspace: two {partition
 // which the decode entry point that allocates nothing uses in place of a caller's workspace.
 constexpr size_t kStaticScratchBytes = 32u << 20;
 constexpr int kStackPlanSeqs = 1024;    // sequences the host plans for without heap storage
+constexpr int kEvenMinChunks = kDynPartitionMin / kChunk;  // chunks per workgroup of an even split, at least
+constexpr int kEvenFlag = 1 << 29;      // plan slot of an even split with a run-time partition: flag | quota
 
 struct AttnParams {
   const uint16_t *q;
@@ -42,6 +44,9 @@ struct AttnParams {
   const float *v_scale;  // fp8 only
   const int32_t *plan;   // {partition, number of items} written by the plan kernel, or null
   int32_t *plan_slot;    // where this launch's split-KV kernel records its partition for the merge
+  int32_t *seq_parts;    // [num_seqs] pieces per sequence, written by an even split with a run-time
+                         // partition for its merge (the pieces have no common size)
+  int32_t even_wgs;      // workgroups of an even split (its grid)
   float *ws_ml;          // [num_seqs*ws_rows][nparts_max][Hq][2]  (m natural-log units, l)
   _Float16 *ws_acc;      // [num_seqs*ws_rows][nparts_max][Hq][64] partition output, normalised
   int32_t target_items_lo; // workgroups at one per CU (<= target_items)
@@ -63,6 +68,8 @@ struct AttnParams {
                              // eight KV heads: the split-KV launch may give each wave two KV heads
   int32_t share_cus;         // host-side launch flag: 1 = hold the split-KV kernel to one
                              // workgroup per CU (a prefill launch runs beside it)
+  int32_t dma;               // host-side launch flag: 1 = bf16 cache and no prefill launch beside: the
+                             // split-KV kernels stream their chunks by direct global -> LDS loads
   long long exact_items;     // host-side: the launch's exact number of work items when the host
                              // has the sequence lengths, 0 = not known (a bound is launched)
   float softmax_scale;
@@ -81,6 +88,15 @@ struct ItemTable {
   int32_t has_blk;  // blk[] holds the page ids of every item's first four pages
   unsigned long long e[kItemTableMax];
   int32_t blk[kItemTableMax][4];
+};
+
+// Start of every workgroup's range in an even split (see splitkv_even_kernel), listed by the
+// host when it has the sequence lengths: entry = seq | unit << 16, `q` units per workgroup.
+// n == 0: every workgroup finds its start by a scan of the device arrays.
+constexpr int kEvenTableMax = 1024;
+struct EvenTable {
+  int32_t n, q;
+  uint32_t start[kEvenTableMax];
 };
 
 // Query tiles of a prefill launch listed by the host, heaviest (most keys to walk) first:

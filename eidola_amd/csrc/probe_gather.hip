@@ -16,7 +16,13 @@ namespace {
 
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
-template <bool ROWS>
+template <bool NT>
+__device__ __forceinline__ u32x4 ld16(const uint8_t *p) {
+  if (NT) return __builtin_nontemporal_load((const u32x4 *)p);  // (streaming: no reuse expected)
+  return *(const u32x4 *)p;
+}
+
+template <bool ROWS, bool NT>
 __device__ __forceinline__ void load_batch(const uint8_t *pool, const int *tb, const int p0,
                                            const int n, const int lane, const int wave,
                                            u32x4 (&r)[8]) {
@@ -26,17 +32,17 @@ __device__ __forceinline__ void load_batch(const uint8_t *pool, const int *tb, c
     const int page = tb[p0 + (b < n ? b : n - 1)];  // (clamped: every load is issued)
     if (ROWS) {  // wave w takes token rows 2w, 2w+1 whole: 1 KiB contiguous per load instruction
       const size_t off = (size_t)page * 16384 + wave * 2048 + lane * 16;
-      r[2 * b] = *(const u32x4 *)(pool + off);
-      r[2 * b + 1] = *(const u32x4 *)(pool + off + 1024);
+      r[2 * b] = ld16<NT>(pool + off);
+      r[2 * b + 1] = ld16<NT>(pool + off + 1024);
     } else {  // wave w takes KV head w of all 16 rows: 16 slices of 128 bytes, 1 KiB apart
       const size_t off = (size_t)page * 16384 + i16 * 1024 + wave * 128 + g * 32;
-      r[2 * b] = *(const u32x4 *)(pool + off);
-      r[2 * b + 1] = *(const u32x4 *)(pool + off + 16);
+      r[2 * b] = ld16<NT>(pool + off);
+      r[2 * b + 1] = ld16<NT>(pool + off + 16);
     }
   }
 }
 
-template <bool ROWS>
+template <bool ROWS, bool NT>
 __global__ __launch_bounds__(512, 4) void gather_probe_kernel(const uint8_t *k, const uint8_t *v,
                                                               const int *table, const int pages_per_wg,
                                                               const int delay, uint32_t *sink) {
@@ -46,8 +52,8 @@ __global__ __launch_bounds__(512, 4) void gather_probe_kernel(const uint8_t *k, 
   for (int p0 = 0; p0 < pages_per_wg; p0 += 4) {
     const int n = min(4, pages_per_wg - p0);
     u32x4 a[8], b[8];
-    load_batch<ROWS>(k, tb, p0, n, lane, wave, a);
-    load_batch<ROWS>(v, tb, p0, n, lane, wave, b);
+    load_batch<ROWS, NT>(k, tb, p0, n, lane, wave, a);
+    load_batch<ROWS, NT>(v, tb, p0, n, lane, wave, b);
     uint32_t x = 0;
 #pragma unroll
     for (int i = 0; i < 8; ++i) x ^= a[i][0] ^ a[i][1] ^ a[i][2] ^ a[i][3] ^ b[i][0] ^ b[i][1] ^ b[i][2] ^ b[i][3];
@@ -64,7 +70,9 @@ extern "C" int eid_probe_gather(const void *k, const void *v, const int *table, 
                                 int pages_per_wg, int delay, int lds_bytes, int whole_rows,
                                 unsigned *sink, void *stream) {
   if (nwg < 1 || pages_per_wg < 1 || delay < 0 || lds_bytes < 0 || lds_bytes > 160 * 1024) return -1;
-  auto kern = whole_rows ? gather_probe_kernel<true> : gather_probe_kernel<false>;
+  // whole_rows: 0 head slices, 1 whole rows, 2 whole rows with non-temporal loads, 3 head slices with them
+  auto kern = whole_rows == 1 ? gather_probe_kernel<true, false> : whole_rows == 2 ? gather_probe_kernel<true, true>
+              : whole_rows == 3 ? gather_probe_kernel<false, true> : gather_probe_kernel<false, false>;
   if (lds_bytes > 64 * 1024 &&
       hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                           lds_bytes) != hipSuccess)

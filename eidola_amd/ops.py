@@ -486,7 +486,8 @@ def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_le
 
 def workspace_layout(desc):
     """(partition, nparts_max, ws_rows, ml_offset, acc_offset): after a 256-byte plan header
-    the split-KV workspace holds
+    (and, with a run-time partition, one int32 per sequence: its number of pieces) the
+    split-KV workspace holds
     ml  float32 [num_seqs*ws_rows, nparts_max, Hq, 2]  (m in natural-log units, l) and
     o   float16 [num_seqs*ws_rows, nparts_max, Hq, 64] (partition output sum e^(s-m) v / l) at
     the byte offsets returned."""
@@ -504,7 +505,13 @@ def workspace_layout(desc):
     else:
         span = desc.max_kv_len
     nparts = (span + P - 1) // P
+    head = 256
+    if desc.partition_size == 0 and P == 256 and nparts > 1:
+        # run-time partition (see make_plan in eid_api.cpp): equal ranges of chunks, whose ends
+        # fall anywhere in a sequence, and the per-sequence piece counts behind the plan header
+        nparts += 1
+        head += (desc.num_seqs * 4 + 255) // 256 * 256
     ws_rows = min(desc.max_q_len, qmax)
     cells = desc.num_seqs * ws_rows * desc.num_q_heads * nparts
     ml_bytes = (cells * 8 + 255) // 256 * 256
-    return P, nparts, ws_rows, 256, 256 + ml_bytes
+    return P, nparts, ws_rows, head, head + ml_bytes
