@@ -82,13 +82,18 @@ def split_kernel_ms(w, steps, torch):
 
 def split_kernel_dispatch_ms(w, steps, torch, ea):
     """Average milliseconds of the split-KV KERNEL inside full steps: a pair of HIP events per step
-    that the library attaches to the kernel's own dispatch (eid_debug_set_kernel_events,
-    hipExtLaunchKernel), so the time between them is the kernel's duration as rocprofv3 reports
-    it.  None when the step does not take the host-listed launch (no host copies of the lengths,
-    two launches, a captured stream): the events then stay as this function recorded them."""
+    that the MEASUREMENT build of the library (libeidola_attn_measure.so: the same sources with
+    -DEID_MEASURE, include/eidola_attn_measure.h) attaches to the kernel's own dispatch
+    (hipExtLaunchKernel), so the time between them is the kernel's duration as rocprofv3 reports
+    it.  The serving library has no such hook; the steps of this pass run through the
+    measurement build, every other figure of the run through the serving library."""
     if not w.fused:
         return None
-    lib = ea.load_library()
+    from eidola_amd import _lib
+    lib = _lib.load_measure_library()
+    calls = [c.bound_to(lib) for c in w.fused]
+    for i in range(2 * w.n):   # (the second library's first launches: module load, attributes)
+        calls[i % w.n]()
     pairs = []
     for _ in range(steps):
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -99,7 +104,7 @@ def split_kernel_dispatch_ms(w, steps, torch, ea):
     try:
         for i, (a, b) in enumerate(pairs):
             lib.eid_debug_set_kernel_events(a.cuda_event, b.cuda_event)
-            w.fused[i % w.n]()
+            calls[i % w.n]()
     finally:
         lib.eid_debug_set_kernel_events(None, None)
     torch.cuda.synchronize()
@@ -893,14 +898,15 @@ def timeline_bench(torch, ea, synth, np):
     64-token chunk), the stamps inside the kernel, how busy the device's workgroup slots are
     over the kernel's span and how long the tail is."""
     from eidola_amd import _lib
-    lib = _lib.load_library()
+    lib = _lib.load_measure_library()   # (the timeline hook exists in the measurement build only)
     res = []
 
     def one(name, w, waves, unit_name, slots_per_cu):
+        attn = [c.bound_to(lib) for c in w.attn]
         n_rec = 1 << 17
         buf = torch.zeros(n_rec * 8, dtype=torch.int64, device="cuda:0")
         for i in range(300):   # (past the clock's settling time)
-            w.attn[i % w.n]()
+            attn[i % w.n]()
         torch.cuda.synchronize()
         lib.eid_debug_set_timeline(buf.data_ptr(), n_rec)
         try:
@@ -908,7 +914,7 @@ def timeline_bench(torch, ea, synth, np):
             for rep in range(3):
                 buf.zero_()
                 for i in range(20):   # the last of back-to-back calls is the one recorded
-                    w.attn[(rep + i) % w.n]()
+                    attn[(rep + i) % w.n]()
                 torch.cuda.synchronize()
                 runs.append(buf.view(-1, 8).cpu().numpy().copy())
         finally:

@@ -103,13 +103,15 @@ class BatchInfo(C.Structure):
 
 EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_qkv_rope_kv_write", "eid_attn_decode",
            "eid_attn_decode_noalloc", "eid_attn_varlen", "eid_lse_merge", "eid_o_proj",
-           "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version",
-           "eid_debug_set_timeline", "eid_debug_set_kernel_events")
+           "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
+# only in the measurement build (include/eidola_attn_measure.h)
+MEASURE_EXPORTS = ("eid_debug_set_timeline", "eid_debug_set_kernel_events")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
                  "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
                  "eid_sched_block_refs", "eid_sched_build_batch")
 
 _lib = None
+_measure_lib = None
 
 
 def lib_path():
@@ -120,12 +122,32 @@ def lib_path():
                         "libeidola_attn_hip.so")
 
 
+def measure_lib_path():
+    override = os.environ.get("EID_ATTN_MEASURE_LIB")
+    if override:
+        return override
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
+                        "libeidola_attn_measure.so")
+
+
+def load_measure_library():
+    """The measurement build of the library (the same sources with -DEID_MEASURE): a second,
+    independent copy in the process, with the two eid_debug_* hooks.  For benchmarks only."""
+    global _measure_lib
+    if _measure_lib is None:
+        _measure_lib = _bind(measure_lib_path(), measure=True)
+    return _measure_lib
+
+
 def load_library():
     """Load the HIP library; raises (never falls back) when it has not been built."""
     global _lib
-    if _lib is not None:
-        return _lib
-    path = lib_path()
+    if _lib is None:
+        _lib = _bind(lib_path(), measure=False)
+    return _lib
+
+
+def _bind(path, measure):
     if not os.path.exists(path):
         raise EidError(EID_ERR_HIP, f"{path} is missing: run `python -c 'import "
                        "__graft_entry__ as g; g.build()'` or `make -C eidola_amd/csrc`")
@@ -153,10 +175,11 @@ def load_library():
     lib.eid_last_error.restype = C.c_char_p
     lib.eid_version.argtypes = []
     lib.eid_version.restype = C.c_uint32
-    lib.eid_debug_set_timeline.argtypes = [P, C.c_int64]
-    lib.eid_debug_set_timeline.restype = None
-    lib.eid_debug_set_kernel_events.argtypes = [P, P]
-    lib.eid_debug_set_kernel_events.restype = None
+    if measure:
+        lib.eid_debug_set_timeline.argtypes = [P, C.c_int64]
+        lib.eid_debug_set_timeline.restype = None
+        lib.eid_debug_set_kernel_events.argtypes = [P, P]
+        lib.eid_debug_set_kernel_events.restype = None
     # host-side scheduler (include/eidola_sched.h)
     lib.eid_sched_create.argtypes = [C.POINTER(SchedConfig), C.POINTER(P)]
     lib.eid_sched_create.restype = C.c_int32
@@ -175,7 +198,6 @@ def load_library():
     lib.eid_sched_build_batch.argtypes = [P, P, P, C.c_int32, P, P, P, P, P, P,
                                           C.POINTER(BatchInfo)]
     lib.eid_sched_build_batch.restype = C.c_int32
-    _lib = lib
     return lib
 
 

@@ -584,13 +584,25 @@ struct FirstPages {
 
 // No partials inside the key range (the default `emit` of attend).
 struct NoEmit {
-  __device__ __forceinline__ void operator()(int) const {}
+  __device__ __forceinline__ int operator()(int) const { return 0; }
 };
+
+// Waits until at most `n` of the wave's vector memory operations are outstanding (they
+// complete in the order they were issued): the loads issued before the youngest n, stores, say.
+__device__ __forceinline__ void wait_vm_all_but(const int n) {
+  if (n >= 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  else if (n >= 9) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+  else if (n >= 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+  else if (n >= 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
 
 // `emit_every` > 0 (a multiple of the chunk): after every `emit_every` keys from t_begin, except
 // at the end of the range, emit(k) is called with k = 0, 1, ...: the caller stores the partial
 // of that stretch and resets m / lacc / acc, and the loop goes on with the next stretch, its
 // page ids already under way (a range of several partitions walked without a new start).
+// emit returns a lower bound on the number of store instructions it issued (attend_dma lets
+// that many operations stay outstanding when it next waits for its loads).
 template <int NT, bool FP8, bool PAIR = false, class Emit = NoEmit>
 __device__ __forceinline__ void attend(const AttnParams &p, const int s, const int kvh,
                                        const int t_begin, const int t_end, const int seq_len,
@@ -873,9 +885,12 @@ __device__ __forceinline__ void attend_dma(const AttnParams &p, const int s, con
   if (t_begin + kChunk < t_end) pages_of(t_begin + kChunk, blk_next);
 
   int emit_left = emit_every, emit_k = 0;
+  int stores_behind = 0;  // store instructions issued after the loads that are waited for next
   for (int ti = t_begin; ti < t_end; ti += kChunk) {
-    // this chunk's tiles have landed
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // this chunk's tiles have landed (a partial stored since they were requested may still be
+    // on its way: stores behind the loads need not be waited for)
+    wait_vm_all_but(stores_behind);
+    stores_behind = 0;
     Frag8 kf[4][2], vf[4][2];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -895,7 +910,7 @@ __device__ __forceinline__ void attend_dma(const AttnParams &p, const int s, con
     if constexpr (!std::is_same<Emit, NoEmit>::value) {
       emit_left -= kChunk;
       if (emit_left == 0 && ti + kChunk < t_end) {  // (wave-uniform)
-        emit(emit_k++);
+        stores_behind = emit(emit_k++);
         emit_left = emit_every;
       }
     }
@@ -1396,16 +1411,23 @@ __global__ __launch_bounds__(WAVES * 64, ((NT == 1 && !DMA) ? 4 : 2)) void split
 // Here the launch's units - 64-key chunks (run-time partition) or partitions of the caller's
 // size - are laid out sequence after sequence and cut into gridDim.x equal, contiguous ranges
 // of `q` units: workgroup b walks units [b q, (b + 1) q), from the middle of one sequence
-// through whole sequences into the start of another.  Q is loaded once per sequence visited,
-// the page-id prefetch runs through, and partials are stored where a range leaves a
-// (sequence, partition) cell: at the end of the range, at the end of a sequence, and every
-// `partition` keys when the caller fixed the partition.  Equal unit counts are equal work.
+// through whole sequences into the start of another.  Q is loaded once per sequence visited
+// and the page-id prefetch runs through.  Equal unit counts are equal work.
 //
-// Run-time partition: the pieces of a sequence have no common size.  Piece index = workgroup
-// id - id of the workgroup holding the sequence's first unit; the workgroup that holds the
-// first unit records the sequence's number of pieces in p.seq_parts for the merge, and the
-// plan slot receives kEvenFlag | q.  With q >= kEvenMinChunks a sequence of n chunks has at
-// most ceil(n / kEvenMinChunks) + 1 pieces, which is what the workspace is sized for.
+// What a workgroup holds of one sequence is one PIECE: it carries (m, l, acc) through the
+// piece's units - the rescaling of the online softmax IS the log-sum-exp merge of consecutive
+// partitions, done in registers - and stores one partial where its range leaves the sequence.
+// The caller's partition size is then the grid on which ranges may be cut, not a number of
+// round trips through memory: on this machine stores trickling into a saturated stream of
+// loads are dear out of all proportion (a plain gather of config 5's pages at 6.9 TB/s drops
+// to 4.9 TB/s when 4 % of its traffic is partial stores), so a partial per 512 keys costs a
+// quarter of the run time.  p.store_every_partition (a measurement aid) restores that form:
+// a partial per partition, all of them merged by the merge kernel.
+// The pieces of a sequence have no common size.  Piece index = workgroup id - id of the
+// workgroup holding the sequence's first unit; that workgroup records the sequence's number
+// of pieces in p.seq_parts for the merge, and the plan slot receives kEvenFlag | q.  With a
+// run-time partition q >= kEvenMinChunks, so a sequence of n chunks has at most
+// ceil(n / kEvenMinChunks) + 1 pieces, which is what the workspace is sized for.
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ SeqView view_seq_uniform(const AttnParams &p, const int s) {
   // (s is wave-uniform: the loads go through the scalar unit)
@@ -1492,8 +1514,10 @@ __global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kerne
     s = __builtin_amdgcn_readfirstlane(start_lds[1]);
     u = __builtin_amdgcn_readfirstlane(start_lds[2]);
   }
-  // the merge that follows reads the mode (and, with the caller's partition, its size) from here
-  if (b == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = dyn ? (kEvenFlag | q) : p.partition;
+  // pieces (one partial per workgroup and sequence), or a partial per partition of the caller's
+  const bool pieces = dyn || !p.store_every_partition;
+  // the merge that follows reads the mode (and, with a partial per partition, its size) from here
+  if (b == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = pieces ? (kEvenFlag | q) : p.partition;
   const int U = dyn ? kChunk : p.partition;  // keys per unit
   uint8_t *wave_lds = lds + wave * (DMA ? kWaveDmaBytes : kWaveLdsBytes);
   int rem = q;
@@ -1520,7 +1544,7 @@ __global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kerne
     const int lo_last = p.window > 0 ? max(0, L - p.window) : 0;
     // the piece (run-time partition) or the first partition (caller's) and the sequence's count
     int part, nparts;
-    if (dyn) {
+    if (pieces) {
       // units before this sequence: (b q + units of the range used up so far) - u_now
       part = first_seq ? (u_now + q - 1) / q : 0;
       // first workgroup of the sequence holds its unit 0: the sequence starts `off` units into it
@@ -1551,14 +1575,16 @@ __global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kerne
     auto emit = [&](const int k) {
       finish<NT, FP8, PAIR>(p, s_now, kvh, row0, qlen, 0, false, part + k, m, lacc, acc);
       reset();
+      // finish() stores (m, l) and two 16-byte pieces per lane for every tile that holds a row
+      return 3 * min(NT, (qlen + 1) / 2);
     };
     if constexpr (DMA)
       attend_dma<NT>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, FirstPages{},
-                     dyn ? 0 : U, emit);
+                     pieces ? 0 : U, emit);
     else
       attend<NT, FP8, PAIR>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc,
-                            FirstPages{}, dyn ? 0 : U, emit);
-    finish<NT, FP8, PAIR>(p, s_now, kvh, row0, qlen, 0, direct, dyn ? part : part + n_here - 1, m, lacc, acc);
+                            FirstPages{}, pieces ? 0 : U, emit);
+    finish<NT, FP8, PAIR>(p, s_now, kvh, row0, qlen, 0, direct, pieces ? part : part + n_here - 1, m, lacc, acc);
   }
 }
 
@@ -2205,7 +2231,11 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
         if (EAGER && c0 == 0 && j0 == 0) {
           if (c < nparts) v[j] = v_early[j];
         } else {
-          if (c < nparts) v[j] = *(const uint2 *)(acc_row + (size_t)c * cstride * kHeadDim);
+          // (16 lanes take one 128-byte cell: whole lines, read once: streaming hint)
+          if (c < nparts) {
+            const u32x2 x = __builtin_nontemporal_load((const u32x2 *)(acc_row + (size_t)c * cstride * kHeadDim));
+            v[j] = make_uint2(x[0], x[1]);
+          }
         }
       }
 #pragma unroll
@@ -2548,27 +2578,52 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
   return num_items * Hkv <= fill[ntiles == 1 ? 0 : ntiles == 3 ? 1 : 2][fp8 ? 1 : 0];
 }
 
-// Measurement aid: a device buffer of `entries` records of 64 bytes that the next prefill
-// launches of the process fill with per-wave time stamps (null: off).
-// Not thread-safe; launches with more waves than entries leave the buffer alone.
-static unsigned long long *g_timeline = nullptr;
-static long long g_timeline_entries = 0;
+// Measurement aids, compiled into the measurement build only (-DEID_MEASURE): the serving
+// library carries neither the entry points nor their process-wide state.
+//  * a device buffer of `entries` records of 64 bytes that the next prefill launches of the
+//    process fill with per-wave time stamps (null: off; launches with more waves than entries
+//    leave the buffer alone);
+//  * a pair of HIP events that the next decode launches attach to the split-KV kernel's own
+//    dispatch (hipExtLaunchKernel): the time between them is the kernel's duration as a
+//    profiler reports it, without the gaps that events recorded around a launch include.
+// The settings are read once per launch (atomics); what they point to is the caller's and
+// must outlive the setting.
+#ifdef EID_MEASURE
+static std::atomic<unsigned long long *> g_timeline{nullptr};
+static std::atomic<long long> g_timeline_entries{0};
 void set_timeline(void *buf, long long entries) {
-  g_timeline = static_cast<unsigned long long *>(buf);
-  g_timeline_entries = buf ? entries : 0;
+  g_timeline_entries.store(0);
+  g_timeline.store(static_cast<unsigned long long *>(buf));
+  g_timeline_entries.store(buf ? entries : 0);
 }
 static unsigned long long *timeline_for(const long long waves) {
-  return waves <= g_timeline_entries ? g_timeline : nullptr;
+  return waves <= g_timeline_entries.load() ? g_timeline.load() : nullptr;
 }
-
-// Measurement aid: a pair of HIP events that the next decode launches with a host-listed item
-// table attach to the split-KV kernel's own dispatch (hipExtLaunchKernelGGL): the time between
-// them is the kernel's duration as a profiler reports it, without the gaps that events recorded
-// around a launch include.  Null: off.  Not thread-safe.
-static hipEvent_t g_kernel_start = nullptr, g_kernel_stop = nullptr;
+static std::atomic<hipEvent_t> g_kernel_start{nullptr}, g_kernel_stop{nullptr};
 void set_kernel_events(void *start, void *stop) {
-  g_kernel_start = static_cast<hipEvent_t>(start);
-  g_kernel_stop = static_cast<hipEvent_t>(stop);
+  g_kernel_start.store(static_cast<hipEvent_t>(start));
+  g_kernel_stop.store(static_cast<hipEvent_t>(stop));
+}
+#else
+static unsigned long long *timeline_for(const long long) { return nullptr; }
+#endif
+
+// Launches `kern`; in the measurement build, with the two events attached to the dispatch when
+// they are set and the launch is one that they are meant for (`timed`).
+template <typename K, typename... A>
+static hipError_t launch_kernel(K kern, dim3 grid, dim3 block, unsigned shmem, hipStream_t st,
+                                bool timed, const A &...a) {
+#ifdef EID_MEASURE
+  const hipEvent_t e0 = g_kernel_start.load(), e1 = g_kernel_stop.load();
+  if (timed && e0 && e1) {
+    void *kargs[] = {const_cast<void *>(static_cast<const void *>(&a))...};
+    return hipExtLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, kargs, shmem, st, e0, e1, 0);
+  }
+#else
+  (void)timed;
+#endif
+  kern<<<grid, block, shmem, st>>>(a...);
+  return hipGetLastError();
 }
 
 // Workgroups of an even split: resident all at once, one 8-wave workgroup per CU (eight waves
@@ -2611,11 +2666,10 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
 template <int NT, bool FP8, int WAVES, bool PAIR = false>
 static hipError_t launch_even_w(const AttnParams &p, const EvenTable &tab, hipStream_t st) {
   dim3 grid((unsigned)(tab.n > 0 ? tab.n : p.even_wgs), p.num_kv_heads / WAVES / (PAIR ? 2 : 1));
+  const bool timed = NT == 1 && p.cu_seqlens_q == nullptr;  // (the decode entry point's launch)
   if constexpr (!FP8) {
-    if (p.dma) {
-      splitkv_even_kernel<NT, FP8, WAVES, PAIR, true><<<grid, WAVES * 64, 0, st>>>(p, tab);
-      return hipGetLastError();
-    }
+    if (p.dma)
+      return launch_kernel(splitkv_even_kernel<NT, FP8, WAVES, PAIR, true>, grid, dim3(WAVES * 64), 0, st, timed, p, tab);
   }
   // (p.share_cus: one 8-wave workgroup per CU by a request for unused dynamic LDS, see launch_splitkv_w)
   const int kPad = (WAVES == 8 && p.share_cus) ? 16384 : 0;
@@ -2631,8 +2685,7 @@ static hipError_t launch_even_w(const AttnParams &p, const EvenTable &tab, hipSt
       if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
     }
   }
-  splitkv_even_kernel<NT, FP8, WAVES, PAIR><<<grid, WAVES * 64, kPad, st>>>(p, tab);
-  return hipGetLastError();
+  return launch_kernel(splitkv_even_kernel<NT, FP8, WAVES, PAIR>, grid, dim3(WAVES * 64), kPad, st, timed, p, tab);
 }
 template <int NT, bool FP8>
 static hipError_t launch_even_t(const AttnParams &p, const EvenTable &tab, hipStream_t st) {
@@ -2673,17 +2726,10 @@ hipError_t launch_splitkv(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slo
   if (tab && ntiles == 1 && p.nparts_max > 1 && !p.dynamic_partition && !p.share_cus &&
       waves_for(p.num_kv_heads) == 8) {
     dim3 grid((unsigned)tab->n, p.num_kv_heads / 8);
-    if (g_kernel_start && g_kernel_stop && !fp8) {
-      void *kargs[] = {const_cast<AttnParams *>(&p), const_cast<ItemTable *>(tab)};
-      return hipExtLaunchKernel(p.dma ? reinterpret_cast<const void *>(splitkv_table_kernel<1, false, 8, false, true>)
-                                      : reinterpret_cast<const void *>(splitkv_table_kernel<1, false, 8>),
-                                grid, dim3(512), kargs, 0, st, g_kernel_start, g_kernel_stop, 0);
-    }
-    if (fp8 && p.fp8_pair) splitkv_table_kernel<1, true, 4, true><<<grid, 256, 0, st>>>(p, *tab);
-    else if (fp8) splitkv_table_kernel<1, true, 8><<<grid, 512, 0, st>>>(p, *tab);
-    else if (p.dma) splitkv_table_kernel<1, false, 8, false, true><<<grid, 512, 0, st>>>(p, *tab);
-    else splitkv_table_kernel<1, false, 8><<<grid, 512, 0, st>>>(p, *tab);
-    return hipGetLastError();
+    if (fp8 && p.fp8_pair) return launch_kernel(splitkv_table_kernel<1, true, 4, true>, grid, dim3(256), 0, st, true, p, *tab);
+    if (fp8) return launch_kernel(splitkv_table_kernel<1, true, 8>, grid, dim3(512), 0, st, true, p, *tab);
+    if (p.dma) return launch_kernel(splitkv_table_kernel<1, false, 8, false, true>, grid, dim3(512), 0, st, true, p, *tab);
+    return launch_kernel(splitkv_table_kernel<1, false, 8>, grid, dim3(512), 0, st, true, p, *tab);
   }
   if (p.nparts_max > 1 && p.exact_items == 0 && item_bound(p) > 4LL * p.target_items) {
     AttnParams q = p;

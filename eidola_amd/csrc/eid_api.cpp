@@ -3,6 +3,9 @@
 #include <hip/hip_runtime.h>
 
 #include "../../include/eidola_attn.h"
+#ifdef EID_MEASURE
+#include "../../include/eidola_attn_measure.h"
+#endif
 #include "eid_params.h"
 #include <algorithm>
 #include <cmath>
@@ -24,8 +27,10 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
 long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
                           const PfTable *tab);
+#ifdef EID_MEASURE
 void set_timeline(void *buf, long long entries);
 void set_kernel_events(void *start, void *stop);
+#endif
 bool build_prefill_table(const AttnParams &p, const int32_t *seq_lens_host,
                          const int32_t *cu_seqlens_q_host, PfTable *tab);
 hipError_t launch_merge(const AttnParams &p, hipStream_t st);
@@ -203,12 +208,13 @@ Plan make_plan(const eid_attn_desc *d) {
   }
   pl.partition = P;
   pl.nparts_max = (span + P - 1) / P;
-  // Run-time partition: the launch is cut into equal ranges of chunks (at least P keys each),
-  // whose ends fall anywhere in a sequence: one more piece than whole partitions, and the
-  // count of every sequence's pieces goes through the workspace to the merge.
+  // An even split cuts the launch into equal ranges of units, and the count of every sequence's
+  // pieces goes through the workspace to the merge.  Run-time partition: the units are chunks
+  // (ranges of at least P keys), and a range's ends fall anywhere in a sequence: one more
+  // piece than whole partitions.
   pl.parts_bytes = 0;
-  if (pl.dynamic && pl.nparts_max > 1) {
-    pl.nparts_max += 1;
+  if (pl.nparts_max > 1) {
+    if (pl.dynamic) pl.nparts_max += 1;
     pl.parts_bytes = ((size_t)d->num_seqs * sizeof(int32_t) + 255) / 256 * 256;
   }
   if (getenv("EID_EXP_ODD") && pl.nparts_max > 1) pl.nparts_max |= 1;
@@ -566,6 +572,8 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   const bool even_ok = even_allowed() && pl.nparts_max > 1 && !cp.short_span &&
                        (ntiles == 1 || ntiles == 3 || ntiles == 4);
   p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0) : 0;
+  static const bool every = getenv("EID_STORE_EVERY_PARTITION") != nullptr;  // measurement aid
+  p.store_every_partition = every ? 1 : 0;
   if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) {
     // Without the lengths: a run-time partition always takes the even split (every workgroup
     // finds its range by a scan of the device arrays); the caller's partition takes it when
@@ -616,7 +624,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
       for (size_t i = 0; i < c.n; ++i) {
         const long long n_s = pl.dynamic ? (c.spans[i] + U - 1) / U
                                          : std::min<long long>((c.spans[i] + U - 1) / U, pl.nparts_max);
-        if (!pl.dynamic) cut = cut || n_s > 1;
+        if (p.store_every_partition && !pl.dynamic) cut = cut || n_s > 1;
         else cut = cut || pos / q != (pos + n_s - 1) / q;
         if (n <= eid::kEvenTableMax && c.seq[i] <= 0xffff)
           for (long long b = (pos + q - 1) / q; b * q < pos + n_s; ++b)
@@ -679,11 +687,13 @@ uint32_t eid_version(void) { return (EID_VERSION_MAJOR << 16) | EID_VERSION_MINO
 
 const char *eid_last_error(void) { return g_err; }
 
+#ifdef EID_MEASURE
 void eid_debug_set_timeline(void *device_buf, int64_t entries) { eid::set_timeline(device_buf, entries); }
 
 void eid_debug_set_kernel_events(void *start_event, void *stop_event) {
   eid::set_kernel_events(start_event, stop_event);
 }
+#endif
 
 int32_t eid_partition_size(const eid_attn_desc *desc) {
   if (check_attn_desc(desc)) return 0;

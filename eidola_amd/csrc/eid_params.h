@@ -26,7 +26,7 @@ constexpr int kPlanBytes = 256;         // head of the workspace: two {partition
 constexpr size_t kStaticScratchBytes = 32u << 20;
 constexpr int kStackPlanSeqs = 1024;    // sequences the host plans for without heap storage
 constexpr int kEvenMinChunks = kDynPartitionMin / kChunk;  // chunks per workgroup of an even split, at least
-constexpr int kEvenFlag = 1 << 29;      // plan slot of an even split with a run-time partition: flag | quota
+constexpr int kEvenFlag = 1 << 29;      // plan slot of an even split that stored pieces: flag | quota
 
 struct AttnParams {
   const uint16_t *q;
@@ -44,9 +44,11 @@ struct AttnParams {
   const float *v_scale;  // fp8 only
   const int32_t *plan;   // {partition, number of items} written by the plan kernel, or null
   int32_t *plan_slot;    // where this launch's split-KV kernel records its partition for the merge
-  int32_t *seq_parts;    // [num_seqs] pieces per sequence, written by an even split with a run-time
-                         // partition for its merge (the pieces have no common size)
+  int32_t *seq_parts;    // [num_seqs] pieces per sequence, written by an even split for its merge
+                         // (the pieces have no common size)
   int32_t even_wgs;      // workgroups of an even split (its grid)
+  int32_t store_every_partition;  // even split with the caller's partition: a partial per partition
+                         // instead of one per piece (measurement aid, EID_STORE_EVERY_PARTITION)
   float *ws_ml;          // [num_seqs*ws_rows][nparts_max][Hq][2]  (m natural-log units, l)
   _Float16 *ws_acc;      // [num_seqs*ws_rows][nparts_max][Hq][64] partition output, normalised
   int32_t target_items_lo; // workgroups at one per CU (<= target_items)

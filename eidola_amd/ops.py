@@ -367,6 +367,13 @@ class PreparedCall:
             check(rc)
         return self.out
 
+    def bound_to(self, lib):
+        """The same call through another build of the library (the measurement build)."""
+        other = PreparedCall.__new__(PreparedCall)
+        other.__dict__.update(self.__dict__)
+        other._fn = getattr(lib, self._fn.__name__)
+        return other
+
 
 def prepare(fn_name, geom, q, k_cache, v_cache, block_table, seq_lens, cu_seqlens_q=None, *,
             max_q_len=1, max_kv_len, sinks=None, k_scale=None, v_scale=None, out=None, lse=None,
@@ -486,8 +493,8 @@ def lse_merge(geom, workspace, seq_lens, cu_seqlens_q, *, num_q_tokens, max_q_le
 
 def workspace_layout(desc):
     """(partition, nparts_max, ws_rows, ml_offset, acc_offset): after a 256-byte plan header
-    (and, with a run-time partition, one int32 per sequence: its number of pieces) the
-    split-KV workspace holds
+    (and, when a sequence can have more than one partition, one int32 per sequence: its number
+    of pieces) the split-KV workspace holds
     ml  float32 [num_seqs*ws_rows, nparts_max, Hq, 2]  (m in natural-log units, l) and
     o   float16 [num_seqs*ws_rows, nparts_max, Hq, 64] (partition output sum e^(s-m) v / l) at
     the byte offsets returned."""
@@ -506,10 +513,12 @@ def workspace_layout(desc):
         span = desc.max_kv_len
     nparts = (span + P - 1) // P
     head = 256
-    if desc.partition_size == 0 and P == 256 and nparts > 1:
-        # run-time partition (see make_plan in eid_api.cpp): equal ranges of chunks, whose ends
-        # fall anywhere in a sequence, and the per-sequence piece counts behind the plan header
-        nparts += 1
+    if nparts > 1:
+        # (see make_plan in eid_api.cpp) the per-sequence piece counts of an even split sit behind
+        # the plan header; with a run-time partition the ranges are cut anywhere in a sequence:
+        # one more piece than whole partitions
+        if desc.partition_size == 0 and P == 256:
+            nparts += 1
         head += (desc.num_seqs * 4 + 255) // 256 * 256
     ws_rows = min(desc.max_q_len, qmax)
     cells = desc.num_seqs * ws_rows * desc.num_q_heads * nparts

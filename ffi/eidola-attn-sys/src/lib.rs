@@ -187,10 +187,6 @@ unsafe extern "C" {
 
     pub fn eid_version() -> u32;
 
-    pub fn eid_debug_set_timeline(device_buf: *mut c_void, entries: i64);
-
-    pub fn eid_debug_set_kernel_events(start_event: *mut c_void, stop_event: *mut c_void);
-
     pub fn eid_sched_create(cfg: *const eid_sched_config, out: *mut *mut eid_sched) -> i32;
 
     pub fn eid_sched_destroy(s: *mut eid_sched);

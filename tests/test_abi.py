@@ -41,13 +41,17 @@ def test_workspace_and_partition_planning():
     d = good_desc()
     P = ea.partition_size(d)
     assert P % 64 == 0 and 64 <= P <= 4096
-    nparts = (1000 + P - 1) // P
+    # plan header, one int32 per sequence (pieces of an even split), then (m, l) and the outputs;
+    # a run-time partition plans one more piece than whole partitions of 256 keys
+    Pl, nparts, ws_rows, ml_off, acc_off = ea.ops.workspace_layout(d)
+    assert Pl == P and ws_rows == 1 and nparts == (1000 + P - 1) // P + (1 if d.partition_size == 0 and P == 256 else 0)
     cells = 4 * 1 * 64 * nparts
-    assert ea.workspace_bytes(d) == 256 + (cells * 8 + 255) // 256 * 256 + cells * 128
+    assert ml_off == 256 + 256 and acc_off == ml_off + (cells * 8 + 255) // 256 * 256
+    assert ea.workspace_bytes(d) == acc_off + cells * 128
     d5 = ea.make_desc(ea.AttnGeometry(partition_size=512), num_seqs=128, num_q_tokens=640,
                       max_q_len=5, max_kv_len=65536, max_blocks_per_seq=4096, num_blocks=300000)
     assert ea.partition_size(d5) == 512
-    assert ea.workspace_bytes(d5) == 256 + 128 * 5 * 64 * 128 * (8 + 128)
+    assert ea.workspace_bytes(d5) == 256 + 512 + 128 * 5 * 64 * 128 * (8 + 128)
     # at least one sequence per CU (256 without a device to ask) and no span beyond 2,048
     # tokens: every sequence is planned as one work item, and the workspace shrinks to it
     dm = ea.make_desc(ea.AttnGeometry(), num_seqs=300, num_q_tokens=300, max_q_len=1,

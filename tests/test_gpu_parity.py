@@ -752,31 +752,36 @@ def test_host_copies_of_the_lengths_plan_the_launches(G, kv_dtype, window, parti
 
 
 def test_kernel_events_time_the_split_kv_dispatch(G):
-    """eid_debug_set_kernel_events: a decode call on the host-listed path attaches the two events
-    to the split-KV kernel's dispatch; the outputs do not change, the time between the events is
-    a kernel's worth, and once switched off the events are left alone."""
+    """eid_debug_set_kernel_events exists in the measurement build only (-DEID_MEASURE): a decode
+    call through that build attaches the two events to the split-KV kernel's dispatch; the
+    outputs equal the serving library's, the time between the events is a kernel's worth, and
+    once switched off the events are left alone.  The serving library has no such symbol."""
     from eidola_amd import _lib
-    lib = _lib.load_library()
+    assert not hasattr(_lib.load_library(), "eid_debug_set_kernel_events")
+    lib = _lib.load_measure_library()
     rng = np.random.default_rng(77)
     seq_lens = rng.integers(3000, 9000, size=24)
     b = make_batch(seq_lens, [1] * len(seq_lens), partition=0)
     q, k, v, sinks = logical_tensors(b, seed=9)
     kc_d, vc_d = G.gpu_caches(b, k, v)
     plain = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=True, hint=True)
+    call = ea.prepare("eid_attn_decode", b.geom, G.bf16_dev(q), kc_d, vc_d, G.dev(b.block_table),
+                      G.dev(b.seq_lens), max_kv_len=b.max_kv_len, sinks=G.dev(sinks),
+                      sum_kv_len=int(b.seq_lens.sum()), seq_lens_host=b.seq_lens).bound_to(lib)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     e1.record()
     torch.cuda.synchronize()
     lib.eid_debug_set_kernel_events(e0.cuda_event, e1.cuda_event)
     try:
-        timed = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=True, hint=True)
+        timed = G.bits_host(call()).copy()
     finally:
         lib.eid_debug_set_kernel_events(None, None)
     torch.cuda.synchronize()
     assert np.array_equal(timed, plain)
     ms = e0.elapsed_time(e1)
     assert 0.005 < ms < 5.0, ms    # ~0.3 GB of KV: tens of microseconds, not the back-to-back records
-    again = G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=True, hint=True)
+    again = G.bits_host(call()).copy()
     torch.cuda.synchronize()
     assert np.array_equal(again, plain) and e0.elapsed_time(e1) == ms
 
