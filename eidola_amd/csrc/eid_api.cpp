@@ -572,6 +572,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   const bool even_ok = even_allowed() && pl.nparts_max > 1 && !cp.short_span &&
                        (ntiles == 1 || ntiles == 3 || ntiles == 4);
   p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0) : 0;
+  if (p.mixed_wgs > 0 && p.even_wgs > p.mixed_wgs) p.even_wgs = p.mixed_wgs;
   static const bool every = getenv("EID_STORE_EVERY_PARTITION") != nullptr;  // measurement aid
   p.store_every_partition = every ? 1 : 0;
   if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) {
@@ -945,7 +946,27 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
   const bool has_prefill = desc->max_q_len > qmax;
   static const bool serial = getenv("EID_SERIAL_CLASSES") != nullptr;  // for A/B measurements
   Helper *hs = (has_prefill && !only_prefill && !serial) ? helper_stream() : nullptr;
-  p.share_cus = hs ? 1 : 0;
+  // Two ways to run the classes on two streams.  fp8 cache (and EID_MIXED=share): the split-KV
+  // kernels are held to one register-staged workgroup per CU and a prefill workgroup runs
+  // beside it.  bf16 cache: the split-KV kernels stream through 128 KiB of LDS per CU, which
+  // leaves no room for a prefill workgroup on the same CU, so the two classes share the device
+  // by CUs: the even split of the split-KV rows is launched first with one workgroup for every
+  // second CU (half the CUs move 5.4 TB/s of the 6.2 TB/s that all of them do), the prefill
+  // workgroups fill the other CUs, and take over the rest as the split-KV workgroups end.
+  // Config 3: 272 us, against 309 us one class after the other and 342 us side by side on
+  // every CU.  EID_MIXED_DECODE_WGS sets the number of split-KV workgroups for measurements.
+  static const bool share_env = [] {
+    const char *m = getenv("EID_MIXED");
+    return m && !strcmp(m, "share");
+  }();
+  const bool share = hs && (fp8 || share_env);
+  static const int split_cus = [] {
+    const char *m = getenv("EID_MIXED_DECODE_WGS");
+    return m ? atoi(m) : 0;
+  }();
+  const bool prefill_first = false;
+  p.share_cus = share ? 1 : 0;
+  p.mixed_wgs = (hs && !share) ? (split_cus > 0 ? split_cus : std::max(1, eid::device_cus() / 2)) : 0;
   p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
   HelperJoin joiner;
   if (hs) {
@@ -955,6 +976,25 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     joiner.hs = hs;
     joiner.st = st;
     joiner.forked = true;
+  }
+  // With the host's copies of the lengths the prefill launch gets its query tiles listed,
+  // heaviest first (not under capture: a captured launch serves whatever lengths a replay finds)
+  eid::PfTable pf_tab;
+  pf_tab.n = 0;
+  auto list_tiles = [&](const eid::AttnParams &q) {
+    if (args->seq_lens_host && args->cu_seqlens_q_host && !capturing)
+      eid::build_prefill_table(q, args->seq_lens_host, args->cu_seqlens_q_host, &pf_tab);
+  };
+  auto prefill_on_helper = [&]() {
+    eid::AttnParams pp = p;
+    pp.qlen_lo = qmax + 1;
+    pp.qlen_hi = 0x7fffffff;
+    list_tiles(pp);
+    return eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream, &pf_tab);
+  };
+  if (prefill_first) {
+    e = prefill_on_helper();
+    if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
   }
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
@@ -967,20 +1007,8 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
       if (e != hipSuccess) return hip_fail(e, "split-KV launch");
     }
   }
-  // With the host's copies of the lengths the prefill launch gets its query tiles listed,
-  // heaviest first (not under capture: a captured launch serves whatever lengths a replay finds)
-  eid::PfTable pf_tab;
-  pf_tab.n = 0;
-  auto list_tiles = [&](const eid::AttnParams &q) {
-    if (args->seq_lens_host && args->cu_seqlens_q_host && !capturing)
-      eid::build_prefill_table(q, args->seq_lens_host, args->cu_seqlens_q_host, &pf_tab);
-  };
-  if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
-    eid::AttnParams pp = p;
-    pp.qlen_lo = qmax + 1;
-    pp.qlen_hi = 0x7fffffff;
-    list_tiles(pp);
-    e = eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream, &pf_tab);
+  if (hs && !prefill_first) {  // the prefill rows, enqueued right behind the first split-KV launch
+    e = prefill_on_helper();
     if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
   }
   if (args->split_done_event) {

@@ -47,6 +47,7 @@ struct AttnParams {
   int32_t *seq_parts;    // [num_seqs] pieces per sequence, written by an even split for its merge
                          // (the pieces have no common size)
   int32_t even_wgs;      // workgroups of an even split (its grid)
+  int32_t mixed_wgs;     // host-side: cap on even_wgs for the split-KV rows of a mixed batch, 0 = none
   int32_t store_every_partition;  // even split with the caller's partition: a partial per partition
                          // instead of one per piece (measurement aid, EID_STORE_EVERY_PARTITION)
   float *ws_ml;          // [num_seqs*ws_rows][nparts_max][Hq][2]  (m natural-log units, l)
