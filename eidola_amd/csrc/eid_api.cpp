@@ -964,7 +964,6 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     const char *m = getenv("EID_MIXED_DECODE_WGS");
     return m ? atoi(m) : 0;
   }();
-  const bool prefill_first = false;
   p.share_cus = share ? 1 : 0;
   p.mixed_wgs = (hs && !share) ? (split_cus > 0 ? split_cus : std::max(1, eid::device_cus() / 2)) : 0;
   p.fp8_pair = fp8_pair_applies(desc) ? 1 : 0;
@@ -992,10 +991,6 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
     list_tiles(pp);
     return eid::launch_prefill(pp, desc->num_q_tokens, fp8, hs->stream, &pf_tab);
   };
-  if (prefill_first) {
-    e = prefill_on_helper();
-    if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
-  }
   // q_len 1..2: one 16-row tile per KV head; each split-KV launch is followed by the merge
   // of its own class of sequences (they share the partition plan)
   ClassPlan cp1;
@@ -1007,7 +1002,7 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, vo
       if (e != hipSuccess) return hip_fail(e, "split-KV launch");
     }
   }
-  if (hs && !prefill_first) {  // the prefill rows, enqueued right behind the first split-KV launch
+  if (hs) {  // the prefill rows, enqueued right behind the first split-KV launch
     e = prefill_on_helper();
     if (e != hipSuccess) return hip_fail(e, "prefill launch on the helper stream");
   }

@@ -68,6 +68,7 @@ class _Request:
     def __init__(self, seq_id, prompt_ids, max_new_tokens):
         self.seq_id, self.prompt, self.budget = seq_id, prompt_ids, max_new_tokens
         self.blocks = (len(prompt_ids) + max_new_tokens + 15) // 16   # pages it may come to hold
+        # (generate() has cut prompt and budget to the context: at most max_blocks_per_seq)
         self.fed = 0              # prompt tokens already in the KV cache
         self.last = None          # the sampled token to feed next
         self.produced = 0
@@ -87,19 +88,30 @@ class SyntheticAttentionEngine:
     name = "synthetic"
 
     def __init__(self, layers=4, ctx=4096, seed=0, num_blocks=None, max_seqs=16, chunk=512,
-                 step_tokens=2048):
+                 step_tokens=2048, device="cuda:0"):
+        """`device=None` builds the host side only (scheduler, queues, the batching loop) and
+        leaves `forward` to the caller: the loop can then be tested without a GPU."""
         import numpy as np
         import torch
         import eidola_amd as ea
         self.np, self.torch, self.ea = np, torch, ea
         ea.load_library()
-        dev = "cuda:0"
+        dev = device
         self.dev, self.layers, self.ctx = dev, layers, ctx
         self.max_seqs, self.chunk, self.step_tokens = max_seqs, chunk, step_tokens
         self.H, self.NQKV = 2880, (64 + 2 * 8) * 64
         self.geoms = [ea.AttnGeometry(window=128 if l % 2 == 0 else 0) for l in range(layers)]
         self.max_blocks = (ctx + 15) // 16
         self.num_blocks = num_blocks or (max_seqs + 1) * self.max_blocks
+        self.sched = ea.Scheduler(self.num_blocks, self.max_blocks)
+        self.cv = threading.Condition()
+        self.waiting, self.active = [], []
+        self.committed = 0        # pages the active requests may come to hold between them
+        self.next_id = 1
+        self.steps = self.mixed_steps = self.max_step_seqs = 0   # (for tests and curiosity)
+        self.worker = None
+        if dev is None:
+            return
         g = torch.Generator(device=dev).manual_seed(seed)
         rnd = lambda *shape, scale: (torch.randn(shape, device=dev, generator=g) * scale).to(torch.bfloat16)
         self.emb = rnd(VOCAB, self.H, scale=1.0)
@@ -110,13 +122,6 @@ class SyntheticAttentionEngine:
                    for _ in range(layers)]
         self.vc = [torch.zeros_like(k) for k in self.kc]
         self.cos_sin = torch.from_numpy(ea.yarn_cos_sin(ctx + 1)).to(dev)
-        self.sched = ea.Scheduler(self.num_blocks, self.max_blocks)
-        self.cv = threading.Condition()
-        self.waiting, self.active = [], []
-        self.committed = 0        # pages the active requests may come to hold between them
-        self.next_id = 1
-        self.steps = self.mixed_steps = self.max_step_seqs = 0   # (for tests and curiosity)
-        self.worker = None
 
     def _norm(self, h):
         x = h.float()
@@ -205,6 +210,12 @@ class SyntheticAttentionEngine:
                     self.sched.add_seq(r.seq_id)
                     self.committed += r.blocks
                     self.active.append(r)
+                if not self.active:
+                    # nothing runs and the head of the queue cannot be admitted (generate()
+                    # refuses requests the pool could never hold, so this is a guard): wait
+                    # for the queue to change instead of stepping an empty batch
+                    self.cv.wait(timeout=0.05)
+                    continue
             try:
                 self._step()
             except Exception as e:        # a failed step fails the requests in it, not the process
@@ -214,7 +225,16 @@ class SyntheticAttentionEngine:
     def generate(self, prompt_ids, max_new_tokens):
         """Greedy decoding through the shared batching loop.  Yields byte tokens, EOS on a
         genuine stop (see FakeEngine.generate)."""
-        prompt_ids = list(prompt_ids)[-(self.ctx - max(1, max_new_tokens)):] or [EOS]
+        # The reference asks for min(context_length, 4096) new tokens, i.e. often the whole
+        # context (/root/reference/crates/eidola-app-core/src/lib.rs:5595): the budget is cut to
+        # what the context can hold behind at least one prompt token, and the prompt keeps its
+        # tail (the latest turns) within what is left.
+        max_new_tokens = max(1, min(int(max_new_tokens), self.ctx - 1))
+        keep = self.ctx - max_new_tokens
+        prompt_ids = list(prompt_ids)[-keep:] or [EOS]
+        blocks = min((len(prompt_ids) + max_new_tokens + 15) // 16, self.max_blocks)
+        if blocks > self.num_blocks:   # could never be admitted: refuse it, do not queue it
+            raise RuntimeError(f"request needs {blocks} KV pages, the pool has {self.num_blocks}")
         with self.cv:
             if self.worker is None:
                 self.worker = threading.Thread(target=self._run, name="eidola-engine-steps", daemon=True)
@@ -269,6 +289,11 @@ class Handler(BaseHTTPRequestHandler):
             messages = req["messages"]
             if not isinstance(messages, list) or not messages:
                 raise ValueError("messages must be a non-empty list")
+            # `tools` (eidola-common/src/lib.rs:129-131) is accepted and not acted upon: the
+            # synthetic model cannot call tools, and an engine that ignores the list answers in
+            # plain text, which the reference handles.  A malformed list is still a bad request.
+            if "tools" in req and not isinstance(req["tools"], list):
+                raise ValueError("tools must be a list")
             max_new = int(req.get("max_completion_tokens", req.get("max_tokens", 256)))
             if max_new < 1:
                 raise ValueError("max_completion_tokens must be positive")

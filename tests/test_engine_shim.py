@@ -167,3 +167,89 @@ def test_started_and_polled_the_way_the_reference_does():
     finally:
         child.terminate()
         child.wait(timeout=10)
+
+
+# ---- the batching loop on the host: the real scheduler, a stubbed forward (no GPU) ----------
+def stub_engine(ctx=64, num_blocks=None, max_seqs=4, answer=ord("a")):
+    """SyntheticAttentionEngine without its device side: forward() votes for one byte."""
+    import torch
+    eng = shim.SyntheticAttentionEngine(layers=1, ctx=ctx, num_blocks=num_blocks, max_seqs=max_seqs,
+                                        chunk=16, step_tokens=32, device=None)
+    eng.forward_calls = []
+
+    def forward(seq_ids, token_lists):
+        q_lens = [len(t) for t in token_lists]
+        eng.sched.build_batch(seq_ids, q_lens)     # raises on a request the pool cannot hold
+        eng.forward_calls.append((list(seq_ids), q_lens))
+        logits = torch.zeros((len(seq_ids), shim.VOCAB))
+        logits[:, answer] = 1.0
+        return logits
+    eng.forward = forward
+    return eng
+
+
+@pytest.mark.parametrize("max_new", [64, 65, 4096])   # == ctx, > ctx, the reference's usual 4096
+def test_a_budget_of_the_whole_context_keeps_the_tail_of_a_long_prompt(max_new):
+    """The reference sends max_completion_tokens = min(context_length, 4096)
+    (/root/reference/crates/eidola-app-core/src/lib.rs:5595), which is the engine's -c: the
+    budget shrinks to the context, the prompt to its tail, and nothing outgrows its table row."""
+    eng = stub_engine(ctx=64)
+    prompt = list(range(1, 200))                      # longer than the context
+    out = list(eng.generate(prompt, max_new))
+    assert out == [ord("a")] * 63                     # ctx - 1 new tokens behind one prompt token
+    fed = sum(q for _, qs in eng.forward_calls for q in qs)
+    assert fed == 1 + 62                              # one prompt token, then 62 decode rows (the last token is not fed back)
+    assert eng.sched.free_blocks == eng.num_blocks and eng.committed == 0
+
+
+def test_a_long_prompt_with_a_small_budget_keeps_its_latest_tokens():
+    eng = stub_engine(ctx=64)
+    seen = []
+    real = eng.forward
+
+    def forward(seq_ids, token_lists):
+        seen.extend(t for ts in token_lists for t in ts if len(ts) > 1 or not seen)
+        return real(seq_ids, token_lists)
+    eng.forward = forward
+    prompt = list(range(1, 200))
+    assert list(eng.generate(prompt, 4)) == [ord("a")] * 4
+    assert seen[:60] == prompt[-60:]                  # ctx - 4 prompt tokens: the tail
+
+
+def test_a_request_the_pool_can_never_hold_is_refused_and_the_engine_goes_on():
+    """A request needing more pages than the pool has used to sit at the head of the queue
+    for ever, with the stepping thread spinning on an empty batch behind it."""
+    eng = stub_engine(ctx=256, num_blocks=4, max_seqs=2)   # 4 pages = 64 tokens in all
+    with pytest.raises(RuntimeError, match="KV pages"):
+        list(eng.generate(list(range(1, 100)), 100))
+    assert not eng.waiting and not eng.active
+    assert list(eng.generate([1, 2, 3], 5)) == [ord("a")] * 5   # the next request is served
+    assert eng.sched.free_blocks == 4
+
+
+def test_concurrent_requests_wait_for_pages_and_all_finish():
+    eng = stub_engine(ctx=64, num_blocks=6, max_seqs=4)   # two requests of 3 pages fit at a time
+    results = {}
+
+    def run(i):
+        results[i] = list(eng.generate(list(range(1, 30)), 10))
+    threads = [threading.Thread(target=run, args=(i,)) for i in range(5)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=30)
+    assert all(results.get(i) == [ord("a")] * 10 for i in range(5))
+    assert eng.max_step_seqs <= 2 and eng.sched.free_blocks == 6 and eng.committed == 0
+
+
+def test_tools_in_the_request_are_accepted_and_ignored(server):
+    """`tools` is part of the reference's request body
+    (/root/reference/crates/eidola-common/src/lib.rs:129-131); this engine answers in plain text."""
+    body = reference_body("m", [{"role": "user", "content": "abc"}], 16)
+    body["tools"] = [{"type": "function", "function": {"name": "f", "parameters": {"type": "object"}}}]
+    resp = post(server, body)
+    assert resp["choices"][0]["message"]["content"] == "cba"
+    body["tools"] = "not a list"
+    with pytest.raises(urllib.error.HTTPError) as ei:
+        post(server, body)
+    assert ei.value.code == 400 and "tools" in json.loads(ei.value.read())["error"]["message"]

@@ -38,8 +38,8 @@ def test_decode_steps_agree_with_one_prefill_pass(engine):
     a, b = logits.double().cpu().numpy(), ref.double().cpu().numpy()
     assert np.isfinite(a).all() and np.isfinite(b).all()
     cos = float(a @ b / (np.linalg.norm(a) * np.linalg.norm(b)))
-    assert cos > 0.9995, cos
-    assert np.abs(a - b).max() < 0.05 * np.abs(b).std() + 0.5, (np.abs(a - b).max(), b.std())
+    assert cos > 0.99998, cos   # (observed 0.999996: a wrong window on one layer of three gives ~0.999)
+    assert np.abs(a - b).max() < 0.03 * np.abs(b).std(), (np.abs(a - b).max(), b.std())   # (observed 0.009)
     assert int(a[:257].argmax()) == int(b[:257].argmax())
 
 
@@ -47,8 +47,8 @@ def _close(a, b):
     a, b = a.double().cpu().numpy(), b.double().cpu().numpy()
     assert np.isfinite(a).all() and np.isfinite(b).all()
     cos = float(a @ b / (np.linalg.norm(a) * np.linalg.norm(b)))
-    assert cos > 0.9995, cos
-    assert np.abs(a - b).max() < 0.05 * np.abs(b).std() + 0.5, (np.abs(a - b).max(), b.std())
+    assert cos > 0.99998, cos   # (observed 0.999996: a wrong window on one layer of three gives ~0.999)
+    assert np.abs(a - b).max() < 0.03 * np.abs(b).std(), (np.abs(a - b).max(), b.std())   # (observed 0.009)
 
 
 def test_sequences_that_share_a_step_do_not_see_each_other(engine):
@@ -140,3 +140,89 @@ def test_http_round_trip_on_the_gpu_engine(engine):
     finally:
         srv.shutdown()
         srv.server_close()
+
+
+# ---- forward() against the same chain built from the CPU oracle's functions --------------------
+def _bits(t):
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def _oracle_forward(eng, mirror, batch, token_lists, full_attention_everywhere=False):
+    """SyntheticAttentionEngine.forward restated on the host: embedding rows, and per layer
+    the norm (fp32, as the engine computes it), orc_o_proj for the QKV projection,
+    orc_rope_kv_write into a CPU mirror of the layer's pages, orc_attn_f64 over that mirror with
+    the batch arrays the engine's scheduler produced, orc_o_proj with the residual.  Returns
+    fp64 logits of every sequence's last row."""
+    import oracle
+    import eidola_amd as ea
+    from eidola_amd import synth
+    f32 = lambda bits: synth.bf16_bits_to_f32(bits).astype(np.float32)
+    to_bits = lambda x: synth.f32_to_bf16_bits(np.ascontiguousarray(x, dtype=np.float32))
+
+    def norm(bits):
+        x = f32(bits)
+        return to_bits(x * (1.0 / np.sqrt((x * x).mean(-1, keepdims=True, dtype=np.float32) + np.float32(1e-6))))
+    toks = [t for ts in token_lists for t in ts]
+    hidden = mirror["emb"][toks].copy()
+    S, T = len(token_lists), len(toks)
+    desc1 = ea.make_desc(eng.geoms[1], num_seqs=1, num_q_tokens=1, max_q_len=1, max_kv_len=1,
+                         max_blocks_per_seq=1, num_blocks=eng.num_blocks)
+    for l in range(eng.layers):
+        g = ea.AttnGeometry() if full_attention_everywhere else eng.geoms[l]
+        qkv, _ = oracle.o_proj(norm(hidden), mirror["wqkv"][l])
+        q = oracle.rope_kv_write(desc1, qkv, batch.positions, mirror["table"], mirror["kc"][l], mirror["vc"][l],
+                                 batch.slot_mapping)
+        desc = ea.make_desc(g, num_seqs=S, num_q_tokens=T, max_q_len=batch.max_q_len, max_kv_len=batch.max_kv_len,
+                            max_blocks_per_seq=batch.block_table.shape[1], num_blocks=eng.num_blocks)
+        o, _ = oracle.attn_f64(desc, q, mirror["kc"][l], mirror["vc"][l], batch.block_table, batch.seq_lens,
+                               batch.cu_seqlens_q, mirror["sinks"][l])
+        hidden, _ = oracle.o_proj(to_bits(o).reshape(T, 4096), mirror["wo"][l], None, hidden)
+    last = batch.cu_seqlens_q[1:].astype(np.int64) - 1
+    return f32(norm(hidden[last])).astype(np.float64) @ f32(mirror["emb"]).astype(np.float64).T
+
+
+def test_forward_against_the_oracle_chain():
+    """One prefill chunk of more than 64 rows beside a shorter one, then decode steps, through
+    two layers (layer 0 with the 128-token window, layer 1 with full attention): the engine's
+    logits against the chain of oracle functions fed with the scheduler's own batch arrays.
+    A control run of the oracle chain with the window switched off must NOT pass, so a wrong
+    window (or wrong positions, slots, cu_seqlens) would not either."""
+    from eidola_amd import synth
+    eng = shim.SyntheticAttentionEngine(layers=2, ctx=1024, seed=11, max_seqs=4)
+    mirror = {"emb": _bits(eng.emb), "wqkv": [_bits(w) for w in eng.wqkv], "wo": [_bits(w) for w in eng.wo],
+              "sinks": [s.cpu().numpy() for s in eng.sinks], "table": eng.cos_sin.cpu().numpy(),
+              "kc": [np.zeros((eng.num_blocks, 16, 8, 64), np.uint16) for _ in range(eng.layers)],
+              "vc": [np.zeros((eng.num_blocks, 16, 8, 64), np.uint16) for _ in range(eng.layers)]}
+    control = {k: ([a.copy() for a in v] if k in ("kc", "vc") else v) for k, v in mirror.items()}
+    batches = []
+    real_build = eng.sched.build_batch
+
+    def recording_build(seq_ids, q_lens):
+        b = real_build(seq_ids, q_lens)
+        batches.append(b)
+        return b
+    eng.sched.build_batch = recording_build
+    rng = np.random.default_rng(21)
+    prompts = [[int(x) for x in rng.integers(0, 256, size=n)] for n in (230, 40)]
+    eng.sched.add_seq(1)
+    eng.sched.add_seq(2)
+    steps = [([1, 2], prompts)] + [([1, 2], [[int(rng.integers(0, 256))], [int(rng.integers(0, 256))]]) for _ in range(3)]
+    worst, worst_control = 0.0, 0.0
+    for ids, toks in steps:
+        got = eng.forward(ids, toks).double().cpu().numpy()
+        b = batches[-1]
+        ref = _oracle_forward(eng, mirror, b, toks)
+        bad = _oracle_forward(eng, control, b, toks, full_attention_everywhere=True)
+        assert np.isfinite(got).all()
+        scale = ref.std()
+        err, err_control = np.abs(got - ref).max() / scale, np.abs(got - bad).max() / scale
+        worst, worst_control = max(worst, err), max(worst_control, err_control)
+        # six bf16 roundings per layer between the two chains, which feed on their own intermediates
+        assert err <= 0.03, (err, scale)
+        assert (got[:, :257].argmax(-1) == ref[:, :257].argmax(-1)).all()
+    assert worst_control > 3 * max(worst, 0.01), (worst, worst_control)   # the check can tell a wrong window
+    # the pages the engine wrote are the pages the oracle chain wrote (K after rotation: within a bf16 step)
+    for l in range(eng.layers):
+        kd = synth.bf16_bits_to_f32(_bits(eng.kc[l])).astype(np.float64)
+        assert np.abs(kd - synth.bf16_bits_to_f32(mirror["kc"][l])).max() <= 0.15
+        assert np.array_equal(_bits(eng.vc[l]) != 0, mirror["vc"][l] != 0)
