@@ -974,8 +974,12 @@ __device__ __forceinline__ void finish(const AttnParams &p, const int s, const i
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) {
         typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
-        const f16x2 h0 = {(_Float16)(acc[nt][mt][0] * inv_l), (_Float16)(acc[nt][mt][1] * inv_l)};
-        const f16x2 h1 = {(_Float16)(acc[nt][mt][2] * inv_l), (_Float16)(acc[nt][mt][3] * inv_l)};
+        // (saturated to the fp16 range: a value entry beyond +-65504, which bf16 can hold, then
+        // gives a bounded error in a sequence of several pieces, not an inf that the merge turns
+        // into NaN)
+        auto h = [&](const float x) { return (_Float16)__builtin_fminf(__builtin_fmaxf(x * inv_l, -65504.f), 65504.f); };
+        const f16x2 h0 = {h(acc[nt][mt][0]), h(acc[nt][mt][1])};
+        const f16x2 h1 = {h(acc[nt][mt][2]), h(acc[nt][mt][3])};
         w[mt][0] = __builtin_bit_cast(uint32_t, h0);
         w[mt][1] = __builtin_bit_cast(uint32_t, h1);
       }

@@ -93,8 +93,15 @@ typedef struct eid_attn_desc {
   int32_t window;             /* 0 = full causal; W>0: row at position p sees p-W+1..p   */
   int32_t kv_dtype;           /* eid_kv_dtype                                            */
   int32_t partition_size;     /* split-KV partition in tokens: a multiple of 64 in
-                                 [64, 4096], or 0 = the kernels size it from the batch at
-                                 run time (>= 256) so the work fills the device evenly   */
+                                 [64, 4096], or 0 = the library cuts the batch itself, into
+                                 equal ranges of 64-key chunks (>= 256 keys each).  A non-zero
+                                 value is the grid on which a sequence may be cut.  Long
+                                 launches are cut into equal contiguous ranges of partitions,
+                                 one per workgroup; a workgroup that holds several consecutive
+                                 partitions of a sequence merges them in registers and stores
+                                 one partial for the whole piece (stores trickling into the
+                                 stream of loads are dear on this machine).  Results do not
+                                 depend on it beyond fp32 round-off.                      */
   int64_t sum_kv_len;         /* optional launch-sizing hint: any value >= the sum of
                                  seq_lens[s] over the batch, or 0 = not known.  An engine's
                                  scheduler holds seq_lens on the host, so the sum is free;
@@ -231,12 +238,18 @@ int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args,
  * alone (the split-KV kernel writes their output itself).  With desc->partition_size == 0
  * the partition is the one the last eid_attn_decode / eid_attn_varlen call on this
  * workspace recorded in its header, so such a call must have preceded.
- * Workspace layout, with R = min(max_q_len, 6) (min(max_q_len, 8), 16 or 32 under the conditions above) and N = partitions per sequence (max):
+ * Workspace layout, with R = min(max_q_len, 6) (min(max_q_len, 8), 16 or 32 under the conditions above) and N = partitions per sequence (max; one more
+ * with partition_size == 0, whose ranges are cut anywhere in a sequence):
  *   256 bytes                         launch plan (written by the library)
+ *   int32 parts [num_seqs]            (only when N > 1, padded to 256 bytes) pieces per sequence
+ *                                     as the last even split left them
  *   float ml [num_seqs*R][N][Hq][2]   m (natural-log units, -inf if empty) and
  *                                     l = sum of e^(s-m) over the partition's keys
- *   half  o  [num_seqs*R][N][Hq][64]  the partition's own output sum e^(s-m) v / l (fp16),
- *                                     at the next 256-byte boundary
+ *   half  o  [num_seqs*R][N][Hq][64]  the partition's own output sum e^(s-m) v / l (fp16,
+ *                                     saturated at +-65504), at the next 256-byte boundary
+ * Range of values: a partial output is a convex combination of value rows (times v_scale), so
+ * sequences of several partitions are exact to fp16 while |v| <= 65504; larger entries (bf16
+ * can hold them) saturate there, in those sequences only.
  * (heads innermost: the 64 heads of one (row, partition) cell form one contiguous block,
  * which a split-KV workgroup writes with full-width stores)
  * Behind these, when the batch holds prefill chunks whose query tiles cannot fill the device

@@ -14,6 +14,8 @@ import eidola_amd as ea
 from eidola_amd import KV_BF16, KV_FP8_E4M3, synth
 from eidola_amd.ops import workspace_layout
 
+MAX_ABS_TOL_REL, MEAN_ABS_TOL_REL = 2e-2, 2e-3   # the attention tolerances per unit of value magnitude
+
 from helpers import (make_batch, desc_of, logical_tensors, cpu_caches, oracle_out, fp8_scales,
                      all_slots, empty_caches, assert_close)
 
@@ -994,7 +996,8 @@ def test_config4_fp8_full_size(G):
     torch.cuda.synchronize()
     assert torch.equal(oh, out)
     order = np.argsort(b.seq_lens)
-    seqs = [int(order[0]), int(order[128]), int(order[-1]), 0, 1]
+    seqs = sorted({int(order[i]) for i in (0, 1, 25, 64, 128, 192, 230, 254, 255)} | {0, 1, 2})
+    assert len(seqs) >= 10
     _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, seqs, "config4",
                   ks.cpu().numpy(), vs.cpu().numpy())
 
@@ -1014,9 +1017,13 @@ def test_config5_verify_full_size(G, layer):
                         sinks=G.dev(sinks), sum_kv_len=int(b.seq_lens.sum()))
     torch.cuda.synchronize()
     assert torch.equal(oh, out)
+    # eight sequences: the shortest, the longest, the one nearest to 128 whole partitions of 512
+    # keys (the most pieces a row can have), and five spread over the lengths
     order = np.argsort(b.seq_lens)
-    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, [int(order[0]), int(order[64]), int(order[-1])],
-                  f"config5 layer {layer}")
+    most_parts = int(np.argmax((b.seq_lens + 511) // 512 * 100000 - b.seq_lens % 512))
+    seqs = sorted({int(order[i]) for i in (0, 16, 40, 64, 90, 112, 127)} | {most_parts})
+    assert len(seqs) >= 7 and (b.seq_lens[most_parts] + 511) // 512 == ((b.seq_lens + 511) // 512).max()
+    _sample_check(G, b, q_d, kc_d, vc_d, sinks, out, seqs, f"config5 layer {layer}")
 
 
 def test_step_replayed_from_a_hip_graph(G):
@@ -1166,3 +1173,59 @@ def test_prefill_key_range_split(G, kv_dtype, window):
         assert np.allclose(lse, ref_lse, atol=2e-3)
         assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs), ref,
                      f"split prefill {seq_lens} w={window}, no lse")
+
+
+def test_large_values_across_several_partitions(G):
+    """Split-KV partials carry a partition's normalised output in fp16.  Values of a few
+    ten thousand are exact to fp16 relative precision; beyond 65,504 (which bf16 holds) a
+    sequence cut into several pieces saturates instead of going to inf / NaN, and a sequence
+    that stays in one piece is not affected at all."""
+    seq_lens, q_lens = [3000, 1500, 200], [1, 1, 1]
+    for scale, exact in ((3.0e4, True), (1.0e5, False)):
+        b = make_batch(seq_lens, q_lens, partition=256)
+        q, k, v, sinks = logical_tensors(b, seed=31)
+        # values uniform in [-scale, scale], exactly representable pattern: bf16 of N(0,1) * scale / 4
+        vf = np.clip(synth.bf16_bits_to_f32(v) * (scale / 4), -scale, scale).astype(np.float32)
+        v = synth.f32_to_bf16_bits(vf)
+        kc, vc = cpu_caches(b, k, v)
+        kc_d, vc_d = G.gpu_caches(b, k, v)
+        ref, _ = oracle_out(b, q, kc, vc, sinks)
+        got = synth.bf16_bits_to_f32(G.run_attn(b, q, kc_d, vc_d, sinks)).astype(np.float64)
+        assert np.isfinite(got).all()
+        err = np.abs(got - ref)
+        rows = b.cu_seqlens_q
+        if exact:   # the usual tolerance, relative to the magnitude of the values
+            assert err.max() <= MAX_ABS_TOL_REL * scale and err.mean() <= MEAN_ABS_TOL_REL * scale
+        else:       # bounded, never NaN; the single-piece sequence (200 keys) is exact
+            assert err.max() <= scale
+            one = slice(rows[2], rows[3])
+            assert err[one].max() <= MAX_ABS_TOL_REL * scale
+
+
+def test_a_partial_per_partition_when_asked_for():
+    """EID_STORE_EVERY_PARTITION=1 (a measurement aid read once per process) makes an even
+    split store every partition of the caller's size and leaves all merging to the merge
+    kernel; checked in a process of its own against the oracle, on a verify batch large enough
+    for the even split."""
+    import os
+    import subprocess
+    import sys
+    code = r'''
+import numpy as np, torch, sys, os
+sys.path.insert(0, os.path.join(os.getcwd(), "tests"))
+import gpu_helpers as G
+from helpers import make_batch, logical_tensors, cpu_caches, oracle_out, assert_close
+rng = np.random.default_rng(5)
+seq_lens = rng.integers(1500, 9000, size=40)
+b = make_batch(seq_lens, [5] * 40, partition=128)
+q, k, v, sinks = logical_tensors(b)
+kc, vc = cpu_caches(b, k, v)
+kc_d, vc_d = G.gpu_caches(b, k, v)
+ref, _ = oracle_out(b, q, kc, vc, sinks)
+for host in (False, True):
+    print(assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=host, hint=host), ref, "every partition"))
+'''
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, EID_STORE_EVERY_PARTITION="1")
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout + r.stderr
