@@ -80,6 +80,33 @@ def split_kernel_ms(w, steps, torch):
     return sum(a.elapsed_time(b) for a, b in pairs) / steps
 
 
+def kernel_dispatch_ms(calls, steps, torch, n_sets):
+    """Average milliseconds of the (last) split-KV / prefill kernel of each call in `calls`
+    (PreparedCalls, rotated), from HIP events that the MEASUREMENT build of the library attaches
+    to the kernel's own dispatch; None if the calls launch no such kernel."""
+    from eidola_amd import _lib
+    lib = _lib.load_measure_library()
+    bound = [c.bound_to(lib) for c in calls]
+    for i in range(2 * n_sets):
+        bound[i % n_sets]()
+    pairs = []
+    for _ in range(steps):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        b.record()
+        pairs.append((a, b))
+    torch.cuda.synchronize()
+    try:
+        for i, (a, b) in enumerate(pairs):
+            lib.eid_debug_set_kernel_events(a.cuda_event, b.cuda_event)
+            bound[i % n_sets]()
+    finally:
+        lib.eid_debug_set_kernel_events(None, None)
+    torch.cuda.synchronize()
+    ms = [a.elapsed_time(b) for a, b in pairs]
+    return None if min(ms) < 1e-3 else sum(ms) / steps
+
+
 def split_kernel_dispatch_ms(w, steps, torch, ea):
     """Average milliseconds of the split-KV KERNEL inside full steps: a pair of HIP events per step
     that the MEASUREMENT build of the library (libeidola_attn_measure.so: the same sources with
@@ -349,15 +376,22 @@ def other_configs(a, torch, ea, synth, pool2, check):
     steps, warm = max(10, a.steps // 8), max(3, a.warmup // 4)
     out = {}
 
-    def hbm(work, ms, kernel, extra=None):
+    def hbm(work, ms, kernel, extra=None, kernel_ms=None):
+        """`frac` is quoted on the whole CALL (every launch of it, merge included); frac_kernel on
+        the dominant kernel alone (events on its own dispatch, measurement build)."""
         gbs = work["bytes"] / ms / 1e6
-        r = {"ms_call": ms, "alg_bytes": work["bytes"], "q_tokens": work["q_tokens"],
+        r = {"ms_call": ms, "call_us": ms * 1e3, "kernel_us": kernel_ms * 1e3 if kernel_ms else None,
+             "alg_bytes": work["bytes"], "q_tokens": work["q_tokens"],
              "roofline": {"bound": "hbm", "kernel": kernel, "achieved": gbs, "peak": HBM_PEAK_GBS,
-                          "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
-                          "how": "HIP events around back-to-back eid_attn_* calls (every launch of the "
-                                 "call), page sets rotated"}}
+                          "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "frac_uses": "call_us",
+                          "frac_kernel": (work["bytes"] / kernel_ms / 1e6 / HBM_PEAK_GBS) if kernel_ms else None,
+                          "how": "call_us: HIP events around back-to-back eid_attn_* calls (every launch of the "
+                                 "call), page sets rotated; kernel_us: events attached to the dominant "
+                                 "kernel's dispatch by the measurement build of the library"}}
         r.update(extra or {})
         return r
+
+    kdur = lambda w_, n: kernel_dispatch_ms(w_.attn, n, torch, w_.n)
 
     # ---- 2b: decode, 128-token window (latency-bound: 17 MB of KV) ----
     w = Workload(lambda off: synth.config2(window=128, perm_offset=off), a.sets, 7, torch, ea, synth,
@@ -365,7 +399,7 @@ def other_configs(a, torch, ea, synth, pool2, check):
     ms_step, ms_attn = compact_pass(w, steps * 2, warm, torch)
     out["2b_window"] = hbm(synth.algorithmic_work(w.batches[0]), ms_attn, "shortspan_kernel<1,bf16>",
                            {"ms_per_step": ms_step, "tokens_per_s": 64 / ms_step * 1e3,
-                            "note": "latency-bound: 17 MB of KV per call"})
+                            "note": "latency-bound: 17 MB of KV per call; one launch (kernel = call)"})
     if check:
         order = np.argsort(w.batches[0].seq_lens)
         out["2b_window"]["parity"] = parity_sample(w, [order[0], order[31], order[-1], 0, 1], torch, synth, "2b_window")
@@ -375,36 +409,48 @@ def other_configs(a, torch, ea, synth, pool2, check):
     ms_step, ms_attn = compact_pass(w3, steps, warm, torch)
     b3 = w3.batches[0]
     lw, sw = synth.algorithmic_work(b3, rows="long"), synth.algorithmic_work(b3, rows="short")
-    out["3_mixed"] = {"ms_call": ms_attn, "ms_per_step": ms_step, "q_tokens": b3.num_q_tokens,
+    out["3_mixed"] = {"ms_call": ms_attn, "call_us": ms_attn * 1e3, "kernel_us": None,
+                      "ms_per_step": ms_step, "q_tokens": b3.num_q_tokens,
                       "tokens_per_s": b3.num_q_tokens / ms_step * 1e3,
                       "prefill_TFLOPs_of_the_call": lw["flops"] / ms_attn / 1e9,
                       "decode_GBps_of_the_call": sw["bytes"] / ms_attn / 1e6,
-                      "note": "prefill and split-KV launches run side by side (two streams)"}
+                      "note": "two streams: the split-KV rows take every second CU, the prefill "
+                              "workgroups the others and then the rest"}
     if check:
         lens8 = np.argsort(b3.seq_lens[:8])
         out["3_mixed"]["parity"] = parity_sample(w3, [lens8[0], lens8[-1], 8, 9, 60, 127], torch, synth, "3_mixed")
     wp = Workload(lambda off: subset(full(off), np.arange(8), "config3_prefill_rows", synth), 4, 8,
                   torch, ea, synth, "varlen", pool=pool2)
     _, ms_p = compact_pass(wp, steps, warm, torch)
+    ms_pk = kdur(wp, steps)
     tf = lw["flops"] / ms_p / 1e9
-    out["3_prefill"] = {"ms_call": ms_p, "alg_flops": lw["flops"], "q_tokens": lw["q_tokens"],
+    out["3_prefill"] = {"ms_call": ms_p, "call_us": ms_p * 1e3, "kernel_us": ms_pk * 1e3 if ms_pk else None,
+                        "alg_flops": lw["flops"], "q_tokens": lw["q_tokens"],
                         "roofline": {"bound": "mfma", "kernel": "prefill_kernel<bf16, folded softmax factor>",
                                      "achieved": tf, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                                     "frac": tf / MFMA_BF16_PEAK_TFLOPS,
-                                     "how": "HIP events around back-to-back eid_attn_varlen calls on the 8 "
-                                            "prefill sequences alone"}}
+                                     "frac": tf / MFMA_BF16_PEAK_TFLOPS, "frac_uses": "call_us",
+                                     "frac_kernel": (lw["flops"] / ms_pk / 1e9 / MFMA_BF16_PEAK_TFLOPS) if ms_pk else None,
+                                     "how": "call_us: HIP events around back-to-back eid_attn_varlen calls on "
+                                            "the 8 prefill sequences alone (one launch); kernel_us: events on "
+                                            "the kernel's dispatch (measurement build)"}}
+    if check:
+        out["3_prefill"]["parity"] = parity_sample(wp, [0, 3, 7], torch, synth, "3_prefill")
     wd = Workload(lambda off: subset(full(off), np.arange(8, 128), "config3_decode_rows", synth), 4, 8,
                   torch, ea, synth, "varlen", pool=pool2)
     _, ms_d = compact_pass(wd, steps, warm, torch)
-    out["3_decode"] = hbm(sw, ms_d, "splitkv_kernel<1,bf16,8 waves>")
+    out["3_decode"] = hbm(sw, ms_d, "splitkv_even_kernel<1,bf16,8 waves,direct-to-LDS loads>", kernel_ms=kdur(wd, steps))
+    if check:
+        order = np.argsort(wd.batches[0].seq_lens)
+        out["3_decode"]["parity"] = parity_sample(wd, [order[0], order[30], order[60], order[90], order[-1]], torch,
+                                                  synth, "3_decode")
     w = w3 = wp = wd = None
     # ---- 4: fp8 KV decode ----
     w4 = Workload(lambda off: synth.config4(num_blocks=300_000, perm_offset=off), 3, 9, torch, ea,
                   synth, "decode")
     ms_step, ms_attn = compact_pass(w4, steps, warm, torch)
     out["4_fp8"] = hbm(synth.algorithmic_work(w4.batches[0]), ms_attn,
-                       "splitkv_kernel<1,fp8,4 waves,head pairs>",
-                       {"ms_per_step": ms_step, "tokens_per_s": 256 / ms_step * 1e3})
+                       "splitkv_even_kernel<1,fp8,4 waves,head pairs>",
+                       {"ms_per_step": ms_step, "tokens_per_s": 256 / ms_step * 1e3}, kernel_ms=kdur(w4, steps))
     if check:
         order = np.argsort(w4.batches[0].seq_lens)
         out["4_fp8"]["parity"] = parity_sample(w4, [order[0], order[127], order[-1], 0, 1], torch, synth, "4_fp8")
@@ -418,9 +464,34 @@ def other_configs(a, torch, ea, synth, pool2, check):
         pool5 = w5.pool
         ms_step, ms_attn = compact_pass(w5, max(5, steps // 2), warm, torch)
         t5 += ms_step
+        n5 = max(5, steps // 2)
         out[key] = hbm(synth.algorithmic_work(w5.batches[0]), ms_attn,
-                       "splitkv_kernel<3,bf16,8 waves>" if layer == 0 else "splitkv_kernel<3,bf16,8 waves>, one item per sequence",
-                       {"ms_per_step": ms_step, "partition_size": 512})
+                       "splitkv_even_kernel<3,bf16,8 waves,direct-to-LDS loads>" if layer == 0
+                       else "splitkv_kernel<3,bf16,8 waves,direct-to-LDS loads>, one item per sequence",
+                       {"ms_per_step": ms_step, "partition_size": 512}, kernel_ms=kdur(w5, n5))
+        if layer == 0:
+            out[key]["partials"] = ("ranges cut on the 512-key grid, one workgroup per range; the consecutive "
+                                    "partitions a workgroup holds of one sequence are merged in registers and "
+                                    "stored as one partial; what crosses workgroups goes through the merge kernel")
+            # the same batch with every 512-key partition stored and merged by the merge kernel
+            # (a switch of the measurement build; the calls of this pass run through that build)
+            from eidola_amd import _lib
+            mlib = _lib.load_measure_library()
+            bound = [c.bound_to(mlib) for c in w5.attn]
+            mlib.eid_debug_set_store_every_partition(1)
+            try:
+                for i in range(2 * w5.n):
+                    bound[i % w5.n]()
+                ms_every = event_ms(lambda i: bound[i % w5.n](), n5, torch)
+                ms_every_k = kernel_dispatch_ms(w5.attn, n5, torch, w5.n)
+            finally:
+                mlib.eid_debug_set_store_every_partition(-1)
+            out["5_full_every_partition_stored"] = hbm(
+                synth.algorithmic_work(w5.batches[0]), ms_every,
+                "splitkv_even_kernel<3,bf16,8 waves,direct-to-LDS loads>, a partial per 512-key partition",
+                {"partition_size": 512,
+                 "partials": "every 512-key partition stored (346 MB of partials) and merged by the merge kernel"},
+                kernel_ms=ms_every_k)
         if check:
             order = np.argsort(w5.batches[0].seq_lens)
             out[key]["parity"] = parity_sample(w5, [order[0], order[64], order[-1]], torch, synth, key)
@@ -1027,14 +1098,21 @@ def cpu_baseline(w, torch, synth, threads):
     err = np.abs(synth.bf16_bits_to_f32(gpu).astype(np.float64)
                  - synth.bf16_bits_to_f32(out).astype(np.float64))
     work = synth.algorithmic_work(b)
-    model = ""
+    model, ident = "", {}
     try:
         for ln in open("/proc/cpuinfo"):
-            if ln.startswith("model name"):
+            key = ln.split(":", 1)[0].strip()
+            if key == "model name" and not model:
                 model = ln.split(":", 1)[1].strip()
+            if key in ("vendor_id", "cpu family", "model", "stepping") and key not in ident:
+                ident[key] = ln.split(":", 1)[1].strip()
+            if len(ident) == 4 and model:
                 break
     except OSError:
         pass
+    # (virtual machines often report a shortened model name: the family / model / stepping say which part it is)
+    model = f"{model} ({ident.get('vendor_id', '?')} family {ident.get('cpu family', '?')} model " \
+            f"{ident.get('model', '?')} stepping {ident.get('stepping', '?')})"
     return {"value": work["bytes"] / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
             "nproc": os.cpu_count(), "omp_num_threads_env": os.environ.get("OMP_NUM_THREADS"),
             "cpu_model": model,
@@ -1091,15 +1169,13 @@ def main():
                  a.sets, 7, torch, ea, synth, "decode")
     r = measure(w, a.steps, a.warmup, torch, synth, "config2_decode_full")
     split_ms = r["ms_split"]
-    kernel_ms = None if (a.no_hint or os.environ.get("EID_NO_ITEM_TABLE")) else \
-        split_kernel_dispatch_ms(w, a.steps, torch, ea)
+    kernel_ms = split_kernel_dispatch_ms(w, a.steps, torch, ea)
     achieved = r["alg_bytes"] / (kernel_ms or split_ms) / 1e6
     if kernel_ms:
         log(f"[bench] split-KV kernel by the events on its own dispatch: {kernel_ms*1e3:.1f} us = "
             f"{achieved:.0f} GB/s = {100*achieved/HBM_PEAK_GBS:.1f}% HBM (launch span with the gap before it: "
             f"{split_ms*1e3:.1f} us)")
-    kernel_name = ("splitkv_kernel<1,bf16,8 waves>" if a.no_hint or os.environ.get("EID_NO_ITEM_TABLE")
-                   else "splitkv_table_kernel<1,bf16,8 waves>")
+    kernel_name = "splitkv_even_kernel<1,bf16,8 waves,direct-to-LDS loads>"
     line = {
         "metric": METRIC, "value": r["step_GBps"], "unit": "GB/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": r["ms_per_step"],
@@ -1126,8 +1202,9 @@ def main():
                                  if a.partition == 0 and not a.no_shuffle and not a.unfused else None),
                      "alg_bytes_per_launch": r["alg_bytes"], "launch_us": (kernel_ms or split_ms) * 1e3,
                      "launch_span_us": split_ms * 1e3,
-                     "how": ("HIP events attached to the split-KV kernel's own dispatch inside full steps "
-                             "(hipExtLaunchKernel start / stop events): the kernel's duration; launch_span_us = "
+                     "how": ("HIP events attached to the split-KV kernel's own dispatch inside full steps, run "
+                             "through the measurement build of the library (the same sources with -DEID_MEASURE; "
+                             "hipExtLaunchKernel start / stop events): the kernel's duration; launch_span_us = "
                              "from an event before the eid_attn_decode call to the library's split_done_event "
                              "(the kernel plus the launch gap before it)") if kernel_ms else
                             ("HIP events inside full steps: before the eid_attn_decode call -> the "

@@ -105,7 +105,8 @@ EXPORTS = ("eid_kv_write", "eid_rope_kv_write", "eid_qkv_rope_kv_write", "eid_at
            "eid_attn_decode_noalloc", "eid_attn_varlen", "eid_lse_merge", "eid_o_proj",
            "eid_workspace_bytes", "eid_partition_size", "eid_last_error", "eid_version")
 # only in the measurement build (include/eidola_attn_measure.h)
-MEASURE_EXPORTS = ("eid_debug_set_timeline", "eid_debug_set_kernel_events")
+MEASURE_EXPORTS = ("eid_debug_set_timeline", "eid_debug_set_kernel_events",
+                   "eid_debug_set_store_every_partition")
 SCHED_EXPORTS = ("eid_sched_create", "eid_sched_destroy", "eid_sched_add_seq",
                  "eid_sched_free_seq", "eid_sched_seq_len", "eid_sched_free_blocks",
                  "eid_sched_block_refs", "eid_sched_build_batch")
@@ -180,6 +181,8 @@ def _bind(path, measure):
         lib.eid_debug_set_timeline.restype = None
         lib.eid_debug_set_kernel_events.argtypes = [P, P]
         lib.eid_debug_set_kernel_events.restype = None
+        lib.eid_debug_set_store_every_partition.argtypes = [C.c_int32]
+        lib.eid_debug_set_store_every_partition.restype = None
     # host-side scheduler (include/eidola_sched.h)
     lib.eid_sched_create.argtypes = [C.POINTER(SchedConfig), C.POINTER(P)]
     lib.eid_sched_create.restype = C.c_int32

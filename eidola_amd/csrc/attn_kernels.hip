@@ -2422,6 +2422,59 @@ int device_cus() {
   return cus;
 }
 
+// Measurement aids, compiled into the measurement build only (-DEID_MEASURE): the serving
+// library carries neither the entry points nor their process-wide state.
+//  * a device buffer of `entries` records of 64 bytes that the next prefill launches of the
+//    process fill with per-wave time stamps (null: off; launches with more waves than entries
+//    leave the buffer alone);
+//  * a pair of HIP events that the next decode launches attach to the split-KV kernel's own
+//    dispatch (hipExtLaunchKernel): the time between them is the kernel's duration as a
+//    profiler reports it, without the gaps that events recorded around a launch include.
+// The settings are read once per launch (atomics); what they point to is the caller's and
+// must outlive the setting.
+#ifdef EID_MEASURE
+static std::atomic<unsigned long long *> g_timeline{nullptr};
+static std::atomic<long long> g_timeline_entries{0};
+void set_timeline(void *buf, long long entries) {
+  g_timeline_entries.store(0);
+  g_timeline.store(static_cast<unsigned long long *>(buf));
+  g_timeline_entries.store(buf ? entries : 0);
+}
+static unsigned long long *timeline_for(const long long waves) {
+  return waves <= g_timeline_entries.load() ? g_timeline.load() : nullptr;
+}
+static std::atomic<hipEvent_t> g_kernel_start{nullptr}, g_kernel_stop{nullptr};
+void set_kernel_events(void *start, void *stop) {
+  g_kernel_start.store(static_cast<hipEvent_t>(start));
+  g_kernel_stop.store(static_cast<hipEvent_t>(stop));
+}
+//  * a switch for the even split with the caller's partition: 1 = a partial per partition, all
+//    merged by the merge kernel; 0 = one partial per piece; -1 = as EID_STORE_EVERY_PARTITION says.
+static std::atomic<int> g_store_every_partition{-1};
+void set_store_every_partition(int mode) { g_store_every_partition.store(mode); }
+int store_every_partition_override() { return g_store_every_partition.load(); }
+#else
+static unsigned long long *timeline_for(const long long) { return nullptr; }
+#endif
+
+// Launches `kern`; in the measurement build, with the two events attached to the dispatch when
+// they are set and the launch is one that they are meant for (`timed`).
+template <typename K, typename... A>
+static hipError_t launch_kernel(K kern, dim3 grid, dim3 block, unsigned shmem, hipStream_t st,
+                                bool timed, const A &...a) {
+#ifdef EID_MEASURE
+  const hipEvent_t e0 = g_kernel_start.load(), e1 = g_kernel_stop.load();
+  if (timed && e0 && e1) {
+    void *kargs[] = {const_cast<void *>(static_cast<const void *>(&a))...};
+    return hipExtLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, kargs, shmem, st, e0, e1, 0);
+  }
+#else
+  (void)timed;
+#endif
+  kern<<<grid, block, shmem, st>>>(a...);
+  return hipGetLastError();
+}
+
 template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false, bool DMA = false>
 static int fill_of() {
   static const int fill = device_fill(splitkv_kernel<NT, FP8, WAVES, RS, PAIR, DMA>, WAVES * 64);
@@ -2492,10 +2545,8 @@ template <int NT, bool FP8, int WAVES, int RS = 1, bool PAIR = false>
 static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
   dim3 grid((unsigned)item_bound(p), p.num_kv_heads / (WAVES / RS) / (PAIR ? 2 : 1));
   if constexpr (!FP8 && RS == 1) {
-    if (p.dma) {  // (never beside a prefill launch: its LDS leaves no room for one)
-      splitkv_kernel<NT, FP8, WAVES, RS, PAIR, true><<<grid, WAVES * 64, 0, st>>>(p);
-      return hipGetLastError();
-    }
+    if (p.dma)  // (never beside a prefill launch: its LDS leaves no room for one)
+      return launch_kernel(splitkv_kernel<NT, FP8, WAVES, RS, PAIR, true>, grid, dim3(WAVES * 64), 0, st, true, p);
   }
   // With a prefill launch beside it (mixed batch, p.share_cus): one 8-wave workgroup per CU.
   // A second resident workgroup adds little to a kernel that streams from HBM (it only
@@ -2515,8 +2566,7 @@ static hipError_t launch_splitkv_w(const AttnParams &p, hipStream_t st) {
       if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);
     }
   }
-  splitkv_kernel<NT, FP8, WAVES, RS, PAIR><<<grid, WAVES * 64, kPad, st>>>(p);
-  return hipGetLastError();
+  return launch_kernel(splitkv_kernel<NT, FP8, WAVES, RS, PAIR>, grid, dim3(WAVES * 64), kPad, st, true, p);
 }
 
 template <int NT, bool FP8>
@@ -2582,54 +2632,6 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
   return num_items * Hkv <= fill[ntiles == 1 ? 0 : ntiles == 3 ? 1 : 2][fp8 ? 1 : 0];
 }
 
-// Measurement aids, compiled into the measurement build only (-DEID_MEASURE): the serving
-// library carries neither the entry points nor their process-wide state.
-//  * a device buffer of `entries` records of 64 bytes that the next prefill launches of the
-//    process fill with per-wave time stamps (null: off; launches with more waves than entries
-//    leave the buffer alone);
-//  * a pair of HIP events that the next decode launches attach to the split-KV kernel's own
-//    dispatch (hipExtLaunchKernel): the time between them is the kernel's duration as a
-//    profiler reports it, without the gaps that events recorded around a launch include.
-// The settings are read once per launch (atomics); what they point to is the caller's and
-// must outlive the setting.
-#ifdef EID_MEASURE
-static std::atomic<unsigned long long *> g_timeline{nullptr};
-static std::atomic<long long> g_timeline_entries{0};
-void set_timeline(void *buf, long long entries) {
-  g_timeline_entries.store(0);
-  g_timeline.store(static_cast<unsigned long long *>(buf));
-  g_timeline_entries.store(buf ? entries : 0);
-}
-static unsigned long long *timeline_for(const long long waves) {
-  return waves <= g_timeline_entries.load() ? g_timeline.load() : nullptr;
-}
-static std::atomic<hipEvent_t> g_kernel_start{nullptr}, g_kernel_stop{nullptr};
-void set_kernel_events(void *start, void *stop) {
-  g_kernel_start.store(static_cast<hipEvent_t>(start));
-  g_kernel_stop.store(static_cast<hipEvent_t>(stop));
-}
-#else
-static unsigned long long *timeline_for(const long long) { return nullptr; }
-#endif
-
-// Launches `kern`; in the measurement build, with the two events attached to the dispatch when
-// they are set and the launch is one that they are meant for (`timed`).
-template <typename K, typename... A>
-static hipError_t launch_kernel(K kern, dim3 grid, dim3 block, unsigned shmem, hipStream_t st,
-                                bool timed, const A &...a) {
-#ifdef EID_MEASURE
-  const hipEvent_t e0 = g_kernel_start.load(), e1 = g_kernel_stop.load();
-  if (timed && e0 && e1) {
-    void *kargs[] = {const_cast<void *>(static_cast<const void *>(&a))...};
-    return hipExtLaunchKernel(reinterpret_cast<const void *>(kern), grid, block, kargs, shmem, st, e0, e1, 0);
-  }
-#else
-  (void)timed;
-#endif
-  kern<<<grid, block, shmem, st>>>(a...);
-  return hipGetLastError();
-}
-
 // Workgroups of an even split: resident all at once, one 8-wave workgroup per CU (eight waves
 // keep a CU's share of the memory system busy; of two resident workgroups the younger mostly
 // waits), smaller workgroups so that a CU holds eight waves.  EID_EVEN_WGS_PER_CU overrides
@@ -2675,7 +2677,7 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
 template <int NT, bool FP8, int WAVES, bool PAIR = false>
 static hipError_t launch_even_w(const AttnParams &p, const EvenTable &tab, hipStream_t st) {
   dim3 grid((unsigned)(tab.n > 0 ? tab.n : p.even_wgs), p.num_kv_heads / WAVES / (PAIR ? 2 : 1));
-  const bool timed = NT == 1 && p.cu_seqlens_q == nullptr;  // (the decode entry point's launch)
+  const bool timed = true;
   if constexpr (!FP8) {
     if (p.dma)
       return launch_kernel(splitkv_even_kernel<NT, FP8, WAVES, PAIR, true>, grid, dim3(WAVES * 64), 0, st, timed, p, tab);
@@ -2811,14 +2813,12 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
   const bool pre = p.lse == nullptr;  // an exact lse needs the unfolded softmax factor
   AttnParams q = p;
   q.timeline = timeline_for((long long)grid.x * kPfWaves);
-  if (fp8) {
-    if (pre) prefill_kernel<true, true><<<grid, kPfWaves * 64, 0, st>>>(q, t);
-    else prefill_kernel<true, false><<<grid, kPfWaves * 64, 0, st>>>(q, t);
-  } else {
-    if (pre) prefill_kernel<false, true><<<grid, kPfWaves * 64, 0, st>>>(q, t);
-    else prefill_kernel<false, false><<<grid, kPfWaves * 64, 0, st>>>(q, t);
-  }
-  hipError_t e = hipGetLastError();
+  const dim3 block(kPfWaves * 64);
+  hipError_t e;
+  if (fp8) e = pre ? launch_kernel(prefill_kernel<true, true>, grid, block, 0, st, true, q, t)
+                   : launch_kernel(prefill_kernel<true, false>, grid, block, 0, st, true, q, t);
+  else e = pre ? launch_kernel(prefill_kernel<false, true>, grid, block, 0, st, true, q, t)
+               : launch_kernel(prefill_kernel<false, false>, grid, block, 0, st, true, q, t);
   if (e != hipSuccess || p.pf_splits <= 1) return e;
   dim3 mgrid(p.num_q_heads / 4, num_q_tokens);
   prefill_merge_kernel<<<mgrid, 256, 0, st>>>(p);

@@ -30,6 +30,8 @@ hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipSt
 #ifdef EID_MEASURE
 void set_timeline(void *buf, long long entries);
 void set_kernel_events(void *start, void *stop);
+void set_store_every_partition(int mode);
+int store_every_partition_override();
 #endif
 bool build_prefill_table(const AttnParams &p, const int32_t *seq_lens_host,
                          const int32_t *cu_seqlens_q_host, PfTable *tab);
@@ -575,6 +577,9 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   if (p.mixed_wgs > 0 && p.even_wgs > p.mixed_wgs) p.even_wgs = p.mixed_wgs;
   static const bool every = getenv("EID_STORE_EVERY_PARTITION") != nullptr;  // measurement aid
   p.store_every_partition = every ? 1 : 0;
+#ifdef EID_MEASURE
+  if (eid::store_every_partition_override() >= 0) p.store_every_partition = eid::store_every_partition_override();
+#endif
   if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) {
     // Without the lengths: a run-time partition always takes the even split (every workgroup
     // finds its range by a scan of the device arrays); the caller's partition takes it when
@@ -694,6 +699,8 @@ void eid_debug_set_timeline(void *device_buf, int64_t entries) { eid::set_timeli
 void eid_debug_set_kernel_events(void *start_event, void *stop_event) {
   eid::set_kernel_events(start_event, stop_event);
 }
+
+void eid_debug_set_store_every_partition(int32_t mode) { eid::set_store_every_partition(mode); }
 #endif
 
 int32_t eid_partition_size(const eid_attn_desc *desc) {

@@ -24,14 +24,22 @@ extern "C" {
 void eid_debug_set_timeline(void *device_buf, int64_t entries);
 
 /* Measurement aid, no counterpart in the reference and no part of a serving path: two
- * hipEvent_t (created with timing enabled) that the next eid_attn_decode calls of this process
- * attach to the split-KV kernel's own dispatch (bf16 cache, one row per sequence, more than one
- * partition in the plan, stream not capturing): after the
- * stream has drained, hipEventElapsedTime(start, stop) is that kernel's duration as a profiler
- * reports it, without the gaps that events recorded around a launch include.  Every such launch
- * overwrites both events.  NULL, NULL switches it off (the default).
- * Process-wide and not thread-safe: set it with no eid_* call in flight. */
+ * hipEvent_t (created with timing enabled) that the next attention calls of this process attach
+ * to the dispatch of every split-KV and prefill kernel they launch (not the merges, the plan
+ * kernel or the short-span kernel): after the stream has drained, hipEventElapsedTime(start,
+ * stop) is the duration of the LAST such kernel as a profiler reports it, without the gaps that
+ * events recorded around a launch include.  Meant for calls with one such kernel (a decode
+ * call; a ragged call whose sequences are of one class).  NULL, NULL switches it off (the
+ * default).  Process-wide: set it with no eid_* call in flight. */
 void eid_debug_set_kernel_events(void *start_event, void *stop_event);
+
+/* Measurement aid: how an even split with the caller's partition size (desc.partition_size != 0)
+ * stores its partials from now on.  1: one partial per partition of that size, all of them merged
+ * by the merge kernel (what a workgroup per partition would do); 0: one partial per piece (the
+ * consecutive partitions a workgroup holds of one sequence, merged in registers: the library's
+ * way); -1: as the environment variable EID_STORE_EVERY_PARTITION said at the first call (the
+ * default).  Process-wide. */
+void eid_debug_set_store_every_partition(int32_t mode);
 
 #ifdef __cplusplus
 }
