@@ -2666,12 +2666,7 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
     else fill = ntiles == 1 ? even_fill_t<1, false>(waves) : ntiles == 3 ? even_fill_t<3, false>(waves) : even_fill_t<4, false>(waves);
   }
   const int per_cu = per_cu_env > 0 ? per_cu_env : (pair && fp8 && ntiles == 1) ? 4 : max(1, 8 / waves);
-  static const int total_env = [] {   // experiment: cap on the workgroups of an even split
-    const char *e = getenv("EID_EVEN_WGS_TOTAL");
-    return e ? atoi(e) : 0;
-  }();
-  const int wgs = max(1, min(fill, per_cu * device_cus()) / (Hkv > 8 ? Hkv / 8 : 1));
-  return total_env > 0 ? min(wgs, total_env) : wgs;
+  return max(1, min(fill, per_cu * device_cus()) / (Hkv > 8 ? Hkv / 8 : 1));
 }
 
 template <int NT, bool FP8, int WAVES, bool PAIR = false>

@@ -219,7 +219,6 @@ Plan make_plan(const eid_attn_desc *d) {
     if (pl.dynamic) pl.nparts_max += 1;
     pl.parts_bytes = ((size_t)d->num_seqs * sizeof(int32_t) + 255) / 256 * 256;
   }
-  if (getenv("EID_EXP_ODD") && pl.nparts_max > 1) pl.nparts_max |= 1;
   pl.ws_rows = std::min(d->max_q_len, short_q_max(d));
   const size_t cells = (size_t)d->num_seqs * pl.ws_rows * d->num_q_heads * pl.nparts_max;
   pl.ml_bytes = (cells * 2 * sizeof(float) + 255) / 256 * 256;
