@@ -875,7 +875,11 @@ def gather_bench(torch, ea, synth, np):
             ("shuffled", 32, 0, 75, 0), ("shuffled", 32, 0, 0, 0), ("shuffled", 16, 0, 75, 0), ("shuffled", 64, 0, 75, 0),
             ("contiguous", 32, 0, 75, 0), ("shuffled", 32, 40, 75, 0), ("shuffled", 32, 128, 75, 0),
             ("shuffled", 32, 0, 75, 1), ("shuffled", 32, 0, 0, 1), ("contiguous", 32, 0, 75, 1), ("contiguous", 32, 0, 0, 1),
-            ("shuffled_x8", 32, 0, 75, 0), ("shuffled_x8", 32, 0, 75, 1), ("contiguous_x8", 32, 0, 75, 1)):
+            ("shuffled_x8", 32, 0, 75, 0), ("shuffled_x8", 32, 0, 75, 1), ("contiguous_x8", 32, 0, 75, 1),
+            # the same with the non-temporal hint on the loads (2: whole rows, 3: head slices), and
+            # one workgroup per CU as the decode kernel's even split launches them
+            ("shuffled", 32, 0, 75, 2), ("shuffled", 32, 0, 75, 3), ("shuffled", 58, 0, 150, 2), ("shuffled", 58, 0, 150, 0),
+            ("shuffled_x8", 32, 0, 75, 2), ("shuffled_x8", 32, 0, 75, 3), ("shuffled_x8", 58, 0, 150, 2)):
         nwg = npages // ppw
         if kind.endswith("_x8"):  # all eight page sets in one launch: the rate without the ends
             nwg *= w.n
@@ -888,9 +892,10 @@ def gather_bench(torch, ea, synth, np):
             run(i)
         ms = event_ms(run, 100, torch)
         nbytes = nwg * ppw * 2 * 16384
-        r = {"config": f"gather_probe_{kind}_{ppw}_pages_per_wg_delay_{delay}_lds_{lds}k_{'rows' if rows else 'heads'}", "ms": ms, "bytes": nbytes,
+        shape = ("one head", "whole rows", "whole rows, non-temporal", "one head, non-temporal")[rows]
+        r = {"config": f"gather_probe_{kind}_{ppw}_pages_per_wg_delay_{delay}_lds_{lds}k_{shape.replace(', ', '_').replace(' ', '_')}", "ms": ms, "bytes": nbytes,
              "GBps": nbytes / ms / 1e6, "workgroups": nwg}
-        log(f"[bench] gather probe, {kind} pages, {ppw} per workgroup ({nwg} workgroups, {lds} KiB LDS, a wave reads {'whole rows' if rows else 'one head'}), {delay} ALU "
+        log(f"[bench] gather probe, {kind} pages, {ppw} per workgroup ({nwg} workgroups, {lds} KiB LDS, a wave reads {shape}), {delay} ALU "
             f"links per batch: {ms*1e3:.1f} us for {nbytes/1e6:.1f} MB = {r['GBps']:.0f} GB/s = {100*r['GBps']/HBM_PEAK_GBS:.1f}% of peak")
         res.append(r)
     # the same access patterns against pages that stay in cache (64 distinct pages, 2 MiB of K and
