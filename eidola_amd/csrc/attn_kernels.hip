@@ -2634,8 +2634,9 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
 
 // Workgroups of an even split: resident all at once, one 8-wave workgroup per CU (eight waves
 // keep a CU's share of the memory system busy; of two resident workgroups the younger mostly
-// waits), smaller workgroups so that a CU holds eight waves.  EID_EVEN_WGS_PER_CU overrides
-// the number per CU for measurements.
+// waits), smaller workgroups so that a CU holds eight waves (the four-wave head-pair kernel
+// of config 4: one per CU 294 us, two 267, three 271, four 280: more ranges are more pieces
+// to store and merge).  EID_EVEN_WGS_PER_CU overrides the number per CU for measurements.
 template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
 static int even_fill_of() {
   static const int fill = device_fill(splitkv_even_kernel<NT, FP8, WAVES, PAIR, DMA>, WAVES * 64);
@@ -2665,7 +2666,7 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
     else if (dma) fill = ntiles == 1 ? even_fill_t<1, false, true>(waves) : ntiles == 3 ? even_fill_t<3, false, true>(waves) : even_fill_t<4, false, true>(waves);
     else fill = ntiles == 1 ? even_fill_t<1, false>(waves) : ntiles == 3 ? even_fill_t<3, false>(waves) : even_fill_t<4, false>(waves);
   }
-  const int per_cu = per_cu_env > 0 ? per_cu_env : (pair && fp8 && ntiles == 1) ? 4 : max(1, 8 / waves);
+  const int per_cu = per_cu_env > 0 ? per_cu_env : max(1, 8 / waves);
   return max(1, min(fill, per_cu * device_cus()) / (Hkv > 8 ? Hkv / 8 : 1));
 }
 

@@ -368,23 +368,27 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 // through that XCD's L2.
 // Requires K % 64 == 0 and N % 16 == 0.
 // ---------------------------------------------------------------------------------------
-namespace {
-constexpr int kTlK = 64;
-constexpr int kTlRowBytes = 144;
-}  // namespace
 
 // WT = 16-row MFMA tiles per wave and dimension: 4 gives the 128 x 128 workgroup tile, 2 a
 // 64 x 64 one for batches too small to fill the device with the big tile (its K loop is as
 // long, but four workgroups share a CU).
-template <int WT>
-__global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
+// KT = K elements per step: 64, or 128 for the small tile (a loading instruction then covers
+// 4 rows x 256 contiguous bytes instead of 8 rows x 128, and there are half as many steps,
+// each of which is a round trip of loads, LDS stores and a barrier whatever it carries).
+template <int WT, int KT = 64>
+__global__ __launch_bounds__(256, (WT == 4 || KT == 128) ? 2 : 4) void oproj_tiled_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
     uint16_t *out, const int T, const int N, const int K, const int tiles_m,
     const int tiles_n) {
   constexpr int kTile = 32 * WT;  // rows of a workgroup tile in either dimension
   constexpr int kWave = 16 * WT;  // rows of a wave tile
+  constexpr int kTlK = KT;
+  constexpr int kTlRowBytes = 2 * KT + 16;  // (144 or 272 bytes: 16 lanes x 16 bytes of 16 rows on distinct banks)
   constexpr int kTileBytes = kTile * kTlRowBytes;
+  constexpr int kSegs = KT / 8;             // 16-byte segments of a row
+  constexpr int kRowsPerPass = 256 / kSegs; // rows the 256 threads cover with one load each
+  constexpr int kPasses = kTile / kRowsPerPass;
   __shared__ __align__(16) uint8_t lds_w[2][kTileBytes];
   __shared__ __align__(16) uint8_t lds_a[2][kTileBytes];
   const int tid = threadIdx.x, lane = tid & 63;
@@ -405,13 +409,13 @@ __global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
   const int tm = first_m + in_group % rows, tn = in_group / rows;
   const int m0 = tm * kTile, n0 = tn * kTile;
 
-  // loader: a wave instruction covers 8 rows x 128 bytes (full lines)
-  const int ld_row = tid >> 3, ld_seg = tid & 7;  // rows ld_row + 32 j
-  const uint16_t *wsrc[WT], *asrc[WT];
+  // loader: a wave instruction covers 8 rows x 128 bytes, or 4 rows x 256 (full lines)
+  const int ld_row = tid / kSegs, ld_seg = tid % kSegs;  // rows ld_row + kRowsPerPass j
+  const uint16_t *wsrc[kPasses], *asrc[kPasses];
 #pragma unroll
-  for (int j = 0; j < WT; ++j) {
-    wsrc[j] = w + (size_t)min(n0 + ld_row + 32 * j, N - 1) * K + ld_seg * 8;
-    asrc[j] = a + (size_t)min(m0 + ld_row + 32 * j, T - 1) * K + ld_seg * 8;
+  for (int j = 0; j < kPasses; ++j) {
+    wsrc[j] = w + (size_t)min(n0 + ld_row + kRowsPerPass * j, N - 1) * K + ld_seg * 8;
+    asrc[j] = a + (size_t)min(m0 + ld_row + kRowsPerPass * j, T - 1) * K + ld_seg * 8;
   }
   const uint32_t st_off = (uint32_t)ld_row * kTlRowBytes + ld_seg * 16;
   f32x4 acc[WT][WT];  // [feature tile][token tile]
@@ -426,19 +430,19 @@ __global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
   // Two register stages: the loads of K step i + 2 are issued while step i is computed and
   // are only needed (moved to LDS) at the end of step i + 1, so every global load has two
   // full steps to arrive.
-  u32x4 wr[2][WT], ar[2][WT];
+  u32x4 wr[2][kPasses], ar[2][kPasses];
   auto fetch = [&](const int st, const int k0) {
 #pragma unroll
-    for (int j = 0; j < WT; ++j) {
+    for (int j = 0; j < kPasses; ++j) {
       wr[st][j] = ld16(wsrc[j] + k0);
       ar[st][j] = ld16(asrc[j] + k0);
     }
   };
   auto stash = [&](const int st, const int buf) {
 #pragma unroll
-    for (int j = 0; j < WT; ++j) {
-      *(u32x4 *)(&lds_w[buf][st_off + j * 32 * kTlRowBytes]) = wr[st][j];
-      *(u32x4 *)(&lds_a[buf][st_off + j * 32 * kTlRowBytes]) = ar[st][j];
+    for (int j = 0; j < kPasses; ++j) {
+      *(u32x4 *)(&lds_w[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = wr[st][j];
+      *(u32x4 *)(&lds_a[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = ar[st][j];
     }
   };
   const int nk = K / kTlK;
@@ -448,7 +452,7 @@ __global__ __launch_bounds__(256, WT == 4 ? 2 : 4) void oproj_tiled_kernel(
     // LDS stores below to wait for all of them
     fetch(par, min(i + 2, nk - 1) * kTlK);
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < KT / 32; ++ks) {
       Frag8 wf[WT], af[WT];
 #pragma unroll
       for (int x = 0; x < WT; ++x) {
@@ -655,8 +659,14 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
                                                             tiles_m, tiles_n);
   } else {
     const int tiles_m = (T + 63) / 64, tiles_n = (N + 63) / 64;
-    oproj_tiled_kernel<2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                            tiles_m, tiles_n);
+    // (K in steps of 128 where K allows: 256 tokens 35.1 -> 26.3 us per call; steps of 256: 25.8)
+    static const bool k64 = getenv("EID_OPROJ_K64") != nullptr;  // for A/B measurements
+    if (K % 128 == 0 && !k64)
+      oproj_tiled_kernel<2, 128><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                   tiles_m, tiles_n);
+    else
+      oproj_tiled_kernel<2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                              tiles_m, tiles_n);
   }
   return hipGetLastError();
 }
