@@ -12,6 +12,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 namespace eid {
@@ -380,11 +381,14 @@ int32_t hip_fail(hipError_t e, const char *what) {
 // list passed by value) would be frozen into the graph and silently go stale when the device
 // arrays change between replays, so under capture the host copies are ignored and the
 // kernels plan from the device arrays, as they do without them.
+// A failed query (the legacy stream while another stream captures in global mode, say) counts
+// as capturing: the launch is then sized from the descriptor, which is right in either case,
+// where a plan from the host copies frozen into somebody's graph would not be.
 bool stream_is_capturing(hipStream_t st) {
   hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(st, &status) != hipSuccess) {
     (void)hipGetLastError();
-    return false;
+    return true;
   }
   return status != hipStreamCaptureStatusNone;
 }
@@ -911,7 +915,39 @@ int32_t eid_attn_decode_noalloc(const eid_attn_desc *desc, const eid_attn_args *
   eid_attn_args own = *args;
   own.workspace = ws;
   own.workspace_bytes = eid::kStaticScratchBytes;
-  return decode_launch(desc, &own, hip_stream, true);
+  // EID_DEBUG: every caller on a GPU shares the one array, and calls that overlap in time race
+  // on it.  The checking mode remembers, per device, the stream of the last call and an event
+  // recorded behind it, and refuses a call from another stream while that event is pending.
+  // (Creates an event per device on first use: the checking mode does allocate.)
+  hipStream_t st = static_cast<hipStream_t>(hip_stream);
+  const bool watch = debug_checks_on() && !stream_is_capturing(st);
+  static std::mutex guard_mu;
+  struct Guard { hipEvent_t done = nullptr; hipStream_t last = nullptr; bool used = false; };
+  static Guard guards[64];
+  int dev = 0;
+  if (watch) {
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(EID_ERR_HIP, "EID_DEBUG: no current device");
+    std::lock_guard<std::mutex> lock(guard_mu);
+    Guard &g = guards[dev];
+    if (g.used && g.last != st && hipEventQuery(g.done) == hipErrorNotReady)
+      return fail(EID_ERR_INVALID_ARG,
+                  "EID_DEBUG: eid_attn_decode_noalloc on one stream while a call on another stream is "
+                  "still using the static workspace of this GPU");
+    (void)hipGetLastError();
+  }
+  const int32_t rc = decode_launch(desc, &own, hip_stream, true);
+  if (watch && rc == EID_OK) {
+    std::lock_guard<std::mutex> lock(guard_mu);
+    Guard &g = guards[dev];
+    if (!g.done && hipEventCreateWithFlags(&g.done, hipEventDisableTiming) != hipSuccess) {
+      g.done = nullptr;
+      return hip_fail(hipGetLastError(), "EID_DEBUG: event for the static workspace");
+    }
+    if (hipEventRecord(g.done, st) != hipSuccess) return hip_fail(hipGetLastError(), "EID_DEBUG: event record");
+    g.last = st;
+    g.used = true;
+  }
+  return rc;
 }
 
 int32_t eid_attn_varlen(const eid_attn_desc *desc, const eid_attn_args *args, void *hip_stream) {

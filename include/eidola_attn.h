@@ -212,7 +212,10 @@ int32_t eid_attn_decode(const eid_attn_desc *desc, const eid_attn_args *args,
  * planning.  All calls on one GPU share the one array: calls that overlap in time on the
  * same GPU (two streams, two threads, two graphs in flight) race on it; serialise them, or
  * give the others eid_attn_decode with their own workspace.  Nothing in the array has to
- * start from a particular value, so it is never cleared.
+ * start from a particular value, so it is never cleared.  With EID_DEBUG=1 in the environment
+ * the call remembers, per GPU, the stream of the last call and an event behind it, and returns
+ * EID_ERR_INVALID_ARG when a call arrives on another stream while that event is pending (the
+ * checking mode creates one event per GPU: it does allocate).
  */
 #define EID_STATIC_WORKSPACE_BYTES (32u << 20)
 int32_t eid_attn_decode_noalloc(const eid_attn_desc *desc, const eid_attn_args *args,

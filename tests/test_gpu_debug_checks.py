@@ -62,3 +62,57 @@ def test_debug_mode_catches_mismatched_host_copies_and_duplicate_slots():
     env = dict(os.environ, EID_DEBUG="1")
     r = subprocess.run([sys.executable, "-c", CHILD], env=env, capture_output=True, text=True, timeout=110)
     assert r.returncode == 0 and "debug checks ok" in r.stdout, r.stdout + r.stderr
+
+
+CHILD_NOALLOC = textwrap.dedent("""
+    import sys, os
+    sys.path.insert(0, %r)
+    import torch
+    import eidola_amd as ea
+    # 16 sequences of 120,000 tokens: the call's kernels run for most of a millisecond, far longer
+    # than the host needs to reach the next call (the checking mode waits for the stream before
+    # every launch, so only the last call's kernels can still be running)
+    S, L = 16, 120000
+    pages = S * (L // 16)
+    geom = ea.AttnGeometry(partition_size=2048)
+    gen = torch.Generator(device="cuda:0").manual_seed(1)
+    kc = torch.randn((pages, 16, 8, 64), generator=gen, device="cuda:0", dtype=torch.bfloat16)
+    vc = torch.randn((pages, 16, 8, 64), generator=gen, device="cuda:0", dtype=torch.bfloat16)
+    q = torch.randn((S, 64, 64), generator=gen, device="cuda:0", dtype=torch.bfloat16)
+    bt = torch.arange(pages, device="cuda:0", dtype=torch.int32).view(S, L // 16).contiguous()
+    sl = torch.full((S,), L, device="cuda:0", dtype=torch.int32)
+    args = (geom, q, kc, vc, bt, sl)
+    out, out2 = torch.zeros_like(q), torch.zeros_like(q)
+    torch.cuda.synchronize()
+    one, two = torch.cuda.Stream(), torch.cuda.Stream()
+    # (first uses take milliseconds: the library's one-time set-up, a stream's hardware queue)
+    with torch.cuda.stream(one):
+        ea.attn_decode_noalloc(*args, max_kv_len=L, out=out)
+    with torch.cuda.stream(two):
+        torch.zeros(8, device="cuda:0").add_(1)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(one):
+        ea.attn_decode_noalloc(*args, max_kv_len=L, out=out)
+    with torch.cuda.stream(two):
+        try:
+            ea.attn_decode_noalloc(*args, max_kv_len=L, out=out2)
+        except ea.EidError as e:
+            assert e.name == "EID_ERR_INVALID_ARG" and "static workspace" in str(e), str(e)
+        else:
+            raise AssertionError("overlapping use of the static workspace accepted")
+    torch.cuda.synchronize()
+    with torch.cuda.stream(two):   # the first stream has drained: the other one may have the array
+        ea.attn_decode_noalloc(*args, max_kv_len=L, out=out2)
+    with torch.cuda.stream(two):   # and again on the same stream, back to back: one stream orders its calls
+        ea.attn_decode_noalloc(*args, max_kv_len=L, out=out2)
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    print("static workspace guard ok")
+""") % (ROOT,)
+
+
+def test_debug_mode_refuses_overlapping_calls_on_the_static_workspace():
+    assert torch.cuda.is_available()
+    env = dict(os.environ, EID_DEBUG="1")
+    r = subprocess.run([sys.executable, "-c", CHILD_NOALLOC], env=env, capture_output=True, text=True, timeout=110)
+    assert r.returncode == 0 and "static workspace guard ok" in r.stdout, r.stdout + r.stderr
