@@ -5,7 +5,8 @@
 //
 // Engine, per wavefront, per chunk of 64 context tokens (four 16-token pages):
 //   S^T[token][row] = K[token][:] . Q[row][:]   v_mfma_f32_16x16x32_bf16, tokens on M so a
-//        lane's 16-byte global load of a K row IS its A operand (no LDS hop for K);
+//        lane's 16 bytes of a K row ARE its A operand: loaded straight from the page (attend),
+//        or read from the wave's LDS tile that whole-line loads filled (attend_dma);
 //   online softmax in base 2 on the accumulator layout (a lane owns 4 tokens of one row,
 //        the row maximum crosses the four 16-lane rows with v_permlane{16,32}_swap);
 //   P^T leaves the softmax already in B-operand layout (tokens on the contraction axis);
