@@ -918,6 +918,135 @@ __device__ __forceinline__ void attend_dma(const AttnParams &p, const int s, con
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Head pairs over an fp8 cache (decode rows), the iteration's raw bytes brought in by direct
+// global -> LDS loads.  The register path's loads already cover whole 128-byte lines (two
+// neighbouring heads' 64-byte rows), so nothing is reshaped: a lane's 16 bytes land at
+// tile + 16 lane, exactly the register image the conversion expects, and come back with one
+// ds_read_b128.  What the detour buys is the same as in attend_dma: once an iteration's raw
+// bytes are in registers the NEXT iteration's loads are issued into the same 8 KiB (K and V
+// of 32 tokens x 2 heads) and are in flight while this one is converted, staged and
+// multiplied, where the register path has nothing in flight during its arithmetic.
+// Per wave: the V staging rows of attend (kWaveLdsBytes), then the two raw tiles.
+// ---------------------------------------------------------------------------------------
+constexpr int kPairRawBytes = 4 * 1024;                               // one tensor, one iteration
+constexpr int kWavePairDmaBytes = kWaveLdsBytes + 2 * kPairRawBytes;  // 17 KiB
+
+template <class Emit = NoEmit>
+__device__ __forceinline__ void attend_dma_pair(const AttnParams &p, const int s, const int kvh,
+                                                const int t_begin, const int t_end, const int seq_len,
+                                                const int pos_first, const int lo_last,
+                                                const Frag8 (&qf)[1][2], const RowInfo &ri,
+                                                uint8_t *wave_lds, float (&m)[1], f32x4 (&lacc)[1],
+                                                f32x4 (&acc)[1][4], const int emit_every = 0,
+                                                const Emit emit = Emit{}) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, g = lane >> 4;
+  const int Hkv = p.num_kv_heads;
+  const uint32_t row_bytes = (uint32_t)Hkv * kHeadDim;
+  const size_t page_bytes = (size_t)kBlock * row_bytes;
+  // a block of 16 slots is 8 token rows x 2 heads (lane i16 = 2 * token + head), two per page
+  const uint32_t lane_off = (uint32_t)(i16 >> 1) * row_bytes + (uint32_t)(kvh + (i16 & 1)) * kHeadDim +
+                            (uint32_t)g * 16;
+  constexpr int kBlkTok = kBlock / 2, kIter = kChunk / 2;
+  const int tok_lane = i16 >> 1;
+  const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
+  const int nblk_total = (t_end + kBlock - 1) / kBlock;
+  const float c2 = p.softmax_scale * kLog2e * p.k_scale[kvh + (i16 >> 3)];
+  uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
+  const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
+  uint8_t *rawk = wave_lds + kWaveLdsBytes, *rawv = rawk + kPairRawBytes;
+
+  auto pages_of = [&](const int ti, int (&blk)[2]) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) blk[b] = bt[min(ti / kBlock + b, nblk_total - 1)];
+  };
+  // (every block is loaded: past the end of the range the last page comes in again, real and
+  // finite data whose scores are masked and whose V rows are zeroed below)
+  auto issue = [&](const int (&blk)[2]) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const size_t off = (size_t)clamp_page(blk[b >> 1], p.last_block) * page_bytes + lane_off +
+                         (uint32_t)(b & 1) * kBlkTok * row_bytes;
+      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.k_cache + off), (dma_lptr_t *)(rawk + b * 1024), 16, 0, kDmaAux);
+      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.v_cache + off), (dma_lptr_t *)(rawv + b * 1024), 16, 0, kDmaAux);
+    }
+  };
+
+  // newest token: quantised and stored into the cache before anything of its page is requested
+  if (p.k_new && seq_len - 1 >= t_begin && seq_len - 1 < t_end) {  // wave-uniform
+    const int pos_new = seq_len - 1;
+    const int page = clamp_page(bt[pos_new / kBlock], p.last_block);
+    const bool mine = tok_lane == (pos_new & (kBlkTok - 1));
+    const size_t src = ((size_t)s * Hkv + kvh + (i16 & 1)) * kHeadDim + g * 16;
+    const size_t dst = (size_t)page * page_bytes + lane_off + (uint32_t)((pos_new & (kBlock - 1)) >= kBlkTok) * kBlkTok * row_bytes;
+#pragma unroll
+    for (int kv = 0; kv < 2; ++kv) {
+      const uint16_t *from = (kv ? p.v_new : p.k_new) + src;
+      const float sc = (kv ? p.v_scale : p.k_scale)[kvh + (i16 & 1)];
+      const u32x4 x = quantize16_fp8(*(const u32x4 *)from, *(const u32x4 *)(from + 8), sc);
+      if (mine) *(u32x4 *)(const_cast<uint8_t *>(kv ? p.v_cache : p.k_cache) + dst) = x;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the row is in place before its page is read
+  }
+
+  int blk[2];
+  pages_of(t_begin, blk);
+  issue(blk);
+  if (t_begin + kIter < t_end) pages_of(t_begin + kIter, blk);
+
+  int emit_left = emit_every, emit_k = 0;
+  int stores_behind = 0;
+  for (int ti = t_begin; ti < t_end; ti += kIter) {
+    wait_vm_all_but(stores_behind);
+    stores_behind = 0;
+    u32x4 kraw[4], vraw[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      kraw[b] = *(const u32x4 *)(rawk + b * 1024 + lane * 16);
+      vraw[b] = *(const u32x4 *)(rawv + b * 1024 + lane * 16);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (ti + kIter < t_end) {
+      issue(blk);
+      if (ti + 2 * kIter < t_end) pages_of(ti + 2 * kIter, blk);
+    }
+    // ---- V: zero rows past the sequence end, widen, stage in LDS; K operands ----
+    const bool tail = ti + kIter > seq_len;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      uint32_t lo4[4], hi4[4];
+      fp8x8_to_bf16x8(vraw[b][0], vraw[b][1], lo4);
+      fp8x8_to_bf16x8(vraw[b][2], vraw[b][3], hi4);
+      u32x4 v0 = u32x4{lo4[0], lo4[1], lo4[2], lo4[3]}, v1 = u32x4{hi4[0], hi4[1], hi4[2], hi4[3]};
+      if (tail) {  // last iteration of the sequence only
+        asm volatile("" ::: "memory");
+        if (ti + b * kBlkTok + tok_lane >= seq_len) {
+          v0 = u32x4{0, 0, 0, 0};
+          v1 = u32x4{0, 0, 0, 0};
+        }
+      }
+      *(u32x4 *)(lds_wr + b * kVPageBytes) = v0;
+      *(u32x4 *)(lds_wr + b * kVPageBytes + 16) = v1;
+    }
+    Frag8 kf[4][2];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      fp8x8_to_bf16x8(kraw[b][0], kraw[b][1], kf[b][0].w);
+      fp8x8_to_bf16x8(kraw[b][2], kraw[b][3], kf[b][1].w);
+    }
+    const bool need_mask = (ti < lo_last) || (ti + kIter > pos_first + 1);
+    chunk_step<1, kVRowBytes, false, true>(kf, lds_rd, qf, ri, ti, need_mask, c2, m, lacc, acc);
+    if constexpr (!std::is_same<Emit, NoEmit>::value) {
+      emit_left -= kIter;
+      if (emit_left == 0 && ti + kIter < t_end) {  // (wave-uniform)
+        stores_behind = emit(emit_k++);
+        emit_left = emit_every;
+      }
+    }
+  }
+}
+
 // Finish a row tile: either normalise with the sink and store bf16 output (+lse), or store
 // the partition's partial (m, l, acc) for the merge kernel.
 //
@@ -1488,9 +1617,10 @@ __device__ __forceinline__ bool even_find_start(const AttnParams &p, const int b
 // (two waves per SIMD, i.e. all 256 registers: eight waves per CU; the head-pair kernel moves
 // half the bytes per wave and load, and keeps sixteen)
 template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
-__global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kernel(const AttnParams p,
-                                                                                const EvenTable tab) {
-  __shared__ __align__(1024) uint8_t lds[WAVES * (DMA ? kWaveDmaBytes : kWaveLdsBytes)];
+__global__ __launch_bounds__(WAVES * 64, ((PAIR && !DMA) ? 4 : 2)) void splitkv_even_kernel(const AttnParams p,
+                                                                                          const EvenTable tab) {
+  constexpr int kWaveBytes = !DMA ? kWaveLdsBytes : PAIR ? kWavePairDmaBytes : kWaveDmaBytes;
+  __shared__ __align__(1024) uint8_t lds[WAVES * kWaveBytes];
   __shared__ int start_lds[4];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int kvh = (blockIdx.y * WAVES + wave) * (PAIR ? 2 : 1);
@@ -1524,7 +1654,7 @@ __global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kerne
   // the merge that follows reads the mode (and, with a partial per partition, its size) from here
   if (b == 0 && blockIdx.y == 0 && threadIdx.x == 0) p.plan_slot[0] = pieces ? (kEvenFlag | q) : p.partition;
   const int U = dyn ? kChunk : p.partition;  // keys per unit
-  uint8_t *wave_lds = lds + wave * (DMA ? kWaveDmaBytes : kWaveLdsBytes);
+  uint8_t *wave_lds = lds + wave * kWaveBytes;
   int rem = q;
   bool first_seq = true;
   SeqView v = view_seq_uniform(p, s);
@@ -1583,7 +1713,9 @@ __global__ __launch_bounds__(WAVES * 64, (PAIR ? 4 : 2)) void splitkv_even_kerne
       // finish() stores (m, l) and two 16-byte pieces per lane for every tile that holds a row
       return 3 * min(NT, (qlen + 1) / 2);
     };
-    if constexpr (DMA)
+    if constexpr (DMA && PAIR)
+      attend_dma_pair(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, pieces ? 0 : U, emit);
+    else if constexpr (DMA)
       attend_dma<NT>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, FirstPages{},
                      pieces ? 0 : U, emit);
     else
@@ -2678,6 +2810,10 @@ static hipError_t launch_even_w(const AttnParams &p, const EvenTable &tab, hipSt
   if constexpr (!FP8) {
     if (p.dma)
       return launch_kernel(splitkv_even_kernel<NT, FP8, WAVES, PAIR, true>, grid, dim3(WAVES * 64), 0, st, timed, p, tab);
+  }
+  if constexpr (PAIR) {
+    if (p.dma_pair)
+      return launch_kernel(splitkv_even_kernel<NT, FP8, WAVES, true, true>, grid, dim3(WAVES * 64), 0, st, timed, p, tab);
   }
   // (p.share_cus: one 8-wave workgroup per CU by a request for unused dynamic LDS, see launch_splitkv_w)
   const int kPad = (WAVES == 8 && p.share_cus) ? 16384 : 0;

@@ -568,6 +568,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   // bf16 cache and no prefill launch beside this one: the chunks stream in by direct global -> LDS loads
   static const bool no_dma = getenv("EID_NO_DMA") != nullptr;  // for A/B measurements
   p.dma = (!fp8 && !p.share_cus && !no_dma) ? 1 : 0;
+  p.dma_pair = (fp8 && p.fp8_pair && ntiles == 1 && !p.share_cus && !no_dma) ? 1 : 0;
   p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0);
   cp.short_span = use_shortspan(d, pl, ntiles);
   cp.merge = pl.nparts_max > 1;
