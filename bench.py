@@ -448,7 +448,7 @@ def other_configs(a, torch, ea, synth, pool2, check):
                   synth, "decode")
     ms_step, ms_attn = compact_pass(w4, steps, warm, torch)
     out["4_fp8"] = hbm(synth.algorithmic_work(w4.batches[0]), ms_attn,
-                       "splitkv_even_kernel<1,fp8,4 waves,head pairs>",
+                       "splitkv_even_kernel<1,fp8,4 waves,head pairs,direct-to-LDS loads>",
                        {"ms_per_step": ms_step, "tokens_per_s": 256 / ms_step * 1e3}, kernel_ms=kdur(w4, steps))
     if check:
         order = np.argsort(w4.batches[0].seq_lens)
