@@ -375,8 +375,14 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 // KT = K elements per step: 64, or 128 for the small tile (a loading instruction then covers
 // 4 rows x 256 contiguous bytes instead of 8 rows x 128, and there are half as many steps,
 // each of which is a round trip of loads, LDS stores and a barrier whatever it carries).
-template <int WT, int KT = 64>
-__global__ __launch_bounds__(256, (WT == 4 || KT == 128) ? 2 : 4) void oproj_tiled_kernel(
+// SPLIT = 2: the workgroup is two such groups of 4 waves, each walking one half of K with LDS
+// stages of its own (the barriers are the workgroup's, so the halves advance in step); at the
+// end the second group hands its sums over through LDS and the first runs the epilogue.  For
+// batches whose tiles do not fill the device (one workgroup per CU at most) this puts twice
+// the loads in flight per CU and halves the number of steps, with no workspace and no
+// reduction across workgroups.
+template <int WT, int KT = 64, int SPLIT = 1>
+__global__ __launch_bounds__(256 * SPLIT, SPLIT > 1 ? 1 : (WT == 4 || KT == 128) ? 2 : 4) void oproj_tiled_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
     uint16_t *out, const int T, const int N, const int K, const int tiles_m,
@@ -389,9 +395,12 @@ __global__ __launch_bounds__(256, (WT == 4 || KT == 128) ? 2 : 4) void oproj_til
   constexpr int kSegs = KT / 8;             // 16-byte segments of a row
   constexpr int kRowsPerPass = 256 / kSegs; // rows the 256 threads cover with one load each
   constexpr int kPasses = kTile / kRowsPerPass;
-  __shared__ __align__(16) uint8_t lds_w[2][kTileBytes];
-  __shared__ __align__(16) uint8_t lds_a[2][kTileBytes];
-  const int tid = threadIdx.x, lane = tid & 63;
+  __shared__ __align__(16) uint8_t lds_w_all[SPLIT][2][kTileBytes];
+  __shared__ __align__(16) uint8_t lds_a_all[SPLIT][2][kTileBytes];
+  const int grp = SPLIT > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;  // which part of K
+  uint8_t (*lds_w)[kTileBytes] = lds_w_all[grp];
+  uint8_t (*lds_a)[kTileBytes] = lds_a_all[grp];
+  const int tid = threadIdx.x & 255, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
   const int wm = wave >> 1, wn = wave & 1;
@@ -414,8 +423,8 @@ __global__ __launch_bounds__(256, (WT == 4 || KT == 128) ? 2 : 4) void oproj_til
   const uint16_t *wsrc[kPasses], *asrc[kPasses];
 #pragma unroll
   for (int j = 0; j < kPasses; ++j) {
-    wsrc[j] = w + (size_t)min(n0 + ld_row + kRowsPerPass * j, N - 1) * K + ld_seg * 8;
-    asrc[j] = a + (size_t)min(m0 + ld_row + kRowsPerPass * j, T - 1) * K + ld_seg * 8;
+    wsrc[j] = w + (size_t)min(n0 + ld_row + kRowsPerPass * j, N - 1) * K + ld_seg * 8 + grp * (K / SPLIT);
+    asrc[j] = a + (size_t)min(m0 + ld_row + kRowsPerPass * j, T - 1) * K + ld_seg * 8 + grp * (K / SPLIT);
   }
   const uint32_t st_off = (uint32_t)ld_row * kTlRowBytes + ld_seg * 16;
   f32x4 acc[WT][WT];  // [feature tile][token tile]
@@ -445,7 +454,7 @@ __global__ __launch_bounds__(256, (WT == 4 || KT == 128) ? 2 : 4) void oproj_til
       *(u32x4 *)(&lds_a[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = ar[st][j];
     }
   };
-  const int nk = K / kTlK;
+  const int nk = K / SPLIT / kTlK;
   auto step = [&](const int par, const int i) {  // par = i % 2, a literal at both call sites
     // unconditional (the last steps refetch the final slab and never use it): a fetch under
     // a branch would leave the number of loads in flight unknown at the join and force the
@@ -477,6 +486,31 @@ __global__ __launch_bounds__(256, (WT == 4 || KT == 128) ? 2 : 4) void oproj_til
     if (i + 1 < nk) step(1, i + 1);
   }
 
+  if constexpr (SPLIT > 1) {
+    // (every wave is past the last step's barrier: the stages are free) the other groups' sums ->
+    // LDS (each into its own stages) -> first group, added in group order
+    static_assert(WT * WT * 4 * 256 * 4 <= 2 * kTileBytes, "a group's sums fit its stages");
+    if (grp > 0) {
+      f32x4 *red = reinterpret_cast<f32x4 *>(&lds_w_all[grp][0][0]);
+#pragma unroll
+      for (int ft = 0; ft < WT; ++ft)
+#pragma unroll
+        for (int tt = 0; tt < WT; ++tt) red[(ft * WT + tt) * 256 + tid] = acc[ft][tt];
+    }
+    __syncthreads();
+    if (grp > 0) return;
+#pragma unroll
+    for (int gg = 1; gg < SPLIT; ++gg) {
+      const f32x4 *red = reinterpret_cast<const f32x4 *>(&lds_w_all[gg][0][0]);
+#pragma unroll
+      for (int ft = 0; ft < WT; ++ft)
+#pragma unroll
+        for (int tt = 0; tt < WT; ++tt) {
+          const f32x4 o = red[(ft * WT + tt) * 256 + tid];
+          acc[ft][tt] = f32x4{acc[ft][tt][0] + o[0], acc[ft][tt][1] + o[1], acc[ft][tt][2] + o[2], acc[ft][tt][3] + o[3]};
+        }
+    }
+  }
   oproj_epilogue<WT, WT>(acc, bias, resid, out, T, N, m0 + wm * kWave + i16, n0 + wn * kWave + 4 * g);
 }
 
@@ -659,9 +693,16 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
                                                             tiles_m, tiles_n);
   } else {
     const int tiles_m = (T + 63) / 64, tiles_n = (N + 63) / 64;
-    // (K in steps of 128 where K allows: 256 tokens 35.1 -> 26.3 us per call; steps of 256: 25.8)
+    // (K in steps of 128 where K allows: 256 tokens 35.1 -> 26.3 us per call; steps of 256: 25.8;
+    // two halves of K side by side: 22.5)
     static const bool k64 = getenv("EID_OPROJ_K64") != nullptr;  // for A/B measurements
-    if (K % 128 == 0 && !k64)
+    static const bool nosplit = getenv("EID_OPROJ_NOSPLIT") != nullptr;
+    // (tiles for at most one workgroup per CU: two halves of K side by side on every CU)
+    // (four groups with steps of 64 measured the same 22.3 us: the tiles' 189 MB through L2 are the floor)
+    if (K % 256 == 0 && !k64 && !nosplit && tiles_m * tiles_n <= device_cus())
+      oproj_tiled_kernel<2, 128, 2><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                      tiles_m, tiles_n);
+    else if (K % 128 == 0 && !k64)
       oproj_tiled_kernel<2, 128><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
                                                                    tiles_m, tiles_n);
     else

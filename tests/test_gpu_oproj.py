@@ -124,7 +124,12 @@ def test_wide_and_tiled_kernels_agree(G, monkeypatch):
     o_m = G.bits_host(ea.o_proj(a_d, w_d))
     torch.cuda.synchronize()
     # the same products summed in the same K order by the same MFMA: bit for bit
-    assert np.array_equal(o_t, o_w) and np.array_equal(o_t, o_m)
+    assert np.array_equal(o_w, o_m)
+    # the 64 x 64 kernel walks the two halves of K side by side here (77 tiles for 256 CUs) and
+    # adds the two sums at the end: equal up to one bf16 step on the few boundary cases
+    ft, fw = _f32(o_t).astype(np.float64), _f32(o_w).astype(np.float64)
+    assert np.mean(o_t == o_w) >= 0.98
+    assert np.all(np.abs(ft - fw) <= 2.0 ** -7 * np.maximum(np.abs(ft), np.abs(fw)) + 1e-3)
 
 
 @pytest.mark.parametrize("T", [33, 300])
