@@ -578,7 +578,7 @@ def rope_bench(torch, ea, synth, steps=50):
 
 def oproj_bench(torch, ea):
     """eid_o_proj on gpt-oss's shape (4096 -> 2880, bias + residual) for a 64-token decode
-    step, a 256-token batch and config 3's 4,216 tokens.  16 weight copies (377 MB, more than
+    step, batches of 256, 512 and 1,024 tokens and config 3's 4,216 tokens.  16 weight copies (377 MB, more than
     the last-level cache) are used in turn, as the layers of a model would be; 16 launches
     are captured in a HIP graph and its replay timed with events, so the figure is device
     time, not Python call overhead.  Up to 64 tokens the kernel is HBM-bound (algorithmic
@@ -588,7 +588,7 @@ def oproj_bench(torch, ea):
     ws = [torch.randn(N, K, device="cuda:0").to(torch.bfloat16) * 0.02 for _ in range(L)]
     bias = torch.randn(N, device="cuda:0").to(torch.bfloat16)
     out = []
-    for T in (64, 256, 4216):
+    for T in (64, 256, 512, 1024, 4216):
         x = torch.randn(T, K, device="cuda:0").to(torch.bfloat16)
         res = torch.randn(T, N, device="cuda:0").to(torch.bfloat16)
         y = torch.empty(T, N, dtype=torch.bfloat16, device="cuda:0")

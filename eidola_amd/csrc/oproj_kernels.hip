@@ -369,9 +369,9 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 // Requires K % 64 == 0 and N % 16 == 0.
 // ---------------------------------------------------------------------------------------
 
-// WT = 16-row MFMA tiles per wave and dimension: 4 gives the 128 x 128 workgroup tile, 2 a
-// 64 x 64 one for batches too small to fill the device with the big tile (its K loop is as
-// long, but four workgroups share a CU).
+// WF, WT = 16-row MFMA tiles per wave along features and tokens: 4, 4 gives the 128 x 128
+// workgroup tile, 2, 2 a 64 x 64 one for batches too small to fill the device with the big tile
+// (its K loop is as long, but four workgroups share a CU), 4, 2 128 features x 64 tokens.
 // KT = K elements per step: 64, or 128 for the small tile (a loading instruction then covers
 // 4 rows x 256 contiguous bytes instead of 8 rows x 128, and there are half as many steps,
 // each of which is a round trip of loads, LDS stores and a barrier whatever it carries).
@@ -381,25 +381,26 @@ __global__ __launch_bounds__(kSkWaves * 64) void oproj_skinny_kernel(
 // batches whose tiles do not fill the device (one workgroup per CU at most) this puts twice
 // the loads in flight per CU and halves the number of steps, with no workspace and no
 // reduction across workgroups.
-template <int WT, int KT = 64, int SPLIT = 1>
-__global__ __launch_bounds__(256 * SPLIT, SPLIT > 1 ? 1 : (WT == 4 || KT == 128) ? 2 : 4) void oproj_tiled_kernel(
+template <int WF, int WT, int KT = 64, int SPLIT = 1>
+__global__ __launch_bounds__(256 * SPLIT, SPLIT > 1 ? 1 : (WF == 4 || KT == 128) ? 2 : 4) void oproj_tiled_kernel(
     const uint16_t *__restrict__ a, const uint16_t *__restrict__ w,
     const uint16_t *__restrict__ bias, const uint16_t *resid,
     uint16_t *out, const int T, const int N, const int K, const int tiles_m,
     const int tiles_n) {
-  constexpr int kTile = 32 * WT;  // rows of a workgroup tile in either dimension
-  constexpr int kWave = 16 * WT;  // rows of a wave tile
+  // WF / WT = 16-row MFMA tiles per wave along the features / the tokens (2 x 2 waves)
+  constexpr int kTileN = 32 * WF, kTileM = 32 * WT;  // rows of the workgroup tile
+  constexpr int kWaveN = 16 * WF, kWaveM = 16 * WT;  // rows of a wave tile
   constexpr int kTlK = KT;
   constexpr int kTlRowBytes = 2 * KT + 16;  // (144 or 272 bytes: 16 lanes x 16 bytes of 16 rows on distinct banks)
-  constexpr int kTileBytes = kTile * kTlRowBytes;
+  constexpr int kBytesN = kTileN * kTlRowBytes, kBytesM = kTileM * kTlRowBytes;
   constexpr int kSegs = KT / 8;             // 16-byte segments of a row
   constexpr int kRowsPerPass = 256 / kSegs; // rows the 256 threads cover with one load each
-  constexpr int kPasses = kTile / kRowsPerPass;
-  __shared__ __align__(16) uint8_t lds_w_all[SPLIT][2][kTileBytes];
-  __shared__ __align__(16) uint8_t lds_a_all[SPLIT][2][kTileBytes];
+  constexpr int kPassesN = kTileN / kRowsPerPass, kPassesM = kTileM / kRowsPerPass;
+  __shared__ __align__(16) uint8_t lds_w_all[SPLIT][2][kBytesN];
+  __shared__ __align__(16) uint8_t lds_a_all[SPLIT][2][kBytesM];
   const int grp = SPLIT > 1 ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 8) : 0;  // which part of K
-  uint8_t (*lds_w)[kTileBytes] = lds_w_all[grp];
-  uint8_t (*lds_a)[kTileBytes] = lds_a_all[grp];
+  uint8_t (*lds_w)[kBytesN] = lds_w_all[grp];
+  uint8_t (*lds_a)[kBytesM] = lds_a_all[grp];
   const int tid = threadIdx.x & 255, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int i16 = lane & 15, g = lane >> 4;
@@ -416,43 +417,42 @@ __global__ __launch_bounds__(256 * SPLIT, SPLIT > 1 ? 1 : (WT == 4 || KT == 128)
   const int rows = min(tiles_m - first_m, 8);
   const int in_group = logical % group_size;
   const int tm = first_m + in_group % rows, tn = in_group / rows;
-  const int m0 = tm * kTile, n0 = tn * kTile;
+  const int m0 = tm * kTileM, n0 = tn * kTileN;
 
   // loader: a wave instruction covers 8 rows x 128 bytes, or 4 rows x 256 (full lines)
   const int ld_row = tid / kSegs, ld_seg = tid % kSegs;  // rows ld_row + kRowsPerPass j
-  const uint16_t *wsrc[kPasses], *asrc[kPasses];
+  const uint16_t *wsrc[kPassesN], *asrc[kPassesM];
 #pragma unroll
-  for (int j = 0; j < kPasses; ++j) {
+  for (int j = 0; j < kPassesN; ++j)
     wsrc[j] = w + (size_t)min(n0 + ld_row + kRowsPerPass * j, N - 1) * K + ld_seg * 8 + grp * (K / SPLIT);
-    asrc[j] = a + (size_t)min(m0 + ld_row + kRowsPerPass * j, T - 1) * K + ld_seg * 8 + grp * (K / SPLIT);
-  }
-  const uint32_t st_off = (uint32_t)ld_row * kTlRowBytes + ld_seg * 16;
-  f32x4 acc[WT][WT];  // [feature tile][token tile]
 #pragma unroll
-  for (int ft = 0; ft < WT; ++ft)
+  for (int j = 0; j < kPassesM; ++j)
+    asrc[j] = a + (size_t)min(m0 + ld_row + kRowsPerPass * j, T - 1) * K + ld_seg * 8 + grp * (K / SPLIT);
+  const uint32_t st_off = (uint32_t)ld_row * kTlRowBytes + ld_seg * 16;
+  f32x4 acc[WF][WT];  // [feature tile][token tile]
+#pragma unroll
+  for (int ft = 0; ft < WF; ++ft)
 #pragma unroll
     for (int tt = 0; tt < WT; ++tt) acc[ft][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const uint32_t rd_w = (uint32_t)(wn * kWave + i16) * kTlRowBytes + g * 16;
-  const uint32_t rd_a = (uint32_t)(wm * kWave + i16) * kTlRowBytes + g * 16;
+  const uint32_t rd_w = (uint32_t)(wn * kWaveN + i16) * kTlRowBytes + g * 16;
+  const uint32_t rd_a = (uint32_t)(wm * kWaveM + i16) * kTlRowBytes + g * 16;
 
   // Two register stages: the loads of K step i + 2 are issued while step i is computed and
   // are only needed (moved to LDS) at the end of step i + 1, so every global load has two
   // full steps to arrive.
-  u32x4 wr[2][kPasses], ar[2][kPasses];
+  u32x4 wr[2][kPassesN], ar[2][kPassesM];
   auto fetch = [&](const int st, const int k0) {
 #pragma unroll
-    for (int j = 0; j < kPasses; ++j) {
-      wr[st][j] = ld16(wsrc[j] + k0);
-      ar[st][j] = ld16(asrc[j] + k0);
-    }
+    for (int j = 0; j < kPassesN; ++j) wr[st][j] = ld16(wsrc[j] + k0);
+#pragma unroll
+    for (int j = 0; j < kPassesM; ++j) ar[st][j] = ld16(asrc[j] + k0);
   };
   auto stash = [&](const int st, const int buf) {
 #pragma unroll
-    for (int j = 0; j < kPasses; ++j) {
-      *(u32x4 *)(&lds_w[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = wr[st][j];
-      *(u32x4 *)(&lds_a[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = ar[st][j];
-    }
+    for (int j = 0; j < kPassesN; ++j) *(u32x4 *)(&lds_w[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = wr[st][j];
+#pragma unroll
+    for (int j = 0; j < kPassesM; ++j) *(u32x4 *)(&lds_a[buf][st_off + j * kRowsPerPass * kTlRowBytes]) = ar[st][j];
   };
   const int nk = K / SPLIT / kTlK;
   auto step = [&](const int par, const int i) {  // par = i % 2, a literal at both call sites
@@ -462,14 +462,13 @@ __global__ __launch_bounds__(256 * SPLIT, SPLIT > 1 ? 1 : (WT == 4 || KT == 128)
     fetch(par, min(i + 2, nk - 1) * kTlK);
 #pragma unroll
     for (int ks = 0; ks < KT / 32; ++ks) {
-      Frag8 wf[WT], af[WT];
+      Frag8 wf[WF], af[WT];
 #pragma unroll
-      for (int x = 0; x < WT; ++x) {
-        wf[x].u = *(const u32x4 *)(&lds_w[par][rd_w + x * 16 * kTlRowBytes + ks * 64]);
-        af[x].u = *(const u32x4 *)(&lds_a[par][rd_a + x * 16 * kTlRowBytes + ks * 64]);
-      }
+      for (int x = 0; x < WF; ++x) wf[x].u = *(const u32x4 *)(&lds_w[par][rd_w + x * 16 * kTlRowBytes + ks * 64]);
 #pragma unroll
-      for (int ft = 0; ft < WT; ++ft)
+      for (int x = 0; x < WT; ++x) af[x].u = *(const u32x4 *)(&lds_a[par][rd_a + x * 16 * kTlRowBytes + ks * 64]);
+#pragma unroll
+      for (int ft = 0; ft < WF; ++ft)
 #pragma unroll
         for (int tt = 0; tt < WT; ++tt) acc[ft][tt] = mfma16x32(wf[ft], af[tt], acc[ft][tt]);
     }
@@ -488,30 +487,34 @@ __global__ __launch_bounds__(256 * SPLIT, SPLIT > 1 ? 1 : (WT == 4 || KT == 128)
 
   if constexpr (SPLIT > 1) {
     // (every wave is past the last step's barrier: the stages are free) the other groups' sums ->
-    // LDS (each into its own stages) -> first group, added in group order
-    static_assert(WT * WT * 4 * 256 * 4 <= 2 * kTileBytes, "a group's sums fit its stages");
+    // LDS (each into its own stages: the weight stages first, then the activation stages) ->
+    // first group, added in group order
+    constexpr int kInW = 2 * kBytesN / 4096, kInA = 2 * kBytesM / 4096;  // tiles of 256 x 16 bytes
+    static_assert(WF * WT <= kInW + kInA, "a group's sums fit its stages");
+    auto cell = [&](const int gg, const int idx) {
+      return idx < kInW ? reinterpret_cast<f32x4 *>(&lds_w_all[gg][0][0]) + idx * 256 + tid
+                        : reinterpret_cast<f32x4 *>(&lds_a_all[gg][0][0]) + (idx - kInW) * 256 + tid;
+    };
     if (grp > 0) {
-      f32x4 *red = reinterpret_cast<f32x4 *>(&lds_w_all[grp][0][0]);
 #pragma unroll
-      for (int ft = 0; ft < WT; ++ft)
+      for (int ft = 0; ft < WF; ++ft)
 #pragma unroll
-        for (int tt = 0; tt < WT; ++tt) red[(ft * WT + tt) * 256 + tid] = acc[ft][tt];
+        for (int tt = 0; tt < WT; ++tt) *cell(grp, ft * WT + tt) = acc[ft][tt];
     }
     __syncthreads();
     if (grp > 0) return;
 #pragma unroll
     for (int gg = 1; gg < SPLIT; ++gg) {
-      const f32x4 *red = reinterpret_cast<const f32x4 *>(&lds_w_all[gg][0][0]);
 #pragma unroll
-      for (int ft = 0; ft < WT; ++ft)
+      for (int ft = 0; ft < WF; ++ft)
 #pragma unroll
         for (int tt = 0; tt < WT; ++tt) {
-          const f32x4 o = red[(ft * WT + tt) * 256 + tid];
+          const f32x4 o = *cell(gg, ft * WT + tt);
           acc[ft][tt] = f32x4{acc[ft][tt][0] + o[0], acc[ft][tt][1] + o[1], acc[ft][tt][2] + o[2], acc[ft][tt][3] + o[3]};
         }
     }
   }
-  oproj_epilogue<WT, WT>(acc, bias, resid, out, T, N, m0 + wm * kWave + i16, n0 + wn * kWave + 4 * g);
+  oproj_epilogue<WF, WT>(acc, bias, resid, out, T, N, m0 + wm * kWaveM + i16, n0 + wn * kWaveN + 4 * g);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -659,55 +662,67 @@ hipError_t launch_o_proj(const uint16_t *a, const uint16_t *w, const uint16_t *b
   // Which tiling?  Every kernel covers the output in rounds of workgroups, and a workgroup that
   // walks all of K takes about as long whatever its tile (the K steps' load latency): measured
   // for 2880 x 4096, a round of the 256 x 192 kernel (one workgroup per CU) takes ~85 us and a
-  // round of the direct-to-LDS 128 x 128 kernel (two per CU) ~63 us.  The cheaper plan wins;
-  // batches too small to give three quarters of the CUs a 128 x 128 tile take 64 x 64 tiles.
+  // round of the direct-to-LDS 128 x 128 kernel (two per CU) ~63 us.  The cheaper plan wins.
+  // Batches whose tiles give at most one workgroup per CU take the register-staged kernel with
+  // the two halves of K side by side in one workgroup.  Such a workgroup is bound by what its CU
+  // takes in per unit of time (~48 GB/s of tile rows, whatever the tile), i.e. by
+  // K x (tile features + tile tokens) bytes: of the tiles that cover the output with no more
+  // workgroups than CUs (features x tokens: 64 x 64, 96 x 64, 128 x 64, 96 x 128, 128 x 128) the
+  // one with the smallest sum is taken.
   // EID_OPROJ_KERNEL=wide|mid|tiled overrides the choice (tests, measurements); "tiled" is the
-  // register-staged kernel that the direct-to-LDS ones replaced above ~1,000 tokens.
-  {
-    const int cus = device_cus();
-    const long tw = (long)((T + 255) / 256) * ((N + 191) / 192);
-    const long tb = (long)((T + 127) / 128) * ((N + 127) / 128);
-    const double wide_cost = (double)((tw + cus - 1) / cus) * 85.0;
-    const double mid_cost = (double)((tb + 2 * cus - 1) / (2 * cus)) * 63.0;
-    int plan = 4 * tb < 3 * cus ? 0 : wide_cost < mid_cost ? 2 : 1;  // 0 = 64 x 64 tiles, 1 = mid, 2 = wide
-    if (const char *e = getenv("EID_OPROJ_KERNEL")) plan = e[0] == 'w' ? 2 : e[0] == 'm' ? 1 : e[0] == 't' ? 0 : plan;
-    if (plan == 2) {
-      const int tiles_m = (T + 255) / 256, tiles_n = (N + 191) / 192;
-      oproj_wide_kernel<6, 4, 2, 4, 1><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                                         tiles_m, tiles_n);
-      return hipGetLastError();
-    }
-    if (plan == 1) {
-      const int tiles_m = (T + 127) / 128, tiles_n = (N + 127) / 128;
-      oproj_wide_kernel<4, 4, 2, 2, 2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                                         tiles_m, tiles_n);
-      return hipGetLastError();
-    }
+  // register-staged kernel; EID_OPROJ_NOSPLIT=1 and EID_OPROJ_K64=1 take its earlier forms (one
+  // group of four waves; K in steps of 64) for A/B measurements.
+  const int cus = device_cus();
+  static const bool k64 = getenv("EID_OPROJ_K64") != nullptr;
+  static const bool nosplit = getenv("EID_OPROJ_NOSPLIT") != nullptr;
+  const long t64 = (long)((T + 63) / 64) * ((N + 63) / 64);
+  const long tb = (long)((T + 127) / 128) * ((N + 127) / 128);
+  struct Cand { int nf, nt; };
+  static const Cand cands[5] = {{64, 64}, {96, 64}, {128, 64}, {96, 128}, {128, 128}};
+  int best = -1;
+  for (int c = 0; c < 5; ++c) {
+    const long cnt = (long)((T + cands[c].nt - 1) / cands[c].nt) * ((N + cands[c].nf - 1) / cands[c].nf);
+    if (cnt <= cus && (best < 0 || cands[c].nf + cands[c].nt < cands[best].nf + cands[best].nt)) best = c;
   }
-  // The 128 x 128 tile once it gives most CUs a workgroup, else 64 x 64 (measured
-  // crossover for 2880 x 4096: between 1,024 and 1,500 tokens, 184 and 276 big tiles).
-  const int big = ((T + 127) / 128) * ((N + 127) / 128);
-  if (4 * big >= 3 * device_cus()) {
+  const long tw = (long)((T + 255) / 256) * ((N + 191) / 192);
+  const double wide_cost = (double)((tw + cus - 1) / cus) * 85.0;
+  const double mid_cost = (double)((tb + 2 * cus - 1) / (2 * cus)) * 63.0;
+  int plan = 4 * tb < 3 * cus ? 0 : wide_cost < mid_cost ? 2 : 1;  // 0 = register-staged tiles, 1 = mid, 2 = wide
+  const bool split_ok = K % 256 == 0 && !k64 && !nosplit && best >= 0;
+  if (split_ok) plan = 0;
+  if (const char *e = getenv("EID_OPROJ_KERNEL")) plan = e[0] == 'w' ? 2 : e[0] == 'm' ? 1 : e[0] == 't' ? 0 : plan;
+  if (plan == 2) {
+    const int tiles_m = (T + 255) / 256, tiles_n = (N + 191) / 192;
+    oproj_wide_kernel<6, 4, 2, 4, 1><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                       tiles_m, tiles_n);
+    return hipGetLastError();
+  }
+  if (plan == 1) {
     const int tiles_m = (T + 127) / 128, tiles_n = (N + 127) / 128;
-    oproj_tiled_kernel<4><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                            tiles_m, tiles_n);
+    oproj_wide_kernel<4, 4, 2, 2, 2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
+                                                                       tiles_m, tiles_n);
+    return hipGetLastError();
+  }
+  if (plan == 0 && split_ok) {
+    const int tm = (T + cands[best].nt - 1) / cands[best].nt, tn = (N + cands[best].nf - 1) / cands[best].nf;
+    const unsigned grid = (unsigned)(tm * tn);
+    switch (best) {  // (256 tokens: 35.1 us with steps of 64, 26.3 with steps of 128, 22.5 split)
+      case 0: oproj_tiled_kernel<2, 2, 128, 2><<<grid, 512, 0, st>>>(a, w, bias, resid, out, T, N, K, tm, tn); break;
+      case 1: oproj_tiled_kernel<3, 2, 64, 2><<<grid, 512, 0, st>>>(a, w, bias, resid, out, T, N, K, tm, tn); break;
+      case 2: oproj_tiled_kernel<4, 2, 64, 2><<<grid, 512, 0, st>>>(a, w, bias, resid, out, T, N, K, tm, tn); break;
+      case 3: oproj_tiled_kernel<3, 4, 64, 2><<<grid, 512, 0, st>>>(a, w, bias, resid, out, T, N, K, tm, tn); break;
+      default: oproj_tiled_kernel<4, 4, 64, 2><<<grid, 512, 0, st>>>(a, w, bias, resid, out, T, N, K, tm, tn); break;
+    }
+  } else if (4 * tb >= 3 * cus) {
+    // the 128 x 128 tile once it gives most CUs a workgroup, else 64 x 64
+    oproj_tiled_kernel<4, 4><<<(unsigned)tb, 256, 0, st>>>(a, w, bias, resid, out, T, N, K, (T + 127) / 128,
+                                                          (N + 127) / 128);
+  } else if (K % 128 == 0 && !k64) {
+    oproj_tiled_kernel<2, 2, 128><<<(unsigned)t64, 256, 0, st>>>(a, w, bias, resid, out, T, N, K, (T + 63) / 64,
+                                                                (N + 63) / 64);
   } else {
-    const int tiles_m = (T + 63) / 64, tiles_n = (N + 63) / 64;
-    // (K in steps of 128 where K allows: 256 tokens 35.1 -> 26.3 us per call; steps of 256: 25.8;
-    // two halves of K side by side: 22.5)
-    static const bool k64 = getenv("EID_OPROJ_K64") != nullptr;  // for A/B measurements
-    static const bool nosplit = getenv("EID_OPROJ_NOSPLIT") != nullptr;
-    // (tiles for at most one workgroup per CU: two halves of K side by side on every CU)
-    // (four groups with steps of 64 measured the same 22.3 us: the tiles' 189 MB through L2 are the floor)
-    if (K % 256 == 0 && !k64 && !nosplit && tiles_m * tiles_n <= device_cus())
-      oproj_tiled_kernel<2, 128, 2><<<tiles_m * tiles_n, 512, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                                      tiles_m, tiles_n);
-    else if (K % 128 == 0 && !k64)
-      oproj_tiled_kernel<2, 128><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                                   tiles_m, tiles_n);
-    else
-      oproj_tiled_kernel<2><<<tiles_m * tiles_n, 256, 0, st>>>(a, w, bias, resid, out, T, N, K,
-                                                              tiles_m, tiles_n);
+    oproj_tiled_kernel<2, 2><<<(unsigned)t64, 256, 0, st>>>(a, w, bias, resid, out, T, N, K, (T + 63) / 64,
+                                                           (N + 63) / 64);
   }
   return hipGetLastError();
 }
