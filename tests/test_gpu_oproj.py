@@ -99,6 +99,15 @@ def test_tiled_kernel_shapes(G, T, N, K, with_bias, with_res):
     _run(G, T, N, K, with_bias, with_res, seed=T + K)
 
 
+# the two halves of K side by side in one workgroup, on every tile the host chooses from
+# (features x tokens): 64 x 64 (320 tokens), 96 x 64 (512; 640 tokens of 2,000 features ending
+# inside a tile), 128 x 64 (640), 96 x 128 (900; 700 tokens of 3,008 features), 128 x 128 (1,300)
+@pytest.mark.parametrize("T,N,K", [(320, 2880, 4096), (512, 2880, 4096), (640, 2000, 1024), (640, 2880, 4096),
+                                   (900, 2880, 4096), (700, 3008, 512), (1300, 2880, 4096)])
+def test_split_k_tiles(G, T, N, K):
+    _run(G, T, N, K, True, True, seed=T + N + K)
+
+
 @pytest.mark.parametrize("T,N,K", [(65, 2880, 4096), (128, 128, 64), (129, 16, 128), (200, 144, 576),
                                    (257, 2880, 512), (1000, 1040, 1024), (513, 208, 192),
                                    (2790, 1648, 192)])
