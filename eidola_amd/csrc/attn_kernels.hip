@@ -2292,11 +2292,27 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   const int head = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int wsrow = blockIdx.y;
   const int s = wsrow / p.ws_rows, t = wsrow % p.ws_rows;
+  // Everything that does not depend on another load is requested at once, before the first
+  // branch: the row's place in the batch, the sequence's length, the launch's partition slot,
+  // the sequence's piece count and the (m, l) pairs of the first 64 cells (cells that were not
+  // written hold anything and are dropped once the count is known).  Taken one after the other
+  // these were five dependent round trips of a kernel that lasts seven.
   float2 ml_early = make_float2(-INFINITY, 0.f);
   uint2 v_early[8];
-  if (EAGER) {
+  {
     const size_t base = (size_t)wsrow * p.nparts_max * p.num_q_heads + head;
     if (lane < p.nparts_max) ml_early = *(const float2 *)(p.ws_ml + (base + (size_t)lane * p.num_q_heads) * 2);
+  }
+  const int L_dev = p.seq_lens[s];
+  const int P_dev = p.plan_slot ? p.plan_slot[0] : p.partition;
+  const int parts_dev = p.nparts_max > 1 ? p.seq_parts[s] : 1;
+  int row0 = s, qlen = 1;
+  if (p.cu_seqlens_q) {
+    row0 = p.cu_seqlens_q[s];
+    qlen = p.cu_seqlens_q[s + 1] - row0;
+  }
+  if (EAGER) {
+    const size_t base = (size_t)wsrow * p.nparts_max * p.num_q_heads + head;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int c = 4 * j + (lane >> 4);
@@ -2305,19 +2321,14 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
         v_early[j] = *(const uint2 *)(p.ws_acc + (base + (size_t)c * p.num_q_heads) * kHeadDim + (lane & 15) * 4);
     }
   }
-  int row0 = s, qlen = 1;
-  if (p.cu_seqlens_q) {
-    row0 = p.cu_seqlens_q[s];
-    qlen = p.cu_seqlens_q[s + 1] - row0;
-  }
   if (qlen < p.qlen_lo || qlen > p.qlen_hi || qlen > p.ws_rows || t >= qlen) return;
-  const int L = min(p.seq_lens[s], p.max_blocks_per_seq * kBlock);  // as the split-KV kernels read it
+  const int L = min(L_dev, p.max_blocks_per_seq * kBlock);  // as the split-KV kernels read it
   if (L < qlen) return;
   // run-time partition: recorded by the split-KV launch of this class; else the caller's
-  const int P = p.plan_slot ? p.plan_slot[0] : p.partition;
+  const int P = P_dev;
   int nparts;
   if (P & kEvenFlag) {  // an even split with pieces of no common size left the count per sequence
-    nparts = min(p.seq_parts[s], p.nparts_max);
+    nparts = min(parts_dev, p.nparts_max);
   } else {
     if (P < 64 || (P & 63) != 0) return;  // (a slot no split-KV launch has written: nothing to merge)
     nparts = num_partitions(p, L - kv_begin(L, qlen, p.window), P);
@@ -2332,11 +2343,7 @@ __global__ __launch_bounds__(256) void lse_merge_kernel(const AttnParams p) {
   const float sink = p.sinks ? p.sinks[head] : -INFINITY;
   // the first 64 partitions' (m, l), kept for both passes
   float2 ml0 = make_float2(-INFINITY, 0.f);
-  if (EAGER) {
-    if (lane < nparts) ml0 = ml_early;
-  } else {
-    if (lane < nparts) ml0 = *(const float2 *)(p.ws_ml + (base + lane * cstride) * 2);
-  }
+  if (lane < nparts) ml0 = ml_early;
   // pass 1: global maximum over non-empty partitions and the sink
   float M = sink;
   if (ml0.y > 0.f) M = fmaxf(M, ml0.x);
