@@ -1224,6 +1224,18 @@ kc_d, vc_d = G.gpu_caches(b, k, v)
 ref, _ = oracle_out(b, q, kc, vc, sinks)
 for host in (False, True):
     print(assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, host_lens=host, hint=host), ref, "every partition"))
+# decode rows over an fp8 cache (two KV heads per wave, raw bytes through LDS), 128-key partitions
+from eidola_amd import KV_FP8_E4M3
+from helpers import fp8_scales
+seq_lens = rng.integers(2500, 6000, size=48)
+b = make_batch(seq_lens, [1] * 48, partition=128, kv_dtype=KV_FP8_E4M3)
+q, k, v, sinks = logical_tensors(b)
+ks, vs = fp8_scales(k, v)
+kc, vc = cpu_caches(b, k, v, ks, vs)
+kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+ref, _ = oracle_out(b, q, kc, vc, sinks, ks, vs)
+for host in (False, True):
+    print(assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, host_lens=host, hint=host), ref, "every partition, fp8"))
 '''
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     env = dict(os.environ, EID_STORE_EVERY_PARTITION="1")
