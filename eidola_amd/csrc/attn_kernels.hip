@@ -591,8 +591,10 @@ struct NoEmit {
 // Waits until at most `n` of the wave's vector memory operations are outstanding (they
 // complete in the order they were issued): the loads issued before the youngest n, stores, say.
 __device__ __forceinline__ void wait_vm_all_but(const int n) {
-  if (n >= 12) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+  if (n >= 14) asm volatile("s_waitcnt vmcnt(14)" ::: "memory");
+  else if (n >= 11) asm volatile("s_waitcnt vmcnt(11)" ::: "memory");
   else if (n >= 9) asm volatile("s_waitcnt vmcnt(9)" ::: "memory");
+  else if (n >= 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
   else if (n >= 6) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
   else if (n >= 3) asm volatile("s_waitcnt vmcnt(3)" ::: "memory");
   else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -922,15 +924,22 @@ __device__ __forceinline__ void attend_dma(const AttnParams &p, const int s, con
 // Head pairs over an fp8 cache (decode rows), the iteration's raw bytes brought in by direct
 // global -> LDS loads.  The register path's loads already cover whole 128-byte lines (two
 // neighbouring heads' 64-byte rows), so nothing is reshaped: a lane's 16 bytes land at
-// tile + 16 lane, exactly the register image the conversion expects, and come back with one
-// ds_read_b128.  What the detour buys is the same as in attend_dma: once an iteration's raw
-// bytes are in registers the NEXT iteration's loads are issued into the same 8 KiB (K and V
-// of 32 tokens x 2 heads) and are in flight while this one is converted, staged and
-// multiplied, where the register path has nothing in flight during its arithmetic.
-// Per wave: the V staging rows of attend (kWaveLdsBytes), then the two raw tiles.
+// block + 16 lane, exactly the register image the K conversion expects, and come back with one
+// ds_read_b128.  The V^T operands are read from the raw bytes as well: ds_read_b64_tr_b8
+// hands lane i of a 16-lane row byte i of eight 16-byte runs, i.e. one dimension of eight
+// key slots, which widened to bf16 is the MFMA operand; no bf16 copy of V is staged in LDS.
+// What the detour buys is the same as in attend_dma: once an iteration's raw bytes are in
+// registers the NEXT iteration's loads are issued into the same 8 KiB (K and V of 32 tokens
+// x 2 heads) and are in flight while this one is converted and multiplied, where the
+// register path has nothing in flight during its arithmetic.
 // ---------------------------------------------------------------------------------------
-constexpr int kPairRawBytes = 4 * 1024;                               // one tensor, one iteration
-constexpr int kWavePairDmaBytes = kWaveLdsBytes + 2 * kPairRawBytes;  // 17 KiB
+#ifndef EID_PAIR_VBLOCK
+#define EID_PAIR_VBLOCK 1152
+#endif
+constexpr int kPairRawBytes = 4 * 1024;       // one tensor, one iteration
+constexpr int kPairVBlock = EID_PAIR_VBLOCK;  // V blocks 128 bytes apart in bank terms: the two blocks of a transposing read
+constexpr int kPairTileBytes = kPairRawBytes + 4 * kPairVBlock;  // raw K, raw V of one iteration
+constexpr int kWavePairDmaBytes = 2 * kPairTileBytes;            // two iterations under way
 
 template <class Emit = NoEmit>
 __device__ __forceinline__ void attend_dma_pair(const AttnParams &p, const int s, const int kvh,
@@ -953,9 +962,11 @@ __device__ __forceinline__ void attend_dma_pair(const AttnParams &p, const int s
   const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
   const int nblk_total = (t_end + kBlock - 1) / kBlock;
   const float c2 = p.softmax_scale * kLog2e * p.k_scale[kvh + (i16 >> 3)];
-  uint8_t *lds_wr = wave_lds + i16 * kVRowBytes + g * 32;
-  const uint8_t *lds_rd = wave_lds + (4 * g + (i16 >> 2)) * kVRowBytes + 8 * (i16 & 3);
-  uint8_t *rawk = wave_lds + kWaveLdsBytes, *rawv = rawk + kPairRawBytes;
+  // V^T of (dim tile mt, block pair pr): MFMA k index e of lane row g is slot 4 g + e % 4 of block
+  // 2 pr + e / 4 (the order P is packed in); lanes 2 e, 2 e + 1 of the row address that slot's 16
+  // bytes of dims 16 mt ... 16 mt + 15, which sit at block + 16 (16 mt + slot)
+  const uint8_t *k_rd = wave_lds + lane * 16;
+  const uint8_t *vt_rd = wave_lds + kPairRawBytes + (i16 >> 3) * kPairVBlock + 64 * g + 8 * (i16 & 7);
 
   auto pages_of = [&](const int ti, int (&blk)[2]) {
 #pragma unroll
@@ -963,13 +974,14 @@ __device__ __forceinline__ void attend_dma_pair(const AttnParams &p, const int s
   };
   // (every block is loaded: past the end of the range the last page comes in again, real and
   // finite data whose scores are masked and whose V rows are zeroed below)
-  auto issue = [&](const int (&blk)[2]) {
+  auto issue = [&](const int tile_off, const int (&blk)[2]) {
+    uint8_t *rawk = wave_lds + tile_off, *rawv = rawk + kPairRawBytes;
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       const size_t off = (size_t)clamp_page(blk[b >> 1], p.last_block) * page_bytes + lane_off +
                          (uint32_t)(b & 1) * kBlkTok * row_bytes;
       __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.k_cache + off), (dma_lptr_t *)(rawk + b * 1024), 16, 0, kDmaAux);
-      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.v_cache + off), (dma_lptr_t *)(rawv + b * 1024), 16, 0, kDmaAux);
+      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.v_cache + off), (dma_lptr_t *)(rawv + b * kPairVBlock), 16, 0, kDmaAux);
     }
   };
 
@@ -990,57 +1002,181 @@ __device__ __forceinline__ void attend_dma_pair(const AttnParams &p, const int s
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the row is in place before its page is read
   }
 
+  // two iterations' loads are under way at any time: tile i + 2 is requested into the tile that
+  // iteration i has just read into registers
   int blk[2];
   pages_of(t_begin, blk);
-  issue(blk);
-  if (t_begin + kIter < t_end) pages_of(t_begin + kIter, blk);
+  issue(0, blk);
+  if (t_begin + kIter < t_end) {
+    pages_of(t_begin + kIter, blk);
+    issue(kPairTileBytes, blk);
+  }
+  if (t_begin + 2 * kIter < t_end) pages_of(t_begin + 2 * kIter, blk);
 
   int emit_left = emit_every, emit_k = 0;
-  int stores_behind = 0;
+  int stores_last = 0, stores_before = 0;  // store instructions issued after the last / the last but one request
+  int tile_off = 0;
   for (int ti = t_begin; ti < t_end; ti += kIter) {
-    wait_vm_all_but(stores_behind);
-    stores_behind = 0;
-    u32x4 kraw[4], vraw[4];
+    // this iteration's tile has landed; the next tile's eight loads (and partials stored since this
+    // tile was requested) may still be on their way
+    wait_vm_all_but(stores_before + (ti + kIter < t_end ? 8 : 0) + stores_last);
+    u32x4 kraw[4];
+    u32x2 vt[4][2];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      kraw[b] = *(const u32x4 *)(rawk + b * 1024 + lane * 16);
-      vraw[b] = *(const u32x4 *)(rawv + b * 1024 + lane * 16);
-    }
+    for (int b = 0; b < 4; ++b) kraw[b] = *(const u32x4 *)(k_rd + tile_off + b * 1024);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) vt[mt][pr] = lds_read_tr8(vt_rd + tile_off + pr * (2 * kPairVBlock) + mt * 256);
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (ti + kIter < t_end) {
-      issue(blk);
-      if (ti + 2 * kIter < t_end) pages_of(ti + 2 * kIter, blk);
+    if (ti + 2 * kIter < t_end) {
+      issue(tile_off, blk);
+      if (ti + 3 * kIter < t_end) pages_of(ti + 3 * kIter, blk);
     }
-    // ---- V: zero rows past the sequence end, widen, stage in LDS; K operands ----
-    const bool tail = ti + kIter > seq_len;
+    tile_off = kPairTileBytes - tile_off;
+    // ---- V: zero the slots past the sequence end (whatever the page holds there), widen ----
+    if (ti + kIter > seq_len) {  // last iteration of the sequence only
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      uint32_t lo4[4], hi4[4];
-      fp8x8_to_bf16x8(vraw[b][0], vraw[b][1], lo4);
-      fp8x8_to_bf16x8(vraw[b][2], vraw[b][3], hi4);
-      u32x4 v0 = u32x4{lo4[0], lo4[1], lo4[2], lo4[3]}, v1 = u32x4{hi4[0], hi4[1], hi4[2], hi4[3]};
-      if (tail) {  // last iteration of the sequence only
-        asm volatile("" ::: "memory");
-        if (ti + b * kBlkTok + tok_lane >= seq_len) {
-          v0 = u32x4{0, 0, 0, 0};
-          v1 = u32x4{0, 0, 0, 0};
+      for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int t = ti + (2 * pr + h) * kBlkTok + 2 * g;  // bytes 0, 1: token t; 2, 3: t + 1
+          const uint32_t keep = (t < seq_len ? 0x0000FFFFu : 0u) | (t + 1 < seq_len ? 0xFFFF0000u : 0u);
+#pragma unroll
+          for (int mt = 0; mt < 4; ++mt) vt[mt][pr][h] &= keep;
         }
-      }
-      *(u32x4 *)(lds_wr + b * kVPageBytes) = v0;
-      *(u32x4 *)(lds_wr + b * kVPageBytes + 16) = v1;
     }
-    Frag8 kf[4][2];
+    Frag8 kf[4][2], vf[4][2];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) fp8x8_to_bf16x8(vt[mt][pr][0], vt[mt][pr][1], vf[mt][pr].w);
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
       fp8x8_to_bf16x8(kraw[b][0], kraw[b][1], kf[b][0].w);
       fp8x8_to_bf16x8(kraw[b][2], kraw[b][3], kf[b][1].w);
     }
     const bool need_mask = (ti < lo_last) || (ti + kIter > pos_first + 1);
-    chunk_step<1, kVRowBytes, false, true>(kf, lds_rd, qf, ri, ti, need_mask, c2, m, lacc, acc);
+    chunk_core<1, false, true, false>(kf, vf, qf, ri, ti, need_mask, c2, m, lacc, acc, nullptr);
+    stores_before = stores_last;
+    stores_last = 0;
     if constexpr (!std::is_same<Emit, NoEmit>::value) {
       emit_left -= kIter;
       if (emit_left == 0 && ti + kIter < t_end) {  // (wave-uniform)
-        stores_behind = emit(emit_k++);
+        stores_last = emit(emit_k++);
+        emit_left = emit_every;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------
+// One KV head per wave over an fp8 cache (rows of several query tokens per sequence: verify
+// steps), the chunk's raw bytes brought in by direct global -> LDS loads and two chunks' loads
+// under way per wave, as in attend_dma_pair.  A head's row of a token is 64 bytes, half a
+// line: a load instruction takes the rows of a whole page (four lanes per row), and a chunk is
+// 4 KiB of K and 4 KiB of V in a wave-private tile of 64 rows x 64 bytes each.  Slot (r, pos)
+// of a 16-row block holds the row's 16-byte segment pos ^ (r / 4) ^ (2 for odd blocks): the K
+// operand reads (ds_read_b128, one row per lane) and the transposing V reads (ds_read_b64_tr_b8,
+// rows 4 g ... 4 g + 3 of two neighbouring blocks per lane row) then touch every bank once.
+// Rows past the end of the sequence repeat its last row (finite data, masked scores).
+// ---------------------------------------------------------------------------------------
+constexpr int kFp8TensorBytes = kChunk * kHeadDim;       // 64 rows x 64 bytes
+constexpr int kFp8TileBytes = 2 * kFp8TensorBytes;       // K, V of one chunk
+constexpr int kWaveFp8DmaBytes = 2 * kFp8TileBytes;      // two chunks under way
+
+template <int NT, class Emit = NoEmit>
+__device__ __forceinline__ void attend_dma_fp8(const AttnParams &p, const int s, const int kvh,
+                                               const int t_begin, const int t_end, const int seq_len,
+                                               const int pos_first, const int lo_last,
+                                               const Frag8 (&qf)[NT][2], const RowInfo &ri,
+                                               uint8_t *wave_lds, float (&m)[NT], f32x4 (&lacc)[NT],
+                                               f32x4 (&acc)[NT][4], const int emit_every = 0,
+                                               const Emit emit = Emit{}) {
+  const int lane = threadIdx.x & 63;
+  const int i16 = lane & 15, g = lane >> 4;
+  const uint32_t row_bytes = (uint32_t)p.num_kv_heads * kHeadDim;
+  const size_t page_bytes = (size_t)kBlock * row_bytes;
+  const const_i32_ptr bt = as_constant(p.block_table + (size_t)s * p.max_blocks_per_seq);
+  const int nblk_total = (t_end + kBlock - 1) / kBlock;
+  const float c2 = p.softmax_scale * kLog2e * p.k_scale[kvh];
+  // loader: lane (r, pos) = (lane / 4, lane % 4) fills slot pos of row r of a block
+  const int dr = lane >> 2;
+  const uint32_t seg_even = (uint32_t)kvh * kHeadDim + (uint32_t)(((lane & 3) ^ (dr >> 2)) * 16);
+  const uint32_t seg_odd = seg_even ^ 32u;
+  // K operand of block b: the lane's row i16, segment g (dims 16 g ... 16 g + 15)
+  const uint32_t k_rd = (uint32_t)i16 * kHeadDim + (uint32_t)((g ^ (i16 >> 2)) * 16);
+  // V^T of (dim tile mt, block pair pr): MFMA k index e of lane row g is row 4 g + e % 4 of block
+  // 2 pr + e / 4; lanes 2 e, 2 e + 1 of the lane row address that row's segment mt
+  const uint32_t vt_rd = (uint32_t)kFp8TensorBytes + (uint32_t)(i16 >> 3) * 1024 +
+                         (uint32_t)(4 * g + ((i16 >> 1) & 3)) * kHeadDim +
+                         (uint32_t)((g ^ (2 * (i16 >> 3))) * 16) + 8 * (i16 & 1);
+
+  auto pages_of = [&](const int ti, int (&blk)[4]) {
+#pragma unroll
+    for (int b = 0; b < 4; ++b) blk[b] = bt[min(ti / kBlock + b, nblk_total - 1)];
+  };
+  auto issue = [&](const int tile_off, const int ti, const int (&blk)[4]) {
+    uint8_t *ktile = wave_lds + tile_off, *vtile = ktile + kFp8TensorBytes;
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int tok = min(ti + b * kBlock + dr, seq_len - 1);
+      const size_t off = (size_t)clamp_page(blk[b], p.last_block) * page_bytes +
+                         (uint32_t)(tok & (kBlock - 1)) * row_bytes + ((b & 1) ? seg_odd : seg_even);
+      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.k_cache + off), (dma_lptr_t *)(ktile + b * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((dma_gptr_t *)(p.v_cache + off), (dma_lptr_t *)(vtile + b * 1024), 16, 0, 0);
+    }
+  };
+
+  int blk[4];
+  pages_of(t_begin, blk);
+  issue(0, t_begin, blk);
+  if (t_begin + kChunk < t_end) {
+    pages_of(t_begin + kChunk, blk);
+    issue(kFp8TileBytes, t_begin + kChunk, blk);
+  }
+  if (t_begin + 2 * kChunk < t_end) pages_of(t_begin + 2 * kChunk, blk);
+
+  int emit_left = emit_every, emit_k = 0;
+  int stores_last = 0, stores_before = 0;  // store instructions issued after the last / the last but one request
+  int tile_off = 0;
+  for (int ti = t_begin; ti < t_end; ti += kChunk) {
+    // this chunk's tile has landed; the next chunk's eight loads (and partials stored since this
+    // tile was requested) may still be on their way
+    wait_vm_all_but(stores_before + (ti + kChunk < t_end ? 8 : 0) + stores_last);
+    const uint8_t *tile = wave_lds + tile_off;
+    u32x4 kraw[4];
+    u32x2 vt[4][2];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) kraw[b] = *(const u32x4 *)(tile + b * 1024 + (k_rd ^ ((b & 1) ? 32u : 0u)));
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) vt[mt][pr] = lds_read_tr8(tile + pr * 2048 + (vt_rd ^ (uint32_t)(mt * 16)));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (ti + 2 * kChunk < t_end) {
+      issue(tile_off, ti + 2 * kChunk, blk);
+      if (ti + 3 * kChunk < t_end) pages_of(ti + 3 * kChunk, blk);
+    }
+    tile_off = kFp8TileBytes - tile_off;
+    Frag8 kf[4][2], vf[4][2];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      fp8x8_to_bf16x8(kraw[b][0], kraw[b][1], kf[b][0].w);
+      fp8x8_to_bf16x8(kraw[b][2], kraw[b][3], kf[b][1].w);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) fp8x8_to_bf16x8(vt[mt][pr][0], vt[mt][pr][1], vf[mt][pr].w);
+    const bool need_mask = (ti < lo_last) || (ti + kChunk > pos_first + 1);
+    chunk_core<NT, false, false, false>(kf, vf, qf, ri, ti, need_mask, c2, m, lacc, acc, nullptr);
+    stores_before = stores_last;
+    stores_last = 0;
+    if constexpr (!std::is_same<Emit, NoEmit>::value) {
+      emit_left -= kChunk;
+      if (emit_left == 0 && ti + kChunk < t_end) {  // (wave-uniform)
+        stores_last = emit(emit_k++);
         emit_left = emit_every;
       }
     }
@@ -1619,7 +1755,7 @@ __device__ __forceinline__ bool even_find_start(const AttnParams &p, const int b
 template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
 __global__ __launch_bounds__(WAVES * 64, ((PAIR && !DMA) ? 4 : 2)) void splitkv_even_kernel(const AttnParams p,
                                                                                           const EvenTable tab) {
-  constexpr int kWaveBytes = !DMA ? kWaveLdsBytes : PAIR ? kWavePairDmaBytes : kWaveDmaBytes;
+  constexpr int kWaveBytes = !DMA ? kWaveLdsBytes : PAIR ? kWavePairDmaBytes : FP8 ? kWaveFp8DmaBytes : kWaveDmaBytes;
   __shared__ __align__(1024) uint8_t lds[WAVES * kWaveBytes];
   __shared__ int start_lds[4];
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1715,6 +1851,8 @@ __global__ __launch_bounds__(WAVES * 64, ((PAIR && !DMA) ? 4 : 2)) void splitkv_
     };
     if constexpr (DMA && PAIR)
       attend_dma_pair(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, pieces ? 0 : U, emit);
+    else if constexpr (DMA && FP8)
+      attend_dma_fp8<NT>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, pieces ? 0 : U, emit);
     else if constexpr (DMA)
       attend_dma<NT>(p, s_now, kvh, t0, t1, L, pos0, lo_last, qf, ri, wave_lds, m, lacc, acc, FirstPages{},
                      pieces ? 0 : U, emit);
@@ -2775,8 +2913,11 @@ bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv) {
 // Workgroups of an even split: resident all at once, one 8-wave workgroup per CU (eight waves
 // keep a CU's share of the memory system busy; of two resident workgroups the younger mostly
 // waits), smaller workgroups so that a CU holds eight waves (the four-wave head-pair kernel
-// of config 4: one per CU 294 us, two 267, three 271, four 280: more ranges are more pieces
-// to store and merge).  EID_EVEN_WGS_PER_CU overrides the number per CU for measurements.
+// of config 4 with one iteration's loads under way per wave: one per CU 294 us, two 267,
+// three 271, four 280: more ranges are more pieces to store and merge).  The head-pair kernel
+// that keeps two iterations under way per wave is fed by one workgroup per CU (config 4:
+// 251 - 253 us against 255 - 256 with two).  EID_EVEN_WGS_PER_CU overrides the number per CU
+// for measurements.
 template <int NT, bool FP8, int WAVES, bool PAIR = false, bool DMA = false>
 static int even_fill_of() {
   static const int fill = device_fill(splitkv_even_kernel<NT, FP8, WAVES, PAIR, DMA>, WAVES * 64);
@@ -2797,8 +2938,10 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
     return e ? atoi(e) : 0;
   }();
   int fill, waves;
+  bool pair_dma = false;
   if (pair && fp8 && ntiles == 1) {
-    fill = even_fill_of<1, true, 4, true>();
+    pair_dma = dma;
+    fill = pair_dma ? even_fill_of<1, true, 4, true, true>() : even_fill_of<1, true, 4, true>();
     waves = 4;
   } else {
     waves = waves_for(Hkv);
@@ -2806,7 +2949,7 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
     else if (dma) fill = ntiles == 1 ? even_fill_t<1, false, true>(waves) : ntiles == 3 ? even_fill_t<3, false, true>(waves) : even_fill_t<4, false, true>(waves);
     else fill = ntiles == 1 ? even_fill_t<1, false>(waves) : ntiles == 3 ? even_fill_t<3, false>(waves) : even_fill_t<4, false>(waves);
   }
-  const int per_cu = per_cu_env > 0 ? per_cu_env : max(1, 8 / waves);
+  const int per_cu = per_cu_env > 0 ? per_cu_env : pair_dma ? 1 : max(1, 8 / waves);
   return max(1, min(fill, per_cu * device_cus()) / (Hkv > 8 ? Hkv / 8 : 1));
 }
 
@@ -2821,6 +2964,10 @@ static hipError_t launch_even_w(const AttnParams &p, const EvenTable &tab, hipSt
   if constexpr (PAIR) {
     if (p.dma_pair)
       return launch_kernel(splitkv_even_kernel<NT, FP8, WAVES, true, true>, grid, dim3(WAVES * 64), 0, st, timed, p, tab);
+  }
+  if constexpr (FP8 && !PAIR && NT >= 3 && WAVES == 8) {
+    if (p.dma_fp8)
+      return launch_kernel(splitkv_even_kernel<NT, true, 8, false, true>, grid, dim3(512), 0, st, timed, p, tab);
   }
   // (p.share_cus: one 8-wave workgroup per CU by a request for unused dynamic LDS, see launch_splitkv_w)
   const int kPad = (WAVES == 8 && p.share_cus) ? 16384 : 0;

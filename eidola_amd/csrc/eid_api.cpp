@@ -569,6 +569,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   static const bool no_dma = getenv("EID_NO_DMA") != nullptr;  // for A/B measurements
   p.dma = (!fp8 && !p.share_cus && !no_dma) ? 1 : 0;
   p.dma_pair = (fp8 && p.fp8_pair && ntiles == 1 && !p.share_cus && !no_dma) ? 1 : 0;
+  p.dma_fp8 = (fp8 && ntiles >= 3 && !p.share_cus && !no_dma) ? 1 : 0;
   p.target_items = eid::splitkv_fill(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0);
   cp.short_span = use_shortspan(d, pl, ntiles);
   cp.merge = pl.nparts_max > 1;
@@ -577,7 +578,7 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   // even split: one row group per KV head (no sequence of the class has more rows than a wave takes)
   const bool even_ok = even_allowed() && pl.nparts_max > 1 && !cp.short_span &&
                        (ntiles == 1 || ntiles == 3 || ntiles == 4);
-  p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0) : 0;
+  p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0 || p.dma_pair != 0) : 0;
   if (p.mixed_wgs > 0 && p.even_wgs > p.mixed_wgs) p.even_wgs = p.mixed_wgs;
   static const bool every = getenv("EID_STORE_EVERY_PARTITION") != nullptr;  // measurement aid
   p.store_every_partition = every ? 1 : 0;

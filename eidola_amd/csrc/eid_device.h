@@ -104,4 +104,14 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const void *lds_ptr) {
   return __builtin_bit_cast(u32x2, v);
 }
 
+// The same for bytes (gfx950 ds_read_b64_tr_b8): within each 16-lane row the lanes address
+// 16 x 8 bytes, F[lane*8 + e]; lane i receives F[i], F[16+i], ..., F[112+i] (byte k of the
+// result comes from lane 2k + i/8 of the row, its byte i%8).
+__device__ __forceinline__ u32x2 lds_read_tr8(const void *lds_ptr) {
+  typedef int s32x2 __attribute__((ext_vector_type(2)));
+  typedef __attribute__((address_space(3))) s32x2 lds_s32x2;
+  s32x2 v = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_s32x2 *)lds_ptr);
+  return __builtin_bit_cast(u32x2, v);
+}
+
 }  // namespace eid

@@ -74,6 +74,7 @@ struct AttnParams {
   int32_t dma;               // host-side launch flag: 1 = bf16 cache and no prefill launch beside: the
                              // split-KV kernels stream their chunks by direct global -> LDS loads
   int32_t dma_pair;          // host-side launch flag: fp8 head pairs of an even split stream through LDS too
+  int32_t dma_fp8;           // host-side launch flag: so do verify rows over an fp8 cache (one head per wave)
   long long exact_items;     // host-side: the launch's exact number of work items when the host
                              // has the sequence lengths, 0 = not known (a bound is launched)
   float softmax_scale;

@@ -232,6 +232,32 @@ def test_seven_and_eight_query_rows_take_four_tiles(G, kv_dtype, window, partiti
     assert np.allclose(lse, ref_lse, atol=2e-3)
 
 
+@pytest.mark.parametrize("q_lens,partition,host_lens", [
+    ([3, 4, 5, 6] * 10, 128, True),    # three row tiles, the host's ranges
+    ([5] * 40, 0, False),              # ... ranges found on the device
+    ([6, 3] * 20, 128, False),
+    ([7, 8] * 20, 128, True),          # four row tiles
+    ([8] * 40, 0, False),
+])
+def test_verify_rows_over_an_fp8_cache_on_the_even_split(G, q_lens, partition, host_lens):
+    """A verify batch over an fp8 cache that is large enough for the even split (equal ranges of
+    chunks per workgroup): one KV head per wave, the chunks' raw bytes streamed into LDS and the
+    V operands read transposed from the bytes.  Ragged lengths (tails inside a page and inside
+    a chunk), against the oracle with lse."""
+    rng = np.random.default_rng(len(q_lens) + partition + sum(q_lens))
+    seq_lens = rng.integers(1500, 9000, size=len(q_lens))
+    b = make_batch(seq_lens, q_lens, partition=partition, kv_dtype=KV_FP8_E4M3)
+    q, k, v, sinks = logical_tensors(b)
+    ks, vs = fp8_scales(k, v)
+    kc, vc = cpu_caches(b, k, v, ks, vs)
+    kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+    ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
+    out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, host_lens=host_lens,
+                          hint=host_lens)
+    assert_close(out, ref, f"fp8 verify rows, even split, P={partition}")
+    assert np.allclose(lse, ref_lse, atol=2e-3)
+
+
 def test_eighth_row_agrees_with_the_prefill_kernel(G):
     """The same 8-row sequences once in a batch whose longest query is 8 rows (split-KV class,
     four tiles) and once next to a 9-row sequence (then they are prefill rows): two kernels,
@@ -1236,6 +1262,16 @@ kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
 ref, _ = oracle_out(b, q, kc, vc, sinks, ks, vs)
 for host in (False, True):
     print(assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, host_lens=host, hint=host), ref, "every partition, fp8"))
+# verify rows over an fp8 cache (one KV head per wave, raw bytes through LDS)
+seq_lens = rng.integers(1500, 7000, size=40)
+b = make_batch(seq_lens, [4, 6] * 20, partition=128, kv_dtype=KV_FP8_E4M3)
+q, k, v, sinks = logical_tensors(b)
+ks, vs = fp8_scales(k, v)
+kc, vc = cpu_caches(b, k, v, ks, vs)
+kc_d, vc_d = G.gpu_caches(b, k, v, ks, vs)
+ref, _ = oracle_out(b, q, kc, vc, sinks, ks, vs)
+for host in (False, True):
+    print(assert_close(G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, host_lens=host, hint=host), ref, "every partition, fp8 verify"))
 '''
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     env = dict(os.environ, EID_STORE_EVERY_PARTITION="1")
