@@ -10,8 +10,9 @@
 //   online softmax in base 2 on the accumulator layout (a lane owns 4 tokens of one row,
 //        the row maximum crosses the four 16-lane rows with v_permlane{16,32}_swap);
 //   P^T leaves the softmax already in B-operand layout (tokens on the contraction axis);
-//   O^T[dim][row] += V^T[dim][token] . P^T[token][row], with V staged row-major in LDS and
-//        read back transposed by ds_read_b64_tr_b16.
+//   O^T[dim][row] += V^T[dim][token] . P^T[token][row], with V row-major in LDS and read back
+//        transposed: bf16 rows by ds_read_b64_tr_b16, the raw bytes of an fp8 cache by
+//        ds_read_b64_tr_b8 and widened in registers (attend_dma_pair, attend_dma_fp8).
 // "row" = (query token, query head of the KV group): 8 heads share every K/V byte.
 #include <atomic>
 #include "eid_device.h"
@@ -933,11 +934,10 @@ __device__ __forceinline__ void attend_dma(const AttnParams &p, const int s, con
 // x 2 heads) and are in flight while this one is converted and multiplied, where the
 // register path has nothing in flight during its arithmetic.
 // ---------------------------------------------------------------------------------------
-#ifndef EID_PAIR_VBLOCK
-#define EID_PAIR_VBLOCK 1152
-#endif
-constexpr int kPairRawBytes = 4 * 1024;       // one tensor, one iteration
-constexpr int kPairVBlock = EID_PAIR_VBLOCK;  // V blocks 128 bytes apart in bank terms: the two blocks of a transposing read
+constexpr int kPairRawBytes = 4 * 1024;  // one tensor, one iteration
+// V blocks sit 128 bytes apart in bank terms: the two blocks that a transposing read touches
+// fall into different halves of the banks (1,024 apart: 256.4 us on config 4 against 255.1)
+constexpr int kPairVBlock = 1024 + 128;
 constexpr int kPairTileBytes = kPairRawBytes + 4 * kPairVBlock;  // raw K, raw V of one iteration
 constexpr int kWavePairDmaBytes = 2 * kPairTileBytes;            // two iterations under way
 
