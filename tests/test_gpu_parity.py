@@ -232,21 +232,22 @@ def test_seven_and_eight_query_rows_take_four_tiles(G, kv_dtype, window, partiti
     assert np.allclose(lse, ref_lse, atol=2e-3)
 
 
-@pytest.mark.parametrize("q_lens,partition,host_lens", [
-    ([3, 4, 5, 6] * 10, 128, True),    # three row tiles, the host's ranges
-    ([5] * 40, 0, False),              # ... ranges found on the device
-    ([6, 3] * 20, 128, False),
-    ([7, 8] * 20, 128, True),          # four row tiles
-    ([8] * 40, 0, False),
+@pytest.mark.parametrize("q_lens,partition,host_lens,window", [
+    ([3, 4, 5, 6] * 10, 128, True, 0),    # three row tiles, the host's ranges
+    ([5] * 40, 0, False, 0),              # ... ranges found on the device
+    ([6, 3] * 20, 128, False, 0),
+    ([7, 8] * 20, 128, True, 0),          # four row tiles
+    ([8] * 40, 0, False, 0),
+    ([4, 5] * 30, 128, True, 3000),       # a window that starts inside a page and a chunk
 ])
-def test_verify_rows_over_an_fp8_cache_on_the_even_split(G, q_lens, partition, host_lens):
+def test_verify_rows_over_an_fp8_cache_on_the_even_split(G, q_lens, partition, host_lens, window):
     """A verify batch over an fp8 cache that is large enough for the even split (equal ranges of
     chunks per workgroup): one KV head per wave, the chunks' raw bytes streamed into LDS and the
     V operands read transposed from the bytes.  Ragged lengths (tails inside a page and inside
     a chunk), against the oracle with lse."""
     rng = np.random.default_rng(len(q_lens) + partition + sum(q_lens))
     seq_lens = rng.integers(1500, 9000, size=len(q_lens))
-    b = make_batch(seq_lens, q_lens, partition=partition, kv_dtype=KV_FP8_E4M3)
+    b = make_batch(seq_lens, q_lens, window=window, partition=partition, kv_dtype=KV_FP8_E4M3)
     q, k, v, sinks = logical_tensors(b)
     ks, vs = fp8_scales(k, v)
     kc, vc = cpu_caches(b, k, v, ks, vs)
@@ -254,7 +255,7 @@ def test_verify_rows_over_an_fp8_cache_on_the_even_split(G, q_lens, partition, h
     ref, ref_lse = oracle_out(b, q, kc, vc, sinks, ks, vs)
     out, lse = G.run_attn(b, q, kc_d, vc_d, sinks, ks, vs, return_lse=True, host_lens=host_lens,
                           hint=host_lens)
-    assert_close(out, ref, f"fp8 verify rows, even split, P={partition}")
+    assert_close(out, ref, f"fp8 verify rows, even split, P={partition} w={window}")
     assert np.allclose(lse, ref_lse, atol=2e-3)
 
 
