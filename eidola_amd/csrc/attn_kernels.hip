@@ -2950,7 +2950,12 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
     else fill = ntiles == 1 ? even_fill_t<1, false>(waves) : ntiles == 3 ? even_fill_t<3, false>(waves) : even_fill_t<4, false>(waves);
   }
   const int per_cu = per_cu_env > 0 ? per_cu_env : pair_dma ? 1 : max(1, 8 / waves);
-  return max(1, min(fill, per_cu * device_cus()) / (Hkv > 8 ? Hkv / 8 : 1));
+  // the streaming kernels saturate the memory system from seven eighths of the CUs, and fewer
+  // ranges are fewer pieces: 224 workgroups against 256 on one box, call level: config 2 81.0
+  // against 82.0 us, config 3's decode rows 157.8 / 160.8, config 5 1,342 / 1,348, config 4
+  // (fp8) 250.0 / 251.6 (192: 80.9, 158.1, 1,341, 261)
+  const int cus = (dma && per_cu_env <= 0) ? device_cus() * 7 / 8 : device_cus();
+  return max(1, min(fill, per_cu * cus) / (Hkv > 8 ? Hkv / 8 : 1));
 }
 
 template <int NT, bool FP8, int WAVES, bool PAIR = false>
