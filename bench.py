@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 # --calibrate-copy).  See profiles/splitkv_decode_config2.md.  A kernel that is not listed
 # (or a non-default batch) reports traffic as null rather than another kernel's figure.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "splitkv_even_kernel<1,bf16,8 waves,direct-to-LDS loads>": int((240_966 * 2.0 + 2_707 * 1.0) * 1024),
+    "splitkv_even_kernel<1,bf16,8 waves,direct-to-LDS loads>": int((240_870 * 2.0 + 2_468 * 1.0) * 1024),
 }
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 METRIC = "paged sink-attn decode HBM GB/s (% peak) + ragged-batch tokens/s, 1 GPU"
