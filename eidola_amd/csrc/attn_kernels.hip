@@ -2932,7 +2932,7 @@ static int even_fill_t(int waves) {
     default: return even_fill_of<NT, FP8, 1, false, DMA>();
   }
 }
-int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
+int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma, bool all_cus) {
   static const int per_cu_env = [] {
     const char *e = getenv("EID_EVEN_WGS_PER_CU");
     return e ? atoi(e) : 0;
@@ -2954,7 +2954,9 @@ int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma) {
   // ranges are fewer pieces: 224 workgroups against 256 on one box, call level: config 2 81.0
   // against 82.0 us, config 3's decode rows 157.8 / 160.8, config 5 1,342 / 1,348, config 4
   // (fp8) 250.0 / 251.6 (192: 80.9, 158.1, 1,341, 261)
-  const int cus = (dma && per_cu_env <= 0) ? device_cus() * 7 / 8 : device_cus();
+  // (all_cus: a partial per partition of the caller's is stored, 346 MB of them on config 5: the
+  // stores want every CU, 1,742 us against 1,780)
+  const int cus = (dma && !all_cus && per_cu_env <= 0) ? device_cus() * 7 / 8 : device_cus();
   return max(1, min(fill, per_cu * cus) / (Hkv > 8 ? Hkv / 8 : 1));
 }
 

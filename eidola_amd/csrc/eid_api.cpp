@@ -23,7 +23,7 @@ hipError_t launch_shortspan(const AttnParams &p, int ntiles, bool fp8, hipStream
                             const ItemTable *tab = nullptr);
 hipError_t launch_even(AttnParams &p, int ntiles, bool fp8, int32_t *plan_slot, hipStream_t st,
                        const EvenTable *tab);
-int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma);
+int even_wgs(int ntiles, bool fp8, int Hkv, bool pair, bool dma, bool all_cus);
 bool shortspan_applies(int ntiles, bool fp8, long long num_items, int Hkv);
 long long shortspan_items(int num_seqs, int nparts_max, long long sum_kv_len, int window);
 hipError_t launch_prefill(const AttnParams &p, int num_q_tokens, bool fp8, hipStream_t st,
@@ -578,13 +578,15 @@ ClassPlan plan_class(const eid_attn_desc *d, const eid_attn_args *a, const Plan 
   // even split: one row group per KV head (no sequence of the class has more rows than a wave takes)
   const bool even_ok = even_allowed() && pl.nparts_max > 1 && !cp.short_span &&
                        (ntiles == 1 || ntiles == 3 || ntiles == 4);
-  p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0 || p.dma_pair != 0) : 0;
-  if (p.mixed_wgs > 0 && p.even_wgs > p.mixed_wgs) p.even_wgs = p.mixed_wgs;
   static const bool every = getenv("EID_STORE_EVERY_PARTITION") != nullptr;  // measurement aid
   p.store_every_partition = every ? 1 : 0;
 #ifdef EID_MEASURE
   if (eid::store_every_partition_override() >= 0) p.store_every_partition = eid::store_every_partition_override();
 #endif
+  p.even_wgs = even_ok ? eid::even_wgs(ntiles, fp8, d->num_kv_heads, p.fp8_pair != 0, p.dma != 0 || p.dma_pair != 0,
+                                       p.store_every_partition != 0 && !pl.dynamic)
+                       : 0;
+  if (p.mixed_wgs > 0 && p.even_wgs > p.mixed_wgs) p.even_wgs = p.mixed_wgs;
   if (!a->seq_lens_host || (!decode && !cu) || d->num_seqs > kHostPlanMaxSeqs || capturing) {
     // Without the lengths: a run-time partition always takes the even split (every workgroup
     // finds its range by a scan of the device arrays); the caller's partition takes it when
